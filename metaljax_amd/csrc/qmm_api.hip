@@ -1,0 +1,306 @@
+// C ABI of libqmm_hip.so: argument validation and regime dispatch.
+// See include/qmm_hip.h for the contract of every entry point.
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+
+#include "qmm_common.hpp"
+
+namespace qmm {
+
+void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                   int y_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int gs, int bits,
+                   int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st);
+void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
+void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                   int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
+                   const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
+                   int bits, int mode, hipStream_t st);
+int64_t gemm_row_tile();
+void unpack_dispatch(const void* w, void* codes, int64_t rows, int64_t K, int bits, hipStream_t st);
+void pack_dispatch(const void* codes, void* w, int64_t rows, int64_t K, int bits, hipStream_t st);
+void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void* out,
+                      int out_dtype, int64_t rows, int64_t K, int gs, int bits, int mode,
+                      hipStream_t st);
+void take_dispatch(const void* x, int x_dtype, const int32_t* perm, void* out, int64_t rows,
+                   int64_t K, hipStream_t st);
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(QMM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return QMM_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Largest M served by the decode kernel.
+constexpr int64_t kGemvMaxM = 16;
+// Pairs at or below which the gather form runs one decode launch per pair
+// instead of sorting rows by expert.
+constexpr int64_t kGatherGemvMaxPairs = 64;
+
+int check_quant(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* w,
+                const void* s, const void* b) {
+  if (!w || !s) return fail(QMM_ERR_BAD_ARGUMENT, "null weight or scale pointer");
+  if (N < 0 || K < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (mode == QMM_MODE_MXFP4) {
+    if (bits != 4) return fail(QMM_ERR_UNSUPPORTED, "mxfp4 requires bits=4, got %d", bits);
+    if (gs != 32) return fail(QMM_ERR_UNSUPPORTED, "mxfp4 requires group_size=32, got %d", gs);
+    if (b) return fail(QMM_ERR_BAD_ARGUMENT, "mxfp4 takes no biases");
+  } else if (mode == QMM_MODE_AFFINE) {
+    if (bits != 4 && bits != 8) return fail(QMM_ERR_UNSUPPORTED, "affine bits=%d (4 or 8 built)", bits);
+    if (gs != 32 && gs != 64 && gs != 128)
+      return fail(QMM_ERR_UNSUPPORTED, "group_size=%d (32, 64 or 128)", gs);
+    if (!b) return fail(QMM_ERR_BAD_ARGUMENT, "affine mode needs biases");
+    if (tab != QMM_F32 && tab != QMM_BF16 && tab != QMM_F16)
+      return fail(QMM_ERR_UNSUPPORTED, "table dtype %d", tab);
+  } else {
+    return fail(QMM_ERR_UNSUPPORTED, "mode %d", mode);
+  }
+  if (K % 32) return fail(QMM_ERR_BAD_SHAPE, "K=%lld is not a multiple of 32", (long long)K);
+  if (K % gs) return fail(QMM_ERR_BAD_SHAPE, "K=%lld is not a multiple of group_size=%d", (long long)K, gs);
+  if (!aligned16(w)) return fail(QMM_ERR_BAD_ARGUMENT, "weight pointer not 16-byte aligned");
+  return QMM_OK;
+}
+
+int check_io(const void* x, int x_dtype, void* y, int y_dtype) {
+  if (!x || !y) return fail(QMM_ERR_BAD_ARGUMENT, "null activation or output pointer");
+  if (x_dtype != QMM_BF16)
+    return fail(QMM_ERR_UNSUPPORTED, "activation dtype %d (bf16 built)", x_dtype);
+  if (y_dtype != QMM_BF16 && y_dtype != QMM_F32 && y_dtype != QMM_F16)
+    return fail(QMM_ERR_UNSUPPORTED, "output dtype %d", y_dtype);
+  if (!aligned16(x)) return fail(QMM_ERR_BAD_ARGUMENT, "activation pointer not 16-byte aligned");
+  return QMM_OK;
+}
+
+// ---- routing for the gather form: pairs -> rows sorted by expert -----------
+// workspace layout (int32): row_offsets[E+1] | cursor[E] | src_row[P] | out_row[P]
+__global__ __launch_bounds__(1024) void route_kernel(const int32_t* __restrict__ lhs_idx,
+                                                     const int32_t* __restrict__ rhs_idx, int P,
+                                                     int E, int32_t* __restrict__ row_offsets,
+                                                     int32_t* __restrict__ cursor,
+                                                     int32_t* __restrict__ src_row,
+                                                     int32_t* __restrict__ out_row) {
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
+    row_offsets[e] = 0;
+    if (e < E) cursor[e] = 0;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = rhs_idx[p];
+    if (e >= 0 && e < E) atomicAdd(&cursor[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cursor[e];
+      row_offsets[e] = run;
+      cursor[e] = run;
+      run += c;
+    }
+    row_offsets[E] = run;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = rhs_idx[p];
+    if (e < 0 || e >= E) continue;
+    const int pos = atomicAdd(&cursor[e], 1);
+    src_row[pos] = lhs_idx ? lhs_idx[p] : p;
+    out_row[pos] = p;
+  }
+}
+
+size_t route_bytes(int64_t P, int64_t E) {
+  return (size_t)(2 * E + 1 + 2 * P) * sizeof(int32_t) + 64;
+}
+
+}  // namespace
+}  // namespace qmm
+
+using namespace qmm;
+
+extern "C" {
+
+int qmm_abi_version(void) { return 1; }
+
+const char* qmm_last_error(void) { return g_err; }
+
+size_t qmm_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int, int, int, int) { return 0; }
+
+size_t qmm_gather_workspace_bytes(int64_t P, int64_t E) {
+  return P <= kGatherGemvMaxPairs ? 0 : route_bytes(P, E);
+}
+
+int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int, int* kernel, int* grid, int* block) {
+  if (M <= kGemvMaxM) {
+    int t, waves;
+    gemv_geometry(M, N, K, &t, &waves);
+    if (kernel) *kernel = QMM_KERNEL_GEMV;
+    if (grid) *grid = (int)ceil_div(N, 16 * t);
+    if (block) *block = 64 * waves;
+  } else {
+    const int64_t bm = gemm_row_tile();
+    if (kernel) *kernel = QMM_KERNEL_GEMM;
+    if (grid) *grid = (int)(ceil_div(N, 128) * ceil_div(M, bm));
+    if (block) *block = 256;
+  }
+  return QMM_OK;
+}
+
+int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* scales,
+                         const void* biases, int table_dtype, void* y, int y_dtype,
+                         int64_t batch, int64_t M, int64_t N, int64_t K, int group_size,
+                         int bits, int mode, void*, size_t, void* stream) {
+  if (batch < 0 || M < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (batch == 0 || M == 0 || N == 0) return QMM_OK;
+  if (K == 0) return fail(QMM_ERR_BAD_SHAPE, "K=0");
+  int rc = check_quant(N, K, group_size, bits, mode, table_dtype, w, scales, biases);
+  if (rc) return rc;
+  rc = check_io(x, x_dtype, y, y_dtype);
+  if (rc) return rc;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535)
+    return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M <= kGemvMaxM) {
+    gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, batch, M, N, K, group_size,
+                  bits, mode, nullptr, nullptr, st);
+    return check_launch("gemv launch");
+  }
+  const int wbits = mode == QMM_MODE_MXFP4 ? 4 : bits;
+  const int64_t wpr = K * wbits / 32;
+  const int64_t ng = mode == QMM_MODE_MXFP4 ? K / 32 : K / group_size;
+  const int tabsz = mode == QMM_MODE_MXFP4 ? 1 : (table_dtype == QMM_F32 ? 4 : 2);
+  const int ysz = y_dtype == QMM_F32 ? 4 : 2;
+  for (int64_t z = 0; z < batch; ++z) {
+    gemm_dispatch(static_cast<const char*>(x) + z * M * K * 2,
+                  static_cast<const uint32_t*>(w) + z * N * wpr,
+                  static_cast<const char*>(scales) + z * N * ng * tabsz,
+                  biases ? static_cast<const char*>(biases) + z * N * ng * tabsz : nullptr,
+                  table_dtype, static_cast<char*>(y) + z * M * N * ysz, y_dtype, nullptr, nullptr,
+                  nullptr, M, 1, N, K, group_size, bits, mode, st);
+    rc = check_launch("gemm launch");
+    if (rc) return rc;
+  }
+  return QMM_OK;
+}
+
+int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scales,
+                    const void* biases, int table_dtype, void* y, int y_dtype,
+                    const int32_t* row_offsets, int64_t R, int64_t E, int64_t N, int64_t K,
+                    int group_size, int bits, int mode, void*, size_t, void* stream) {
+  if (R < 0 || E < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (R == 0 || N == 0 || E == 0) return QMM_OK;
+  if (!row_offsets) return fail(QMM_ERR_BAD_ARGUMENT, "null row_offsets");
+  int rc = check_quant(N, K, group_size, bits, mode, table_dtype, w, scales, biases);
+  if (rc) return rc;
+  rc = check_io(x, x_dtype, y, y_dtype);
+  if (rc) return rc;
+  if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535)
+    return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
+                E, N, K, group_size, bits, mode, static_cast<hipStream_t>(stream));
+  return check_launch("grouped gemm launch");
+}
+
+int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales,
+                   const void* biases, int table_dtype, void* y, int y_dtype,
+                   const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
+                   int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (P < 0 || T < 0 || E < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (P == 0 || N == 0) return QMM_OK;
+  if (!rhs_idx) return fail(QMM_ERR_BAD_ARGUMENT, "null rhs_idx");
+  int rc = check_quant(N, K, group_size, bits, mode, table_dtype, w, scales, biases);
+  if (rc) return rc;
+  rc = check_io(x, x_dtype, y, y_dtype);
+  if (rc) return rc;
+  if (P > INT32_MAX / 2 || N > INT32_MAX || K > INT32_MAX || E > 65535)
+    return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (P <= kGatherGemvMaxPairs) {
+    gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, P, 1, N, K, group_size, bits,
+                  mode, lhs_idx, rhs_idx, st);
+    return check_launch("gather gemv launch");
+  }
+  const size_t need = route_bytes(P, E);
+  if (!workspace || workspace_bytes < need)
+    return fail(QMM_ERR_WORKSPACE, "gather_qmm needs %zu workspace bytes, got %zu", need,
+                workspace_bytes);
+  int32_t* ro = static_cast<int32_t*>(workspace);
+  int32_t* cursor = ro + E + 1;
+  int32_t* src_row = cursor + E;
+  int32_t* out_row = src_row + P;
+  hipLaunchKernelGGL(route_kernel, dim3(1), dim3(1024), 0, st, lhs_idx, rhs_idx, (int)P, (int)E,
+                     ro, cursor, src_row, out_row);
+  rc = check_launch("route launch");
+  if (rc) return rc;
+  gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, E, N, K,
+                group_size, bits, mode, st);
+  return check_launch("gather gemm launch");
+}
+
+int qmm_dequantize(const void* w, const void* scales, const void* biases, int table_dtype,
+                   void* out, int out_dtype, int64_t rows, int64_t K, int group_size, int bits,
+                   int mode, void* stream) {
+  if (rows < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (rows == 0 || K == 0) return QMM_OK;
+  int rc = check_quant(rows, K, group_size, bits, mode, table_dtype, w, scales, biases);
+  if (rc) return rc;
+  if (!out) return fail(QMM_ERR_BAD_ARGUMENT, "null output pointer");
+  if (out_dtype != QMM_F32 && out_dtype != QMM_BF16 && out_dtype != QMM_F16)
+    return fail(QMM_ERR_UNSUPPORTED, "output dtype %d", out_dtype);
+  if (!aligned16(out)) return fail(QMM_ERR_BAD_ARGUMENT, "output pointer not 16-byte aligned");
+  dequant_dispatch(w, scales, biases, table_dtype, out, out_dtype, rows, K, group_size, bits,
+                   mode, static_cast<hipStream_t>(stream));
+  return check_launch("dequantize launch");
+}
+
+static int check_codes(const void* a, const void* b, int64_t rows, int64_t K, int bits) {
+  if (rows < 0 || K < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (bits != 2 && bits != 4 && bits != 8) return fail(QMM_ERR_UNSUPPORTED, "bits=%d (2, 4 or 8)", bits);
+  if (K % (32 / bits)) return fail(QMM_ERR_BAD_SHAPE, "K=%lld not a multiple of %d", (long long)K, 32 / bits);
+  if (rows * K == 0) return QMM_OK;
+  if (!a || !b) return fail(QMM_ERR_BAD_ARGUMENT, "null pointer");
+  if (!aligned16(a) || !aligned16(b)) return fail(QMM_ERR_BAD_ARGUMENT, "pointer not 16-byte aligned");
+  return QMM_OK;
+}
+
+int qmm_unpack_codes(const void* w, void* codes, int64_t rows, int64_t K, int bits, void* stream) {
+  int rc = check_codes(w, codes, rows, K, bits);
+  if (rc || rows * K == 0) return rc;
+  unpack_dispatch(w, codes, rows, K, bits, static_cast<hipStream_t>(stream));
+  return check_launch("unpack launch");
+}
+
+int qmm_pack_codes(const void* codes, void* w, int64_t rows, int64_t K, int bits, void* stream) {
+  int rc = check_codes(codes, w, rows, K, bits);
+  if (rc || rows * K == 0) return rc;
+  pack_dispatch(codes, w, rows, K, bits, static_cast<hipStream_t>(stream));
+  return check_launch("pack launch");
+}
+
+int qmm_take_k(const void* x, int x_dtype, const int32_t* perm, void* out, int64_t rows,
+               int64_t K, void* stream) {
+  if (rows < 0 || K < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  if (rows * K == 0) return QMM_OK;
+  if (!x || !perm || !out) return fail(QMM_ERR_BAD_ARGUMENT, "null pointer");
+  if (x_dtype != QMM_F32 && x_dtype != QMM_BF16 && x_dtype != QMM_F16)
+    return fail(QMM_ERR_UNSUPPORTED, "dtype %d", x_dtype);
+  take_dispatch(x, x_dtype, perm, out, rows, K, static_cast<hipStream_t>(stream));
+  return check_launch("take launch");
+}
+
+}  // extern "C"

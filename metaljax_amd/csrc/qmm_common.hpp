@@ -1,0 +1,105 @@
+// Device-side helpers shared by the gfx950 quantized-matmul kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qmm_hip.h"
+
+namespace qmm {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) {
+  return __uint_as_float(b << 16);
+}
+
+// float32 -> bf16 bits, round to nearest even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  bf16x2 t;
+  t[0] = (__bf16)f;
+  t[1] = (__bf16)0.0f;
+  return __builtin_bit_cast(uint32_t, t) & 0xFFFFu;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2 t;
+  t[0] = (__bf16)lo;
+  t[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, t);
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+
+// One scale / bias table entry as float32 (exact widening).
+template <int TAB>
+__device__ __forceinline__ float load_table(const void* p, int64_t i) {
+  if constexpr (TAB == QMM_F32) {
+    return static_cast<const float*>(p)[i];
+  } else if constexpr (TAB == QMM_BF16) {
+    return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  } else {
+    return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  }
+}
+
+__device__ __forceinline__ float load_table_rt(const void* p, int64_t i, int tab) {
+  if (tab == QMM_F32) return load_table<QMM_F32>(p, i);
+  if (tab == QMM_BF16) return load_table<QMM_BF16>(p, i);
+  return load_table<QMM_F16>(p, i);
+}
+
+__device__ __forceinline__ void store_out(void* y, int64_t i, float v, int yd) {
+  if (yd == QMM_BF16) {
+    static_cast<uint16_t*>(y)[i] = (uint16_t)f32_to_bf16_bits(v);
+  } else if (yd == QMM_F32) {
+    static_cast<float*>(y)[i] = v;
+  } else {
+    static_cast<uint16_t*>(y)[i] = (uint16_t)f32_to_f16_bits(v);
+  }
+}
+
+// E8M0 byte -> 2^(e-127) as float32.  Byte 0 is the subnormal 2^-127 and byte
+// 255 is NaN, as in the OCP MX specification.
+__device__ __forceinline__ float e8m0_to_f32(uint32_t e) {
+  uint32_t bits = e << 23;
+  if (e == 0u) bits = 0x00400000u;
+  if (e == 255u) bits = 0x7FC00000u;
+  return __uint_as_float(bits);
+}
+
+// E2M1 code (4 bits, bit 3 = sign) -> float32, exact.
+__device__ __forceinline__ float e2m1_to_f32(uint32_t c) {
+  // magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6 as bf16 high bytes+: build f32 bits
+  const uint32_t m = c & 7u;
+  // normal (m >= 2): exponent (m>>1) with bias 1, mantissa bit (m&1);
+  // m == 1 is the subnormal 0.5; m == 0 is zero.
+  uint32_t bits;
+  if (m >= 2u) bits = ((126u + (m >> 1)) << 23) | ((m & 1u) << 22);
+  else bits = m ? 0x3F000000u : 0u;
+  return __uint_as_float(bits | ((c & 8u) << 28));
+}
+
+// v_perm_b32: bytes 0-3 of the selector index come from `lo`, 4-7 from `hi`.
+__device__ __forceinline__ uint32_t byte_perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+  return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+__host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace qmm

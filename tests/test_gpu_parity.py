@@ -1,0 +1,363 @@
+"""GPU parity: the HIP path (through the C ABI, via metaljax_amd.kernels)
+against the CPU oracle on the same seeded inputs.
+
+Two correctness levels:
+  * unpacked codes and dequantized tiles: BIT-EXACT;
+  * outputs: rel-L2 <= 1e-2 for bf16 outputs, <= 1e-3 for float32 outputs
+    (float32 accumulate).  The decode kernel keeps the weight exact, so it is
+    checked against the exactly reconstructed weight; the prefill kernel
+    stages a bf16 weight tile, so its 1e-3 level is checked against the
+    bf16-rounded weight and its distance to the exact weight is bounded at 3e-3.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from metaljax_amd import kernels as K
+from metaljax_amd import synth
+from oracle import c_oracle as C
+from oracle import qmm_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_BF16_OUT = 1e-2
+TOL_F32_OUT = 1e-3
+DEV = "cuda"
+
+
+def bf16_dev(bits_u16):
+    return torch.from_numpy(np.ascontiguousarray(bits_u16).view(np.int16)).to(DEV).view(torch.bfloat16)
+
+
+def words_dev(w):
+    return torch.from_numpy(np.ascontiguousarray(w).view(np.int32)).to(DEV)
+
+
+def out_f32(y):
+    return y.float().cpu().numpy()
+
+
+def make_affine(rng, n, k, bits, gs, tab="bf16", lead=()):
+    codes = rng.integers(0, 1 << bits, size=lead + (n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    s = rng.uniform(0.005, 0.02, lead + (n, k // gs)).astype(np.float32)
+    if tab == "bf16":
+        s = O.round_bf16(s)
+        b = O.round_bf16(-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s)
+        sd, bd = bf16_dev(O.f32_to_bf16_bits(s)), bf16_dev(O.f32_to_bf16_bits(b))
+    elif tab == "f16":
+        s = s.astype(np.float16).astype(np.float32)
+        b = (-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s).astype(np.float16).astype(np.float32)
+        sd = torch.from_numpy(s.astype(np.float16)).to(DEV)
+        bd = torch.from_numpy(b.astype(np.float16)).to(DEV)
+    else:
+        b = (-(rng.uniform(0, 1 << bits, s.shape).astype(np.float32)) * s).astype(np.float32)
+        sd, bd = torch.from_numpy(s).to(DEV), torch.from_numpy(b).to(DEV)
+    return codes, words, s, b, words_dev(words), sd, bd
+
+
+def make_mxfp4(rng, n, k, lead=(), lo=118, hi=132):
+    codes = rng.integers(0, 16, size=lead + (n, k), dtype=np.uint8)
+    codes.reshape(-1, k)[0, :16] = np.arange(16)
+    words = O.pack_codes(codes, 4)
+    sb = rng.integers(lo, hi, size=lead + (n, k // 32)).astype(np.uint8)
+    return codes, words, sb, words_dev(words), torch.from_numpy(sb).to(DEV)
+
+
+def make_x(rng, m, k):
+    x = O.round_bf16(rng.standard_normal((m, k)).astype(np.float32))
+    return x, bf16_dev(O.f32_to_bf16_bits(x))
+
+
+# ------------------------------------------------------------ bit-exact ----
+
+def test_library_reports_loaded():
+    from metaljax_amd import _lib
+    assert _lib.load().qmm_abi_version() == 1
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("shape", [(1, 32), (5, 128), (3, 4, 64), (257, 4096)])
+def test_unpack_and_pack_codes_bit_exact(bits, shape):
+    rng = np.random.default_rng(bits + shape[-1])
+    codes = rng.integers(0, 1 << bits, size=shape, dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    got = K.unpack_codes(words_dev(words), bits).cpu().numpy()
+    np.testing.assert_array_equal(got, codes)
+    packed = K.pack_codes(torch.from_numpy(codes).to(DEV), bits).cpu().numpy().view(np.uint32)
+    np.testing.assert_array_equal(packed, words)
+
+
+def test_pack_layout_hand_computed_words():
+    codes = (np.arange(32, dtype=np.uint8) % 16).reshape(1, 32)
+    packed = K.pack_codes(torch.from_numpy(codes).to(DEV), 4).cpu().numpy().view(np.uint32)
+    np.testing.assert_array_equal(packed[0, :2], np.array([0x76543210, 0xFEDCBA98], np.uint32))
+
+
+def test_empty_inputs():
+    assert K.unpack_codes(torch.zeros((0, 4), dtype=torch.int32, device=DEV), 4).shape == (0, 32)
+    x = torch.zeros((0, 64), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((16, 8), dtype=torch.int32, device=DEV)
+    s = torch.ones((16, 1), dtype=torch.bfloat16, device=DEV)
+    assert K.quantized_matmul(x, w, s, s, group_size=64, bits=4).shape == (0, 16)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("tab", ["bf16", "f32", "f16"])
+def test_dequantize_affine_bit_exact(bits, gs, tab):
+    rng = np.random.default_rng(bits * 1000 + gs)
+    n, k = 48, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab)
+    want = O.dequant_affine(words, s, b, gs, bits)
+    got = K.dequantize(wd, sd, bd, group_size=gs, bits=bits).cpu().numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    got16 = K.dequantize(wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.bfloat16)
+    np.testing.assert_array_equal(got16.view(torch.int16).cpu().numpy().view(np.uint16),
+                                  O.f32_to_bf16_bits(want))
+
+
+@pytest.mark.parametrize("zp_kind", ["zero", "const", "random"])
+@pytest.mark.parametrize("scale_kind", ["pow2", "bf16", "f32"])
+def test_dequantize_of_pack_exact_matrix(zp_kind, scale_kind):
+    """The reference's exactness matrix (tests/test_qmm.py:96-132) through the
+    product pack + the device dequantize."""
+    from metaljax_amd import packing as P
+    bits, gs = 4, 64
+    rng = np.random.default_rng(400 + gs)
+    n, k = 16, 256
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int32)
+    codes[0, :4] = [-8, 7, 0, -1]
+    scale = (rng.random((n, k // gs)).astype(np.float32) + 0.5) * 0.03
+    if scale_kind == "pow2":
+        scale = np.exp2(rng.integers(-8, 2, size=scale.shape)).astype(np.float32)
+    elif scale_kind == "bf16":
+        scale = O.round_bf16(scale)
+    zp = {"zero": np.zeros((n, k // gs), np.int32), "const": np.full((n, k // gs), 3, np.int32),
+          "random": rng.integers(-8, 8, (n, k // gs)).astype(np.int32)}[zp_kind]
+    want = scale.repeat(gs, 1) * (codes.astype(np.float32) - zp.repeat(gs, 1).astype(np.float32))
+    w, s, b = P.pack_exact(codes, scale, zp, bits)
+    got = K.dequantize(words_dev(w), torch.from_numpy(s).to(DEV), torch.from_numpy(b).to(DEV),
+                       group_size=gs, bits=bits).cpu().numpy()
+    if zp_kind == "zero" or scale_kind in ("pow2", "bf16"):
+        np.testing.assert_array_equal(got, want)
+    else:
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-5
+
+
+@pytest.mark.parametrize("shape", [(4, 64), (3, 2, 128), (40, 1024)])
+def test_dequantize_mxfp4_bit_exact(shape):
+    rng = np.random.default_rng(7 + sum(shape))
+    *lead, n, k = shape
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, tuple(lead), lo=1, hi=255)
+    want = O.dequant_mxfp4(O.pack_blocks(codes), sb)
+    got = K.dequantize(wd, sd, None, group_size=32, bits=4, mode="mxfp4").cpu().numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    sb2 = np.clip(sb, 100, 150)
+    want2 = O.dequant_mxfp4(O.pack_blocks(codes), sb2)
+    got16 = K.dequantize(wd, torch.from_numpy(sb2).to(DEV), None, group_size=32, bits=4,
+                         mode="mxfp4", out_dtype=torch.bfloat16).float().cpu().numpy()
+    np.testing.assert_array_equal(got16, want2)        # exact in bf16 too
+
+
+def test_take_k():
+    rng = np.random.default_rng(3)
+    x, xd = make_x(rng, 5, 256)
+    perm = rng.permutation(256).astype(np.int32)
+    got = K.take_k(xd, torch.from_numpy(perm).to(DEV)).float().cpu().numpy()
+    np.testing.assert_array_equal(got, x[:, perm])
+
+
+# ------------------------------------------------------- decode (M <= 16) ----
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("m", [1, 3, 16])
+def test_gemv_affine(bits, gs, m):
+    rng = np.random.default_rng(bits * 100 + gs + m)
+    n, k = 200, 1024                      # N not a multiple of 16
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= TOL_F32_OUT, O.rel_l2(y32, want)
+    assert O.rel_l2(y32, want) <= 2e-5          # in fact far inside the bar
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits))
+    assert O.rel_l2(y16, want) <= TOL_BF16_OUT
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))     # bf16 out = one RNE of the f32 result
+
+
+@pytest.mark.parametrize("tab", ["f32", "f16"])
+def test_gemv_table_dtypes(tab):
+    rng = np.random.default_rng(17)
+    n, k, gs, bits = 64, 512, 64, 4
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab)
+    x, xd = make_x(rng, 2, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5
+
+
+@pytest.mark.parametrize("k", [32, 96, 4096])
+def test_gemv_k_edge_sizes(k):
+    rng = np.random.default_rng(k)
+    n, gs, bits = 33, 32, 4
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    x, xd = make_x(rng, 4, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+def test_gemv_mxfp4(m):
+    rng = np.random.default_rng(40 + m)
+    n, k = 72, 2048
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                   out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+def test_gemv_batched():
+    rng = np.random.default_rng(5)
+    bsz, n, k = 3, 48, 256
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(bsz,))
+    x = O.round_bf16(rng.standard_normal((bsz, 2, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=64, bits=4, out_dtype=torch.float32))
+    for z in range(bsz):
+        assert O.rel_l2(y[z], O.qmm(x[z], words[z], s[z], b[z], 64, 4)) <= 2e-5
+
+
+def test_c1_decode_gemv_full_size():
+    wl = synth.make(1)
+    x, w, s, b, _ = synth.to_device(wl)
+    want = C.qmm(wl.x, wl.w, wl.scales, wl.biases, 64, 4, "affine")
+    y = K.quantized_matmul(x, w, s, b, group_size=64, bits=4)
+    assert O.rel_l2(out_f32(y), want) <= TOL_BF16_OUT
+    y32 = K.quantized_matmul(x, w, s, b, group_size=64, bits=4, out_dtype=torch.float32)
+    assert O.rel_l2(out_f32(y32), want) <= 1e-5
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_c2_small_batch_full_size(m):
+    wl = synth.make(2, M=m)
+    x, w, s, b, _ = synth.to_device(wl)
+    want = C.qmm(wl.x, wl.w, wl.scales, wl.biases, 64, 4, "affine")
+    y32 = K.quantized_matmul(x, w, s, b, group_size=64, bits=4, out_dtype=torch.float32)
+    assert O.rel_l2(out_f32(y32), want) <= 1e-5
+    y = K.quantized_matmul(x, w, s, b, group_size=64, bits=4)
+    assert O.rel_l2(out_f32(y), want) <= TOL_BF16_OUT
+
+
+# -------------------------------------------------------- prefill (M > 16) ----
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(17, 40, 128), (130, 200, 512), (256, 256, 1024), (64, 128, 96)])
+def test_gemm_affine(bits, gs, m, n, k):
+    if k % gs:
+        pytest.skip("K must be a multiple of the group size")
+    rng = np.random.default_rng(bits + gs + m)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    x, xd = make_x(rng, m, k)
+    want_tile = O.qmm(x, words, s, b, gs, bits, weight_rounding="bf16")
+    want_exact = O.qmm(x, words, s, b, gs, bits)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want_tile) <= 2e-5, O.rel_l2(y32, want_tile)
+    assert O.rel_l2(y32, want_exact) <= 3e-3
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits))
+    assert O.rel_l2(y16, want_exact) <= TOL_BF16_OUT
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 40, 128), (256, 136, 1024)])
+def test_gemm_mxfp4(m, n, k):
+    rng = np.random.default_rng(m + n)
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= TOL_F32_OUT, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4"))
+    assert O.rel_l2(y16, want) <= TOL_BF16_OUT
+
+
+def test_c3_prefill_scaled_and_full_size_properties():
+    wl = synth.make(3, scale=0.125, M=256)             # N = 512 rows of the same draw
+    x, w, s, b, _ = synth.to_device(wl)
+    want = C.qmm(wl.x, wl.w, wl.scales, wl.biases, 64, 8, "affine", round_tile_bf16=True)
+    y32 = K.quantized_matmul(x, w, s, b, group_size=64, bits=8, out_dtype=torch.float32)
+    assert O.rel_l2(out_f32(y32), want) <= 2e-5
+    # full size: against a float32 torch matmul on the device-dequantized bf16 tile
+    wl = synth.make(3)
+    x, w, s, b, _ = synth.to_device(wl)
+    y = K.quantized_matmul(x, w, s, b, group_size=64, bits=8, out_dtype=torch.float32)
+    tile = K.dequantize(w, s, b, group_size=64, bits=8, out_dtype=torch.bfloat16)
+    ref = x.float() @ tile.float().T
+    rel = ((y - ref).norm() / ref.norm()).item()
+    assert rel <= 1e-4, rel
+    # linearity in x (size-independent property): f(2x) == 2 f(x) exactly in f32
+    y2 = K.quantized_matmul(x * 2, w, s, b, group_size=64, bits=8, out_dtype=torch.float32)
+    assert torch.equal(y2, y * 2)
+
+
+# ----------------------------------------------------------- grouped / MoE ----
+
+def test_grouped_qmm_with_empty_and_ragged_experts():
+    rng = np.random.default_rng(21)
+    e, n, k = 5, 136, 256
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    sizes = np.array([3, 0, 130, 1, 0])
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    x, xd = make_x(rng, int(ro[-1]), k)
+    want = O.grouped_qmm(x, words, s, b, ro, 64, 4, weight_rounding="bf16")
+    y = out_f32(K.grouped_qmm(xd, wd, sd, bd, torch.from_numpy(ro).to(DEV), group_size=64, bits=4,
+                              out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+@pytest.mark.parametrize("pairs", [8, 300])
+def test_gather_qmm_unsorted_pairs(pairs):
+    """Token-major, unsorted (token, expert) pairs as mx.gather_qmm takes them."""
+    rng = np.random.default_rng(pairs)
+    e, n, k, t = 4, 64, 256, pairs // 2
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = np.repeat(np.arange(t), 2).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    rounding = "f32" if pairs <= 64 else "bf16"
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, weight_rounding=rounding)[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV),
+                             torch.from_numpy(rhs).to(DEV), group_size=64, bits=4,
+                             out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+def test_c5_moe_scaled():
+    wl = synth.make(5, scale=1 / 56)                  # N = 256, 18 tokens... of the same draw
+    x, w, s, b, ro = synth.to_device(wl)
+    want = C.grouped_qmm(wl.x, wl.w, wl.scales, wl.biases, wl.row_offsets, 64, 4, "affine",
+                         round_tile_bf16=True)
+    y = K.grouped_qmm(x, w, s, b, ro, group_size=64, bits=4, out_dtype=torch.float32)
+    assert O.rel_l2(out_f32(y), want) <= 2e-5
+
+
+# ------------------------------------------------------------ error paths ----
+
+def test_unsupported_and_bad_shapes_raise_without_launching():
+    x = torch.zeros((2, 64), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((16, 8), dtype=torch.int32, device=DEV)
+    s = torch.ones((16, 1), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(K.UnsupportedQmm):
+        K.quantized_matmul(x, w, s, s, group_size=16, bits=4)
+    with pytest.raises(K.UnsupportedQmm):
+        K.quantized_matmul(x.float(), w, s, s, group_size=64, bits=4)
+    with pytest.raises(K.QmmError):
+        K.quantized_matmul(x, w, s, None, group_size=64, bits=4)       # affine without biases
+    with pytest.raises(K.QmmError):
+        K.quantized_matmul(x.cpu(), w, s, s, group_size=64, bits=4)    # no CPU path
