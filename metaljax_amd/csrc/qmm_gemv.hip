@@ -20,189 +20,174 @@
 // 4-bit codes are widened as the bf16 value 128+q (one and-or per pair), the
 // 128 is folded into the bias; their pairs come out as (k, k+4), so the
 // activation registers are byte-permuted to the same order.
-#include "qmm_common.hpp"
+#include <type_traits>
+
+#include "qmm_gemv_common.hpp"
 
 namespace qmm {
 
 namespace {
 
-constexpr uint32_t kOnesBf16x2 = 0x3F803F80u;
-
-__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-  u32x4 v = {a, b, c, d};
-  return __builtin_bit_cast(bf16x8, v);
-}
-
-// 8 four-bit codes -> four registers of bf16 pairs (128+q_t, 128+q_{t+4}).
-__device__ __forceinline__ bf16x8 widen_int4(uint32_t w) {
-  const uint32_t m = 0x000F000Fu, one28 = 0x43004300u;
-  return as_bf16x8((w & m) | one28, ((w >> 4) & m) | one28, ((w >> 8) & m) | one28,
-                   ((w >> 12) & m) | one28);
-}
-
-// 8 eight-bit codes (two words) -> bf16 pairs in natural order.  An integer
-// below 256 is exact in the top 16 bits of its float32 form.
-__device__ __forceinline__ bf16x8 widen_int8(uint32_t w0, uint32_t w1) {
-  const float f0 = (float)(w0 & 0xFFu), f1 = (float)((w0 >> 8) & 0xFFu);
-  const float f2 = (float)((w0 >> 16) & 0xFFu), f3 = (float)(w0 >> 24);
-  const float f4 = (float)(w1 & 0xFFu), f5 = (float)((w1 >> 8) & 0xFFu);
-  const float f6 = (float)((w1 >> 16) & 0xFFu), f7 = (float)(w1 >> 24);
-  const uint32_t sel = 0x07060302u;
-  return as_bf16x8(byte_perm(__float_as_uint(f1), __float_as_uint(f0), sel),
-                   byte_perm(__float_as_uint(f3), __float_as_uint(f2), sel),
-                   byte_perm(__float_as_uint(f5), __float_as_uint(f4), sel),
-                   byte_perm(__float_as_uint(f7), __float_as_uint(f6), sel));
-}
-
-// 8 E2M1 codes -> bf16 pairs in natural order (q_2t, q_2t+1), exact: the
-// hardware converter widens the two codes of one byte at a time.
-__device__ __forceinline__ bf16x8 widen_e2m1(uint32_t w) {
-  bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 0);
-  bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 1);
-  bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 2);
-  bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 3);
-  return as_bf16x8(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
-                   __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
-}
-
-// Activations x[m, k..k+8) in natural order -> pairs (k+t, k+t+4).
-__device__ __forceinline__ bf16x8 pair_stride4(u32x4 x) {
-  const uint32_t lo = 0x05040100u, hi = 0x07060302u;
-  return as_bf16x8(byte_perm(x[2], x[0], lo), byte_perm(x[2], x[0], hi),
-                   byte_perm(x[3], x[1], lo), byte_perm(x[3], x[1], hi));
-}
-
-struct GemvArgs {
-  const uint16_t* x;   // bf16 [batch, M, K]
-  const uint32_t* w;   // [batch, N, K*bits/32]
-  const void* s;       // [batch, N, K/gs]
-  const void* b;
-  void* y;             // [batch, M, N]
-  int M, N, K;
-  int gshift;          // log2(group_size / CH)
-  int y_dtype;
-  // gather form: batch entry z multiplies x[lhs_idx[z]] by w[rhs_idx[z]]
-  const int32_t* lhs_idx;
-  const int32_t* rhs_idx;
-};
-
-// MODE: 0 affine, 1 mxfp4.  BITS: 4 or 8.  CH: K-chunk per scale application
-// (64 or 32; mxfp4: 32).  T: 16-row tiles per wavefront.  WAVES: K slices.
-template <int MODE, int BITS, int CH, int T, int WAVES, int TAB>
-__global__ __launch_bounds__(kWave* WAVES) void gemv_kernel(GemvArgs a) {
+// Affine kernel.  BITS: 4 or 8.  CH: K-chunk per scale application (64, or 32
+// for group size 32).  T: 16-row tiles per wavefront.  WAVES: K slices per
+// workgroup.  U: chunks whose loads are all issued before any is consumed --
+// the kernel lives on memory-level parallelism, a wavefront keeps U*T weight
+// loads in flight.  VT: the U = 8 scales (and biases) of a block are one
+// 16-byte load per row (16-bit tables, one table entry per chunk, aligned,
+// every block full).
+//
+// Every address is "descriptor + 32-bit lane offset + uniform offset": the
+// chunk index is wavefront-uniform, so stepping through K costs scalar
+// instructions only.  Lanes past M read the activations out of range (zeros);
+// chunks past the end of a ragged last block read their tables out of range,
+// so their scale and bias are zero.
+template <int BITS, int CH, int T, int WAVES, int TAB, int U, bool VT>
+__global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
   constexpr int STEPS = CH / 32;                 // MFMA steps per chunk
   constexpr int WPL = CH * BITS / 128;           // packed words per lane per chunk
+  constexpr int WPC = CH * BITS / 32;            // packed words per row per chunk
   constexpr int ROWS = 16 * T;
+  constexpr int TABSZ = (TAB == QMM_F32) ? 4 : 2;
   __shared__ float red[WAVES][T][4][kWave];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, kg = lane >> 4;
   const int64_t bz = blockIdx.y;
   const int64_t n0 = (int64_t)blockIdx.x * ROWS;
-  const int64_t wpr = (int64_t)a.K * BITS / 32;  // words per weight row
-  const int64_t ng = (int64_t)(a.K / CH) >> a.gshift;  // table entries per row
+  const int64_t wpr = (int64_t)a.K * BITS / 32;             // words per weight row
+  const int64_t ng = (int64_t)((a.K / CH) >> a.gshift);     // table entries per row
 
   const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
-  const uint16_t* xb = a.x + xz * a.M * (int64_t)a.K;
-  const uint32_t* wb = a.w + wz * a.N * wpr;
-  const char* sb = static_cast<const char*>(a.s);
-  const char* bb = static_cast<const char*>(a.b);
-  constexpr int TABSZ = (MODE == 1) ? 1 : (TAB == QMM_F32 ? 4 : 2);
-  sb += wz * a.N * ng * TABSZ;
-  if (MODE == 0) bb += wz * a.N * ng * TABSZ;
+  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+  const auto rw = make_rsrc(a.w + wz * a.N * wpr, a.N * wpr * 4);
+  const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
+  const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
 
   const int chunks = a.K / CH;
   const int c0 = (int)((int64_t)chunks * wave / WAVES);
   const int c1 = (int)((int64_t)chunks * (wave + 1) / WAVES);
 
-  const uint32_t* wrow[T];
-  int64_t trow[T];
+  uint32_t woff[T], toff[T];                     // lane byte offsets
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     int64_t n = n0 + t * 16 + r;
     if (n >= a.N) n = a.N - 1;
-    wrow[t] = wb + n * wpr + kg * WPL;
-    trow[t] = n * ng;
+    woff[t] = (uint32_t)((n * wpr + kg * WPL) * 4);
+    toff[t] = (uint32_t)(n * ng * TABSZ);
   }
-  const bool xvalid = r < a.M;
-  const uint16_t* xrow = xb + (int64_t)(xvalid ? r : 0) * a.K + kg * (CH / 4);
+  const uint32_t xoff = r < a.M ? (uint32_t)(((int64_t)r * a.K + kg * (CH / 4)) * 2) : kOutOfRange;
 
   f32x4 acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-  const bf16x8 ones = as_bf16x8(kOnesBf16x2, kOnesBf16x2, kOnesBf16x2, kOnesBf16x2);
+  const uint32_t one = pin_vgpr(kOnesBf16x2);
+  const bf16x8 ones = as_bf16x8(one, one, one, one);
+  const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
 
-
-  for (int c = c0; c < c1; ++c) {
-    // packed weights of this chunk, every tile
-    uint32_t q[T][WPL];
+  for (int cb = c0; cb < c1; cb += U) {
+    uint32_t q[U][T][WPL];
+    uint32_t sraw[U][T], braw[U][T];
+    u32x4 svec[T], bvec[T];
+    u32x4 xr[U][STEPS];
+    // ---- every load of the block first
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
-      const uint32_t* p = wrow[t] + (int64_t)c * (CH * BITS / 32);
-      if constexpr (WPL == 4) {
-        u32x4 v = *reinterpret_cast<const u32x4*>(p);
-        q[t][0] = v[0]; q[t][1] = v[1]; q[t][2] = v[2]; q[t][3] = v[3];
-      } else if constexpr (WPL == 2) {
-        u32x2 v = *reinterpret_cast<const u32x2*>(p);
-        q[t][0] = v[0]; q[t][1] = v[1];
-      } else {
-        q[t][0] = *p;
-      }
-    }
-    float sc[T], bi[T];
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-      const int64_t ti = trow[t] + (c >> a.gshift);
-      if constexpr (MODE == 1) {
-        sc[t] = e8m0_to_f32(reinterpret_cast<const uint8_t*>(sb)[ti]);
-        bi[t] = 0.f;
-      } else {
-        sc[t] = load_table<TAB>(sb, ti);
-        bi[t] = load_table<TAB>(bb, ti);
-        if constexpr (BITS == 4) bi[t] = fmaf(-128.f, sc[t], bi[t]);
-      }
-    }
-    // activations of this chunk: lanes past M feed zeros
-    u32x4 xr[STEPS];
-#pragma unroll
-    for (int j = 0; j < STEPS; ++j) {
-      xr[j] = u32x4{0u, 0u, 0u, 0u};
-      if (xvalid) xr[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)c * CH + j * 8);
-    }
-    f32x4 d[T];
-#pragma unroll
-    for (int t = 0; t < T; ++t) d[t] = zero;
-    f32x4 xs = zero;
-#pragma unroll
-    for (int j = 0; j < STEPS; ++j) {
-      bf16x8 xa;
-      if constexpr (MODE == 0 && BITS == 4) xa = pair_stride4(xr[j]);
-      else xa = __builtin_bit_cast(bf16x8, xr[j]);
-      if constexpr (MODE == 0)
-        xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, ones, xs, 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int c = (VT || cb + u < c1) ? cb + u : c1 - 1;          // uniform
+      const uint32_t so = (uint32_t)c * (WPC * 4);
 #pragma unroll
       for (int t = 0; t < T; ++t) {
-        bf16x8 wq;
-        if constexpr (MODE == 1) wq = widen_e2m1(q[t][j]);
-        else if constexpr (BITS == 4) wq = widen_int4(q[t][j]);
-        else wq = widen_int8(q[t][2 * j], q[t][2 * j + 1]);
-        d[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, wq, d[t], 0, 0, 0);
+        if constexpr (WPL == 4) {
+          u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rw, woff[t], so, 0);
+          q[u][t][0] = v[0]; q[u][t][1] = v[1]; q[u][t][2] = v[2]; q[u][t][3] = v[3];
+        } else if constexpr (WPL == 2) {
+          u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rw, woff[t], so, 0);
+          q[u][t][0] = v[0]; q[u][t][1] = v[1];
+        } else {
+          q[u][t][0] = __builtin_amdgcn_raw_buffer_load_b32(rw, woff[t], so, 0);
+        }
+      }
+    }
+    if constexpr (VT) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        svec[t] = __builtin_amdgcn_raw_buffer_load_b128(rs, toff[t], (uint32_t)cb * TABSZ, 0);
+        bvec[t] = __builtin_amdgcn_raw_buffer_load_b128(rb, toff[t], (uint32_t)cb * TABSZ, 0);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t so = cb + u < c1 ? (uint32_t)((cb + u) >> a.gshift) * TABSZ : kOutOfRange;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          if constexpr (TAB == QMM_F32) {
+            sraw[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rs, toff[t], so, 0);
+            braw[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rb, toff[t], so, 0);
+          } else {
+            sraw[u][t] = __builtin_amdgcn_raw_buffer_load_b16(rs, toff[t], so, 0);
+            braw[u][t] = __builtin_amdgcn_raw_buffer_load_b16(rb, toff[t], so, 0);
+          }
+        }
       }
     }
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
+    for (int u = 0; u < U; ++u) {
+      const int c = (VT || cb + u < c1) ? cb + u : c1 - 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[t][i] = fmaf(sc[t], d[t][i], acc[t][i]);
-        if constexpr (MODE == 0) acc[t][i] = fmaf(bi[t], xs[i], acc[t][i]);
+      for (int j = 0; j < STEPS; ++j)
+        xr[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff, (uint32_t)(c * CH + j * 8) * 2, 0);
+    }
+    // ---- then the arithmetic
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      f32x4 d[T];
+      f32x4 xs;
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j) {
+        bf16x8 xa;
+        if constexpr (BITS == 4) xa = pair_stride4(xr[u][j]);
+        else xa = __builtin_bit_cast(bf16x8, xr[u][j]);
+        xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, ones, j ? xs : zero, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          bf16x8 wq;
+          if constexpr (BITS == 4) wq = widen_int4(q[u][t][j], nib, magic);
+          else wq = widen_int8(q[u][t][2 * j], q[u][t][2 * j + 1]);
+          d[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, wq, j ? d[t] : zero, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        float sc, bi;
+        if constexpr (VT) {
+          const uint32_t sw = svec[t][u >> 1], bw = bvec[t][u >> 1];
+          if constexpr (TAB == QMM_BF16) {
+            sc = __uint_as_float((u & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
+            bi = __uint_as_float((u & 1) ? (bw & 0xFFFF0000u) : (bw << 16));
+          } else {
+            sc = f16_bits_to_f32((u & 1) ? (sw >> 16) : (sw & 0xFFFFu));
+            bi = f16_bits_to_f32((u & 1) ? (bw >> 16) : (bw & 0xFFFFu));
+          }
+        } else if constexpr (TAB == QMM_F32) {
+          sc = __uint_as_float(sraw[u][t]); bi = __uint_as_float(braw[u][t]);
+        } else if constexpr (TAB == QMM_BF16) {
+          sc = bf16_bits_to_f32(sraw[u][t]); bi = bf16_bits_to_f32(braw[u][t]);
+        } else {
+          sc = f16_bits_to_f32(sraw[u][t]); bi = f16_bits_to_f32(braw[u][t]);
+        }
+        if constexpr (BITS == 4) bi = fmaf(-128.f, sc, bi);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[t][i] = fmaf(sc, d[t][i], acc[t][i]);
+          acc[t][i] = fmaf(bi, xs[i], acc[t][i]);
+        }
       }
     }
   }
 
-  // meet the K slices in LDS
+  // ---- meet the K slices in LDS
 #pragma unroll
   for (int t = 0; t < T; ++t)
 #pragma unroll
@@ -219,36 +204,176 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_kernel(GemvArgs a) {
   }
 }
 
-template <int MODE, int BITS, int CH, int T, int WAVES, int TAB>
-void launch(const GemvArgs& a, int64_t batch, hipStream_t st) {
-  dim3 grid((unsigned)ceil_div(a.N, 16 * T), (unsigned)batch);
-  hipLaunchKernelGGL((gemv_kernel<MODE, BITS, CH, T, WAVES, TAB>), grid, dim3(kWave * WAVES), 0,
-                     st, a);
+// MXFP4 kernel.  A lane's 16-byte load is exactly one 32-element MX block, so
+// the block's power-of-two scale rides along in the hardware fp4 -> bf16
+// conversion (exact: an E2M1 value has one mantissa bit) and the products need
+// no rescaling afterwards.  One macro chunk = 128 k = four MFMA steps.
+template <int T, int WAVES, int U>
+__global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
+  constexpr int ROWS = 16 * T;
+  __shared__ float red[WAVES][T][4][kWave];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int64_t bz = blockIdx.y;
+  const int64_t n0 = (int64_t)blockIdx.x * ROWS;
+  const int64_t wpr = (int64_t)a.K / 8;
+  const int nblk = a.K / 32;                       // MX blocks per row
+
+  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  const uint16_t* xb = a.x + xz * a.M * (int64_t)a.K;
+  const uint32_t* wb = a.w + wz * a.N * wpr;
+  const uint8_t* sb = static_cast<const uint8_t*>(a.s) + wz * a.N * (int64_t)nblk;
+
+  const int chunks = (nblk + 3) / 4;               // macro chunks of 128 k
+  const int c0 = (int)((int64_t)chunks * wave / WAVES);
+  const int c1 = (int)((int64_t)chunks * (wave + 1) / WAVES);
+
+  const uint32_t* wrow[T];
+  const uint8_t* srow[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    int64_t n = n0 + t * 16 + r;
+    if (n >= a.N) n = a.N - 1;
+    wrow[t] = wb + n * wpr;
+    srow[t] = sb + n * nblk;
+  }
+  const bool xvalid = r < a.M;
+  const uint16_t* xrow = xb + (int64_t)(xvalid ? r : 0) * a.K;
+
+  f32x4 acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int cb = c0; cb < c1; cb += U) {
+    u32x4 q[U][T];
+    uint8_t sraw[U][T];
+    u32x4 xr[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int blk = (cb + u) * 4 + kg;
+      if (cb + u >= c1 || blk >= nblk) blk = nblk - 1;
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+        q[u][t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[t] + (int64_t)blk * 4));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int blk = (cb + u) * 4 + kg;
+      if (cb + u >= c1 || blk >= nblk) blk = nblk - 1;
+#pragma unroll
+      for (int t = 0; t < T; ++t) sraw[u][t] = srow[t][blk];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int blk = (cb + u) * 4 + kg;
+      const bool live = cb + u < c1 && blk < nblk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        xr[u][j] = u32x4{0u, 0u, 0u, 0u};
+        if (xvalid && live)
+          xr[u][j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)blk * 32 + j * 8);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const float sc = e8m0_to_f32(sraw[u][t]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8 xa = __builtin_bit_cast(bf16x8, xr[u][j]);   // zero where not live
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, widen_e2m1(q[u][t][j], sc), acc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t][i][lane] = acc[t][i];
+  __syncthreads();
+  for (int e = threadIdx.x; e < T * 4 * kWave; e += kWave * WAVES) {
+    const int l = e & 63, i = (e >> 6) & 3, t = e >> 8;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][i][l];
+    const int m = 4 * (l >> 4) + i;
+    const int64_t n = n0 + t * 16 + (l & 15);
+    if (m < a.M && n < a.N) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+  }
 }
 
-template <int MODE, int BITS, int CH, int TAB>
-void launch_shape(const GemvArgs& a, int64_t batch, int t, int waves, hipStream_t st) {
-  if (t == 1 && waves == 4) launch<MODE, BITS, CH, 1, 4, TAB>(a, batch, st);
-  else if (t == 1 && waves == 8) launch<MODE, BITS, CH, 1, 8, TAB>(a, batch, st);
-  else if (t == 2 && waves == 4) launch<MODE, BITS, CH, 2, 4, TAB>(a, batch, st);
-  else if (t == 2 && waves == 8) launch<MODE, BITS, CH, 2, 8, TAB>(a, batch, st);
-  else launch<MODE, BITS, CH, 1, 4, TAB>(a, batch, st);
+struct Geometry { int t, waves, u; };
+
+template <int BITS, int CH, int TAB, int T, int WAVES, int U>
+void launch_affine_k(const GemvArgs& a, int64_t batch, hipStream_t st) {
+  dim3 grid((unsigned)ceil_div(a.N, 16 * T), (unsigned)batch);
+  // vector table loads: 16-bit tables, one entry per chunk, 16-byte aligned runs
+  const int chunks = a.K / CH;
+  bool vt = false;
+  if constexpr (TAB != QMM_F32 && U == 8) {
+    vt = a.gshift == 0 && chunks % (8 * WAVES) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.s) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.b) & 15u) == 0;
+    if (vt) {
+      hipLaunchKernelGGL((gemv_affine_kernel<BITS, CH, T, WAVES, TAB, U, true>), grid, dim3(kWave * WAVES), 0, st, a);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemv_affine_kernel<BITS, CH, T, WAVES, TAB, U, false>), grid, dim3(kWave * WAVES), 0, st, a);
+}
+
+template <int BITS, int CH, int TAB>
+void launch_affine_g(const GemvArgs& a, int64_t batch, Geometry g, hipStream_t st) {
+#define QMM_CASE(TT, WW, UU) \
+  if (g.t == TT && g.waves == WW && g.u == UU) return launch_affine_k<BITS, CH, TAB, TT, WW, UU>(a, batch, st)
+  QMM_CASE(1, 4, 4); QMM_CASE(1, 4, 8); QMM_CASE(1, 8, 4); QMM_CASE(1, 8, 8);
+  QMM_CASE(2, 4, 4); QMM_CASE(2, 4, 8); QMM_CASE(2, 8, 4); QMM_CASE(2, 8, 8);
+  QMM_CASE(1, 16, 4); QMM_CASE(2, 16, 4);
+#undef QMM_CASE
+  launch_affine_k<BITS, CH, TAB, 1, 8, 8>(a, batch, st);
 }
 
 template <int BITS, int CH>
-void launch_affine(const GemvArgs& a, int64_t batch, int tab, int t, int waves, hipStream_t st) {
-  if (tab == QMM_BF16) launch_shape<0, BITS, CH, QMM_BF16>(a, batch, t, waves, st);
-  else if (tab == QMM_F32) launch_shape<0, BITS, CH, QMM_F32>(a, batch, t, waves, st);
-  else launch_shape<0, BITS, CH, QMM_F16>(a, batch, t, waves, st);
+void launch_affine(const GemvArgs& a, int64_t batch, int tab, Geometry g, hipStream_t st) {
+  if (tab == QMM_BF16) launch_affine_g<BITS, CH, QMM_BF16>(a, batch, g, st);
+  else if (tab == QMM_F32) launch_affine_g<BITS, CH, QMM_F32>(a, batch, g, st);
+  else launch_affine_g<BITS, CH, QMM_F16>(a, batch, g, st);
+}
+
+template <int T, int WAVES, int U>
+void launch_mxfp4_k(const GemvArgs& a, int64_t batch, hipStream_t st) {
+  dim3 grid((unsigned)ceil_div(a.N, 16 * T), (unsigned)batch);
+  hipLaunchKernelGGL((gemv_mxfp4_kernel<T, WAVES, U>), grid, dim3(kWave * WAVES), 0, st, a);
+}
+
+void launch_mxfp4(const GemvArgs& a, int64_t batch, Geometry g, hipStream_t st) {
+#define QMM_CASE(TT, WW, UU) \
+  if (g.t == TT && g.waves == WW && g.u == UU) return launch_mxfp4_k<TT, WW, UU>(a, batch, st)
+  QMM_CASE(1, 4, 4); QMM_CASE(1, 4, 8); QMM_CASE(1, 8, 4); QMM_CASE(1, 8, 8);
+  QMM_CASE(2, 4, 4); QMM_CASE(2, 8, 4); QMM_CASE(2, 8, 8);
+#undef QMM_CASE
+  launch_mxfp4_k<1, 8, 4>(a, batch, st);
+}
+
+int env_int(const char* name) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : 0;
 }
 
 }  // namespace
 
-// Tile/slice choice.  Overridable for experiments through QMM_GEMV_T /
-// QMM_GEMV_WAVES (read once).
+bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* s,
+                      const void* b);
+void skinny_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int tab, hipStream_t st);
+
+// Tile / slice / unroll choice; QMM_GEMV_T, QMM_GEMV_WAVES and QMM_GEMV_U
+// override it for experiments (read once).
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves) {
-  static const int env_t = [] { const char* e = getenv("QMM_GEMV_T"); return e ? atoi(e) : 0; }();
-  static const int env_w = [] { const char* e = getenv("QMM_GEMV_WAVES"); return e ? atoi(e) : 0; }();
+  static const int env_t = env_int("QMM_GEMV_T"), env_w = env_int("QMM_GEMV_WAVES");
   int tt = (M > 8 && N >= 4096) ? 2 : 1;
   int ww = (K >= 4096) ? 8 : 4;
   if (env_t) tt = env_t;
@@ -262,6 +387,7 @@ void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves) {
 void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int gs, int bits,
                    int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st) {
+  static const int env_u = env_int("QMM_GEMV_U");
   GemvArgs a;
   a.x = static_cast<const uint16_t*>(x);
   a.w = static_cast<const uint32_t*>(w);
@@ -274,21 +400,28 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
   a.y_dtype = y_dtype;
   a.lhs_idx = lhs_idx;
   a.rhs_idx = rhs_idx;
-  int t, waves;
-  gemv_geometry(M, N, K, &t, &waves);
+  static const int no_skinny = env_int("QMM_NO_SKINNY");
+  if (!no_skinny && skinny_supported(N, K, gs, bits, mode, tab, s, b)) {
+    skinny_dispatch(a, batch, gs, bits, tab, st);
+    return;
+  }
+  Geometry g;
+  gemv_geometry(M, N, K, &g.t, &g.waves);
+  g.u = env_u ? env_u : 8;
   if (mode == QMM_MODE_MXFP4) {
     a.gshift = 0;
-    launch_shape<1, 4, 32, QMM_BF16>(a, batch, t, waves, st);
+    if (!env_u) g.u = 4;
+    launch_mxfp4(a, batch, g, st);
     return;
   }
   const int ch = gs >= 64 ? 64 : 32;
   a.gshift = (gs == 128) ? 1 : 0;
   if (bits == 4) {
-    if (ch == 64) launch_affine<4, 64>(a, batch, tab, t, waves, st);
-    else launch_affine<4, 32>(a, batch, tab, t, waves, st);
+    if (ch == 64) launch_affine<4, 64>(a, batch, tab, g, st);
+    else launch_affine<4, 32>(a, batch, tab, g, st);
   } else {
-    if (ch == 64) launch_affine<8, 64>(a, batch, tab, t, waves, st);
-    else launch_affine<8, 32>(a, batch, tab, t, waves, st);
+    if (ch == 64) launch_affine<8, 64>(a, batch, tab, g, st);
+    else launch_affine<8, 32>(a, batch, tab, g, st);
   }
 }
 
