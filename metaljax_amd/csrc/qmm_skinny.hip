@@ -71,7 +71,7 @@ __device__ __forceinline__ void load_tile(u32x4 (&w)[4], __amdgpu_buffer_rsrc_t 
   }
 }
 
-template <int BITS, int WAVES, int TMAX>
+template <int BITS, int WAVES, int TMAX, int GSHIFT>
 __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a, int rows_per_wg) {
   constexpr int KS = kSliceBytes * 8 / BITS;      // codes per slice: 512 | 256
   constexpr int CPS = KS / 64;                    // 64-code chunks per slice: 8 | 4
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
   const int64_t n_end = n_begin + rows_per_wg < a.N ? n_begin + rows_per_wg : a.N;
   const int ntiles = (int)((n_end - n_begin + 15) / 16);        // uniform, <= TMAX
   const int64_t wpr = (int64_t)a.K * BITS / 8;                  // bytes per weight row
-  const int64_t ng = (int64_t)(a.K / 64) >> a.gshift;           // table entries per row
+  const int64_t ng = (int64_t)(a.K / 64) >> GSHIFT;             // table entries per row
   const int slices = a.K / KS;
 
   const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
@@ -112,21 +112,12 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
 
   for (int sl = wave; sl < slices; sl += WAVES) {
     const uint32_t slice_off = (uint32_t)sl * kSliceBytes;
-    const uint32_t tab_off = (uint32_t)((sl * CPS) >> a.gshift) * 2;
-    // ---- issue the global loads: activations first (needed first), then two tiles
-    u32x4 xl[XR][4];
-#pragma unroll
-    for (int rd = 0; rd < XR; ++rd)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = 4 * i + lrow;
-        const uint32_t vo = m < a.M ? (uint32_t)(((int64_t)m * a.K) * 2 + lpiece * 16) : kOutOfRange;
-        xl[rd][i] = __builtin_amdgcn_raw_buffer_load_b128(rx, vo, (uint32_t)(sl * KS + rd * 128) * 2, 0);
-      }
-    // Table rows: lanes 0-15 fetch the 16 scale rows of a tile, lanes 16-31 the
-    // bias rows (one 16-byte run each, 32 L1 requests per tile); they reach
-    // every lane through LDS.
+    const uint32_t tab_off = (uint32_t)((sl * CPS) >> GSHIFT) * 2;
+    // ---- issue the global loads: the first tile (HBM, longest latency), the
+    // activations (row blocks at or past M are not fetched), then the second tile
     u32x4 wl[2][4], tv[2];
+    // Table rows: lanes 0-15 fetch the 16 scale rows of a tile, lanes 16-31 the
+    // bias rows (one 16-byte run each); they reach every lane through LDS.
     auto load_tables = [&](int t, int set) {
       const int64_t n = n_begin + t * 16 + r;
       const uint32_t to = (uint32_t)(n * ng * 2);
@@ -135,6 +126,20 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
       tv[set] = vs | vb;                        // the lanes that miss read zeros
     };
     load_tile(wl[0], rw, n_begin, n_end, wpr, lrow, lpiece, slice_off);
+    u32x4 xl[XR][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool any = 4 * i < a.M;                              // uniform
+#pragma unroll
+      for (int rd = 0; rd < XR; ++rd) {
+        xl[rd][i] = u32x4{0u, 0u, 0u, 0u};
+        if (any) {
+          const int m = 4 * i + lrow;
+          const uint32_t vo = m < a.M ? (uint32_t)(((int64_t)m * a.K) * 2 + lpiece * 16) : kOutOfRange;
+          xl[rd][i] = __builtin_amdgcn_raw_buffer_load_b128(rx, vo, (uint32_t)(sl * KS + rd * 128) * 2, 0);
+        }
+      }
+    }
     load_tables(0, 0);
     if (TMAX > 1 && ntiles > 1) {
       load_tile(wl[1], rw, n_begin + 16, n_end, wpr, lrow, lpiece, slice_off);
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
         // table rows as B operands over the chunk index (lane's row, entries of this slice)
         u32x4 svt = *reinterpret_cast<const u32x4*>(tbuf + r * 16);
         u32x4 bvt = *reinterpret_cast<const u32x4*>(tbuf + 256 + r * 16);
-        if (a.gshift) {   // group 128: one entry serves two chunks -> duplicate each bf16
+        if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
           svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
                       byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
           bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
@@ -263,7 +268,10 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
 template <int BITS, int WAVES, int TMAX>
 void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch);
-  hipLaunchKernelGGL((skinny_affine_kernel<BITS, WAVES, TMAX>), grid, dim3(kWave * WAVES), 0, st, a, rows_per_wg);
+  if (a.gshift)
+    hipLaunchKernelGGL((skinny_affine_kernel<BITS, WAVES, TMAX, 1>), grid, dim3(kWave * WAVES), 0, st, a, rows_per_wg);
+  else
+    hipLaunchKernelGGL((skinny_affine_kernel<BITS, WAVES, TMAX, 0>), grid, dim3(kWave * WAVES), 0, st, a, rows_per_wg);
 }
 
 template <int BITS>

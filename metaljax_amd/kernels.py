@@ -212,3 +212,34 @@ def plan(m, n, k, group_size=64, bits=4, mode="affine"):
     lib.qmm_plan(m, n, k, group_size, bits, _MODE[mode], ctypes.byref(a), ctypes.byref(b),
                  ctypes.byref(c))
     return a.value, b.value, c.value
+
+
+class BoundQmm:
+    """A quantized_matmul call with every argument resolved once.
+
+    For launch-bound loops (decode steps, benchmarks, HIP-graph capture): the
+    tensors are validated and kept alive here and `launch()` only issues the
+    library call on the current stream into the preallocated `y`.
+    """
+
+    def __init__(self, x, w, scales, biases, y, group_size=64, bits=4, mode="affine"):
+        _need_cuda(x, w, scales, biases, y)
+        lead, n, k = _weight_dims(w, bits, mode)
+        if lead or x.dim() != 2:
+            raise UnsupportedQmm(3, "BoundQmm serves the unbatched [M,K] x [N,K] form")
+        for t in (x, w, scales, biases, y):
+            if t is not None and not t.is_contiguous():
+                raise _lib.QmmError(1, "BoundQmm needs contiguous tensors")
+        self._keep = (x, w, scales, biases, y)
+        self._lib = _lib.load()
+        tab = _dt(scales.dtype) if mode == "affine" else BF16
+        self._args = (_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y),
+                      _dt(y.dtype), 1, x.shape[0], n, k, group_size, bits, _MODE[mode], None, 0)
+        self.y = y
+
+    def launch(self, stream=None):
+        st = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        rc = self._lib.qmm_quantized_matmul(*self._args, st)
+        if rc:
+            _lib.check(rc)
+        return self.y
