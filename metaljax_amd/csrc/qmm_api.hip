@@ -14,9 +14,9 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
 void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
-                   const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
-                   int bits, int mode, hipStream_t st);
-int64_t gemm_row_tile();
+                   const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
+                   int64_t K, int gs, int bits, int mode, hipStream_t st);
+int64_t gemm_row_tile(int64_t R, int64_t E);
 void unpack_dispatch(const void* w, void* codes, int64_t rows, int64_t K, int bits, hipStream_t st);
 void pack_dispatch(const void* codes, void* w, int64_t rows, int64_t K, int bits, hipStream_t st);
 void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void* out,
@@ -152,7 +152,7 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int, int* kernel, int* g
     if (grid) *grid = (int)ceil_div(N, 16 * t);
     if (block) *block = 64 * waves;
   } else {
-    const int64_t bm = gemm_row_tile();
+    const int64_t bm = gemm_row_tile(M, 1);
     if (kernel) *kernel = QMM_KERNEL_GEMM;
     if (grid) *grid = (int)(ceil_div(N, 128) * ceil_div(M, bm));
     if (block) *block = 256;
@@ -171,7 +171,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
   if (rc) return rc;
   rc = check_io(x, x_dtype, y, y_dtype);
   if (rc) return rc;
-  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535)
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535 || M * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (M <= kGemvMaxM) {
@@ -190,7 +190,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
                   static_cast<const char*>(scales) + z * N * ng * tabsz,
                   biases ? static_cast<const char*>(biases) + z * N * ng * tabsz : nullptr,
                   table_dtype, static_cast<char*>(y) + z * M * N * ysz, y_dtype, nullptr, nullptr,
-                  nullptr, M, 1, N, K, group_size, bits, mode, st);
+                  nullptr, M, M, 1, N, K, group_size, bits, mode, st);
     rc = check_launch("gemm launch");
     if (rc) return rc;
   }
@@ -208,10 +208,10 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   if (rc) return rc;
   rc = check_io(x, x_dtype, y, y_dtype);
   if (rc) return rc;
-  if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535)
+  if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535 || R * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
   gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
-                E, N, K, group_size, bits, mode, static_cast<hipStream_t>(stream));
+                R, E, N, K, group_size, bits, mode, static_cast<hipStream_t>(stream));
   return check_launch("grouped gemm launch");
 }
 
@@ -227,7 +227,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   if (rc) return rc;
   rc = check_io(x, x_dtype, y, y_dtype);
   if (rc) return rc;
-  if (P > INT32_MAX / 2 || N > INT32_MAX || K > INT32_MAX || E > 65535)
+  if (P > INT32_MAX / 2 || N > INT32_MAX || K > INT32_MAX || E > 65535 || T * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (P <= kGatherGemvMaxPairs) {
@@ -247,7 +247,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
                      ro, cursor, src_row, out_row);
   rc = check_launch("route launch");
   if (rc) return rc;
-  gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, E, N, K,
+  gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
                 group_size, bits, mode, st);
   return check_launch("gather gemm launch");
 }
