@@ -1,0 +1,91 @@
+"""The C-ABI library: it loads, exports every function include/qmm_hip.h
+declares, and its host-only entry points (no device work) behave.  Runs
+without a GPU; no compute entry point is called here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from metaljax_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "qmm_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return sorted(set(re.findall(r"\b(qmm_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        from metaljax_amd import build
+        build.build()
+    return _lib.load()
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(_lib.SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(raw, name), name
+
+
+def test_header_cites_the_reference_for_every_entry_point():
+    text = open(HEADER).read()
+    # each declaration is preceded by a comment naming the reference call it replaces
+    for name in declared_functions():
+        if name in ("qmm_abi_version", "qmm_last_error", "qmm_workspace_bytes",
+                    "qmm_gather_workspace_bytes", "qmm_plan"):
+            continue
+        head = text[:text.index(name + "(")]
+        comment = head[head.rindex("/*"):]
+        assert re.search(r"\.py:\d+", comment), f"{name}: no reference citation"
+
+
+def test_abi_version_and_error_text(lib):
+    assert lib.qmm_abi_version() >= 1
+    assert isinstance(lib.qmm_last_error(), bytes)
+
+
+def test_plan_picks_the_regime(lib):
+    k, g, b = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.qmm_plan(1, 4096, 4096, 64, 4, 0, k, g, b) == 0
+    assert k.value == _lib.KERNEL_GEMV and g.value > 0 and b.value % 64 == 0
+    assert lib.qmm_plan(16, 14336, 4096, 64, 4, 0, k, g, b) == 0
+    assert k.value == _lib.KERNEL_GEMV
+    assert lib.qmm_plan(2048, 4096, 4096, 64, 8, 0, k, g, b) == 0
+    assert k.value == _lib.KERNEL_GEMM and g.value >= 256
+
+
+def test_workspace_queries_need_no_device(lib):
+    assert lib.qmm_workspace_bytes(1, 16, 14336, 4096, 64, 4, 0, _lib.BF16) == 0
+    need = lib.qmm_gather_workspace_bytes(1024, 8)
+    assert need > 0 and need % 4 == 0
+    assert lib.qmm_gather_workspace_bytes(0, 8) >= 0
+
+
+def test_argument_errors_are_reported_before_any_launch(lib):
+    # null pointers / bad enums are rejected on the host (no GPU needed)
+    rc = lib.qmm_quantized_matmul(None, _lib.BF16, None, None, None, _lib.BF16, None, _lib.BF16,
+                                  1, 1, 64, 64, 64, 4, 0, None, 0, None)
+    assert rc != 0
+    assert lib.qmm_last_error()
+    rc = lib.qmm_quantized_matmul(None, _lib.BF16, None, None, None, _lib.BF16, None, _lib.BF16,
+                                  1, 1, 64, 48, 64, 4, 0, None, 0, None)
+    assert rc in (1, 2, 3)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libqmm_hip.so"))
+    with pytest.raises(_lib.QmmLibraryError):
+        _lib.load()
