@@ -17,6 +17,11 @@ void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, i
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
                    int64_t K, int gs, int bits, int mode, hipStream_t st);
 int64_t gemm_row_tile(int64_t R, int64_t E);
+bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K);
+size_t mxfp4_workspace_bytes(int64_t R, int64_t K);
+void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block);
+void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, int y_dtype,
+                         int64_t R, int64_t N, int64_t K, void* workspace, hipStream_t st);
 void unpack_dispatch(const void* w, void* codes, int64_t rows, int64_t K, int bits, hipStream_t st);
 void pack_dispatch(const void* codes, void* w, int64_t rows, int64_t K, int bits, hipStream_t st);
 void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void* out,
@@ -138,13 +143,26 @@ int qmm_abi_version(void) { return 1; }
 
 const char* qmm_last_error(void) { return g_err; }
 
-size_t qmm_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int, int, int, int) { return 0; }
+size_t qmm_workspace_bytes(int64_t, int64_t M, int64_t N, int64_t K, int, int, int mode, int) {
+  if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K))
+    return mxfp4_workspace_bytes(M, K);
+  return 0;
+}
 
 size_t qmm_gather_workspace_bytes(int64_t P, int64_t E) {
   return P <= kGatherGemvMaxPairs ? 0 : route_bytes(P, E);
 }
 
-int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int, int* kernel, int* grid, int* block) {
+int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int mode, int* kernel, int* grid,
+             int* block) {
+  if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K)) {
+    int g, b;
+    mxfp4_geometry(M, N, &g, &b);
+    if (kernel) *kernel = QMM_KERNEL_MXFP4_MFMA;
+    if (grid) *grid = g;
+    if (block) *block = b;
+    return QMM_OK;
+  }
   if (M <= kGemvMaxM) {
     int t, waves;
     gemv_geometry(M, N, K, &t, &waves);
@@ -163,7 +181,8 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int, int* kernel, int* g
 int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* scales,
                          const void* biases, int table_dtype, void* y, int y_dtype,
                          int64_t batch, int64_t M, int64_t N, int64_t K, int group_size,
-                         int bits, int mode, void*, size_t, void* stream) {
+                         int bits, int mode, void* workspace, size_t workspace_bytes,
+                         void* stream) {
   if (batch < 0 || M < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
   if (batch == 0 || M == 0 || N == 0) return QMM_OK;
   if (K == 0) return fail(QMM_ERR_BAD_SHAPE, "K=0");
@@ -184,6 +203,24 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
   const int64_t ng = mode == QMM_MODE_MXFP4 ? K / 32 : K / group_size;
   const int tabsz = mode == QMM_MODE_MXFP4 ? 1 : (table_dtype == QMM_F32 ? 4 : 2);
   const int ysz = y_dtype == QMM_F32 ? 4 : 2;
+  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(M, N, K)) {
+    // block-scaled matrix cores; the activations are split into the workspace first
+    const size_t need = mxfp4_workspace_bytes(M, K);
+    if (!workspace || workspace_bytes < need)
+      return fail(QMM_ERR_WORKSPACE, "mxfp4 needs %zu workspace bytes, got %zu", need,
+                  workspace ? workspace_bytes : (size_t)0);
+    if (!aligned16(workspace) || !aligned16(scales))
+      return fail(QMM_ERR_BAD_ARGUMENT, "workspace / scale pointer not 16-byte aligned");
+    for (int64_t z = 0; z < batch; ++z) {
+      mxfp4_mfma_dispatch(static_cast<const char*>(x) + z * M * K * 2,
+                          static_cast<const uint32_t*>(w) + z * N * wpr,
+                          static_cast<const char*>(scales) + z * N * ng,
+                          static_cast<char*>(y) + z * M * N * ysz, y_dtype, M, N, K, workspace, st);
+      rc = check_launch("mxfp4 launch");
+      if (rc) return rc;
+    }
+    return QMM_OK;
+  }
   for (int64_t z = 0; z < batch; ++z) {
     gemm_dispatch(static_cast<const char*>(x) + z * M * K * 2,
                   static_cast<const uint32_t*>(w) + z * N * wpr,

@@ -1,0 +1,462 @@
+// MXFP4 quantized matmul on the gfx950 block-scaled matrix cores
+// (v_mfma_scale_f32_32x32x64_f8f6f4), for M > 16 and K a multiple of 512.
+//
+// y[m, n] = sum_k x[m, k] * E2M1[code[n, k]] * 2^(scale[n, k/32] - 127)
+//
+// The weight operand goes to the matrix core exactly as stored: 32 four-bit
+// codes (16 bytes) a lane plus the E8M0 byte of that 32-block, so the
+// dequantized weight is exact by construction.  The instruction needs the
+// other operand in a block-scaled narrow format too, so the bf16 activations
+// are split once per call into two FP6 (E2M3) terms, each with one E8M0 scale
+// per 32 elements:
+//     x = hi + lo + eps,   hi = fp6(x),  lo = fp6(x - hi)   (x - hi is exact)
+// which leaves |eps| around 3e-4 of |x| (rms over a 32-block), far inside the
+// output tolerance, at the cost of issuing two MFMAs per useful one.
+//
+// Kernel 1 (mx_split_kernel): x [R, K] bf16 -> the two FP6 terms in the order
+// the matrix core reads them.  A lane's operand is one row's 32-block: 24
+// bytes a term, 48 bytes for both = three 16-byte planes (hi | lo back to
+// back).  For K-step ks (128 elements = 32-blocks kb = 0..3; one 32x32x64 MFMA
+// covers blocks 2u, 2u+1):
+//     aq[ks][plane][kb][row]     (16 bytes each, rows contiguous)
+// so a wavefront's operand load is two 512-byte runs for any first row, and
+//     as[ks/4][t][kb][row]       (4 bytes: the E8M0 bytes of K-steps 4q..4q+3)
+// so one scale register serves four K-steps through the instruction's byte
+// select.
+//
+// Kernel 2 (mxfp4_mfma_kernel): one workgroup = a 64 x 128 output tile, four
+// wavefronts that split K (wavefront w owns K-quads w, w+4, ...; a quad is
+// four K-steps) and are summed through LDS at the end.  No barrier in the main
+// loop: each wavefront stages its own weight codes.
+//   * weight codes: direct-to-LDS loads, 16 bytes a lane, four lanes = one
+//     row's 64 bytes of a K-step (coalesced), into a 4-deep ring; read back
+//     with ds_read_b128 in operand order (lane = column i, block 2u + lane/32).
+//     The 16-byte piece p of row i sits at piece p ^ ((i >> 2) & 3), applied on
+//     the global side of the load, so a 16-lane read phase covers all banks.
+//   * weight scales: 16 bytes a row per K-quad, direct-to-LDS, double buffered;
+//     the lane shifts its block's byte to bits 0-7.
+//   * activation terms: straight from global (L2-resident) into operand
+//     registers, two K-steps ahead.
+// Per K-step a wavefront issues 32 MFMAs of 32x32x64 (2 K-halves x 2 terms x 2
+// row tiles x 4 column tiles) against 24 + 8 loads.  (The 16x16x128 form of
+// the instruction sustains well under half the rate of the 32x32x64 form.)
+#include <type_traits>
+
+#include "qmm_common.hpp"
+
+namespace qmm {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(32))) __bf16 bf16x32;
+typedef __attribute__((ext_vector_type(32))) float f32x32;
+typedef __attribute__((ext_vector_type(16))) unsigned u32x16;
+typedef __attribute__((ext_vector_type(6))) unsigned u32x6;
+
+constexpr int TM = 64, TN = 128;
+constexpr int kStageBytes = TN * 64;             // 128 rows x 64 bytes of codes: one K-step
+constexpr int kStages = 4;
+constexpr int kScaleBytes = TN * 16;             // 128 rows x 16 scale bytes: one K-quad
+constexpr int kWaveLds = kStages * kStageBytes + 2 * kScaleBytes;   // 36864
+constexpr int kLds = 4 * kWaveLds;               // 147456
+constexpr uint32_t kOutOfRange = 0x80000000u;
+constexpr int kFp6 = 2, kFp4 = 4;                // matrix-core format selectors (E2M3, E2M1)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
+  const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {    // s_waitcnt vmcnt(N) only; also a compiler barrier
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+  asm volatile("" ::: "memory");
+}
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, unsigned char* dst, uint32_t voff,
+                                      uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, voff, soff, 0, 0);
+}
+
+// E8M0 byte of the scale that maps a block whose largest magnitude has float
+// exponent field `e` into the FP6 E2M3 range (largest binade 4 .. 7.5).
+__device__ __forceinline__ uint32_t block_scale_byte(uint32_t e) {
+  const int b = (int)e - 2;
+  return (uint32_t)(b < 1 ? 1 : (b > 254 ? 254 : b));
+}
+
+// ---------------------------------------------------------------------------
+// x [R, K] bf16 -> two FP6 terms + scales in matrix-core operand order.
+// One thread = one (row, 32-block); consecutive threads = consecutive rows.
+__global__ __launch_bounds__(256) void mx_split_kernel(const uint16_t* __restrict__ x,
+                                                       u32x4* __restrict__ aq,
+                                                       uint8_t* __restrict__ as, int R, int K,
+                                                       int Rp) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int row = (int)(idx % Rp);
+  const int blk = (int)(idx / Rp);
+  if (blk >= K / 32 || row >= R) return;
+  const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)row * K + blk * 32);
+  u32x16 raw;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const u32x4 v = src[i];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) raw[4 * i + j] = v[j];
+  }
+  uint32_t amax = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t lo = raw[i] & 0x7FFFu, hi = (raw[i] >> 16) & 0x7FFFu;
+    amax = max(amax, max(lo, hi));
+  }
+  const uint32_t byte_hi = block_scale_byte(amax >> 7);
+  const float scale_hi = __uint_as_float(byte_hi << 23);
+  const bf16x32 xv = __builtin_bit_cast(bf16x32, raw);
+  const u32x6 hi6 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(xv, scale_hi);
+  const f32x32 back = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(hi6, scale_hi);
+  // residual: exact in float32, and representable in bf16 (a multiple of
+  // ulp(x) that is smaller than x), so the truncation below loses nothing
+  u32x16 res;
+  uint32_t rmax = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float r0 = __uint_as_float(raw[i] << 16) - back[2 * i];
+    const float r1 = __uint_as_float(raw[i] & 0xFFFF0000u) - back[2 * i + 1];
+    const uint32_t b0 = __float_as_uint(r0), b1 = __float_as_uint(r1);
+    rmax = max(rmax, max(b0 & 0x7FFFFFFFu, b1 & 0x7FFFFFFFu));
+    res[i] = (b0 >> 16) | (b1 & 0xFFFF0000u);
+  }
+  const uint32_t byte_lo = block_scale_byte(rmax >> 23);
+  const float scale_lo = __uint_as_float(byte_lo << 23);
+  const u32x6 lo6 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(__builtin_bit_cast(bf16x32, res), scale_lo);
+
+  const int ks = blk >> 2, kb = blk & 3;
+  const u32x4 planes[3] = {u32x4{hi6[0], hi6[1], hi6[2], hi6[3]}, u32x4{hi6[4], hi6[5], lo6[0], lo6[1]},
+                           u32x4{lo6[2], lo6[3], lo6[4], lo6[5]}};
+#pragma unroll
+  for (int p = 0; p < 3; ++p) aq[(((int64_t)ks * 3 + p) * 4 + kb) * Rp + row] = planes[p];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int64_t so = ((((int64_t)(ks >> 2) * 2 + t) * 4 + kb) * Rp + row) * 4 + (ks & 3);
+    as[so] = (uint8_t)(t ? byte_lo : byte_hi);
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct MxArgs {
+  const void* aq;        // split activations (see the file comment)
+  const void* as;
+  const void* w;         // uint8 [N, K/2]
+  const void* s;         // uint8 [N, K/32]
+  void* y;               // [R, N]
+  int R, N, K, Rp;
+  int y_dtype;
+  int m_tiles, n_tiles;
+};
+
+// The two FP6 terms of a lane's 48 bytes (three 16-byte planes, hi | lo).
+__device__ __forceinline__ i32x8 fp6_term(const u32x4 (&p)[3], int term) {
+  if (term == 0) return i32x8{(int)p[0][0], (int)p[0][1], (int)p[0][2], (int)p[0][3], (int)p[1][0], (int)p[1][1], 0, 0};
+  return i32x8{(int)p[1][2], (int)p[1][3], (int)p[2][0], (int)p[2][1], (int)p[2][2], (int)p[2][3], 0, 0};
+}
+
+__device__ __forceinline__ i32x8 as_fp4_operand(u32x4 v) {
+  return i32x8{(int)v[0], (int)v[1], (int)v[2], (int)v[3], 0, 0, 0, 0};
+}
+
+__global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 31, kh = lane >> 5;       // operand row / column, 32-block within a 64-wide MFMA
+
+  // Workgroups are dealt to the 8 XCDs round-robin in launch order; XCD x is
+  // handed a contiguous run of tiles, row-tile fastest, so the workgroups that
+  // share one L2 share weight column tiles.
+  const int total = a.m_tiles * a.n_tiles;
+  const int per = (total + 7) / 8;
+  const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if (tile >= total) return;
+  const int m0 = (tile % a.m_tiles) * TM, n0 = (tile / a.m_tiles) * TN;
+
+  const int nquads = a.K / 512;
+  const int nq = nquads > wave ? (nquads - wave + 3) / 4 : 0;       // this wavefront's quads
+  const int last_step = 4 * nq - 1;
+  auto kstep_of = [&](int i) {                    // wave-local step -> K-step (clamped)
+    i = i < last_step ? i : last_step;
+    return 4 * (wave + 4 * (i >> 2)) + (i & 3);
+  };
+
+  const int64_t wpitch = a.K / 2, spitch = a.K / 32;
+  const auto rw = make_rsrc(a.w, (int64_t)a.N * wpitch);
+  const auto rs = make_rsrc(a.s, (int64_t)a.N * spitch);
+  const auto ra = make_rsrc(a.aq, (int64_t)(a.K / 128) * 192 * a.Rp);
+  const auto rsa = make_rsrc(a.as, (int64_t)nquads * 32 * a.Rp);
+
+  unsigned char* wbase = smem + wave * kWaveLds;
+  unsigned char* sbase = wbase + kStages * kStageBytes;
+
+  // loop-invariant lane offsets
+  uint32_t wvo[8];                                // weight codes: row 16j + lane/4, piece swizzled
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int n = n0 + 16 * j + (lane >> 2);
+    const int gp = (lane & 3) ^ ((lane >> 4) & 3);
+    wvo[j] = n < a.N ? (uint32_t)(n * wpitch + gp * 16) : kOutOfRange;
+  }
+  uint32_t svo[2];                                // weight scales: row 64h + lane
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int n = n0 + 64 * h + lane;
+    svo[h] = n < a.N ? (uint32_t)(n * spitch) : kOutOfRange;
+  }
+  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + li) * 16);      // + mt*512; block 2u+kh via the scalar offset
+  const uint32_t savo = (uint32_t)((kh * a.Rp + m0 + li) * 4);      // + mt*128
+  // codes of row r, block kb sit at r*64 + ((kb ^ ((r >> 2) & 3)) << 4)
+  const uint32_t rd_row = (uint32_t)(li * 64);
+  const uint32_t rd_swz = (uint32_t)((li >> 2) & 3);
+  const uint32_t rd_off[2] = {rd_row + (((0u + kh) ^ rd_swz) << 4), rd_row + (((2u + kh) ^ rd_swz) << 4)};
+  const uint32_t sh[2] = {(uint32_t)kh * 8, (uint32_t)kh * 8 + 16};  // this lane's scale byte within a K-step's dword
+
+  f32x16 acc[2][4];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
+
+  u32x4 areg[4][2][2][3];                         // [buffer][u][mt][plane]
+  uint32_t sa[2][2][2], sa_nxt[2][2][2];          // [u][mt][term]
+  u32x4 sbq[4];
+
+  // The 12 activation loads and 8 weight loads of a K-step are issued in four
+  // parts (g = 0..3) so they can be spread between the MFMAs of another step.
+  auto issue_a_part = [&](int ks, u32x4 (&dst)[2][2][3], int g) {
+#pragma unroll
+    for (int j = 3 * g; j < 3 * g + 3; ++j) {
+      const int p = j >> 2, u = (j >> 1) & 1, mt = j & 1;
+      const uint32_t so = (uint32_t)(((ks * 3 + p) * 4 + 2 * u) * 16) * (uint32_t)a.Rp;
+      dst[u][mt][p] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo + mt * 512, so, 0);
+    }
+  };
+  auto issue_a = [&](int ks, u32x4 (&dst)[2][2][3]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) issue_a_part(ks, dst, g);
+  };
+  auto issue_sa = [&](int quad, uint32_t (&dst)[2][2][2]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint32_t so = (uint32_t)(((quad * 2 + t) * 4 + 2 * u) * 4) * (uint32_t)a.Rp;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+          dst[u][mt][t] = __builtin_amdgcn_raw_buffer_load_b32(rsa, savo + mt * 128, so, 0);
+      }
+  };
+  auto dma_w_part = [&](int ks, int stage, int g) {
+#pragma unroll
+    for (int j = 2 * g; j < 2 * g + 2; ++j)
+      dma16(rw, wbase + stage * kStageBytes + j * 1024, wvo[j], (uint32_t)ks * 64);
+  };
+  auto dma_w = [&](int ks, int stage) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) dma_w_part(ks, stage, g);
+  };
+  auto dma_s = [&](int quad, int par) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      dma16(rs, sbase + par * kScaleBytes + h * 1024, svo[h], (uint32_t)quad * 16);
+  };
+  auto quad_of = [&](int qi) { return wave + 4 * (qi < nq - 1 ? qi : nq - 1); };
+
+  if (nq > 0) {
+    issue_sa(quad_of(0), sa);
+    dma_s(quad_of(0), 0);
+    issue_a(kstep_of(0), areg[0]);
+    dma_w(kstep_of(0), 0);
+    issue_a(kstep_of(1), areg[1]);
+    dma_w(kstep_of(1), 1);
+    dma_w(kstep_of(2), 2);
+    auto step = [&](int qi, auto tc) {
+      constexpr int t = decltype(tc)::value;
+      const int i = 4 * qi + t;
+      // Landed by now: everything but the loads issued during the previous
+      // step and the two weight loads that ended the step before it, i.e. this
+      // step's activation terms, codes and scales.
+      wait_vmcnt<(t == 1 ? 32 : 22)>();
+      const int ks_a = kstep_of(i + 2), ks_w = kstep_of(i + 3);
+
+      const unsigned char* st = wbase + t * kStageBytes;
+      if (t == 0) {
+        const unsigned char* sq = sbase + (qi & 1) * kScaleBytes + li * 16;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) sbq[nt] = *reinterpret_cast<const u32x4*>(sq + nt * 512);
+      }
+      i32x8 bf[2][4];
+      int sb[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+          bf[u][nt] = as_fp4_operand(*reinterpret_cast<const u32x4*>(st + rd_off[u] + nt * 2048));
+          sb[u][nt] = (int)(sbq[nt][t] >> sh[u]);
+        }
+      // Four groups of 8 MFMAs; after each, a quarter of the loads for later
+      // steps (activation terms two steps ahead, weight codes three steps
+      // ahead), so that load issue hides under the matrix-core work of this
+      // single wavefront per SIMD.  Loads retire in order: the activation part
+      // goes first in each quarter.
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int u = g >> 1, term = g & 1;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const i32x8 af = fp6_term(areg[t][u][mt], term);
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                af, bf[u][nt], acc[mt][nt], kFp6, kFp4, t, (int)sa[u][mt][term], 0, sb[u][nt]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a_part(ks_a, areg[(t + 2) & 3], g);
+        if (t == 0 && g == 0) issue_sa(quad_of(qi + 1), sa_nxt);
+        dma_w_part(ks_w, (t + 3) & 3, g);
+        if (t == 0 && g == 0) dma_s(quad_of(qi + 1), (qi + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (t == 3) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt) {
+            sa[u][mt][0] = sa_nxt[u][mt][0];
+            sa[u][mt][1] = sa_nxt[u][mt][1];
+          }
+      }
+    };
+    for (int qi = 0; qi < nq; ++qi) {
+      step(qi, std::integral_constant<int, 0>{});
+      step(qi, std::integral_constant<int, 1>{});
+      step(qi, std::integral_constant<int, 2>{});
+      step(qi, std::integral_constant<int, 3>{});
+    }
+  }
+  // every direct-to-LDS load (including the clamped repeats) must have landed
+  // before the staging area is reused for the reduction
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // ---- sum the four K-slices: red[wave][tile = mt*4+nt][r][lane]
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        red[(((wave * 8 + mt * 4 + nt) * 16) + r) * 64 + lane] = acc[mt][nt][r];
+  __syncthreads();
+  // wavefront w finishes tiles 2w and 2w+1 (row tile w/2, column tiles 2(w%2), +1)
+  const int mt = wave >> 1, nh = wave & 1;
+  float v[2][16];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) t += red[(((w * 8 + 2 * wave + h) * 16) + r) * 64 + lane];
+      v[h][r] = t;
+    }
+  const bool wide = a.y_dtype != QMM_F32 && (a.N & 7) == 0 &&
+                    (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;
+  if (wide) {
+    // 16-bit outputs: transpose this wavefront's 32 x 64 block through the LDS
+    // left over beside `red`, then store 16 bytes a lane (128 bytes a row)
+    uint16_t* o16 = reinterpret_cast<uint16_t*>(smem + 4 * 8 * 16 * 64 * 4) + wave * (32 * 64);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int rl = 8 * (r >> 2) + 4 * kh + (r & 3), cl = 32 * h + li;
+        o16[rl * 64 + cl] = (uint16_t)(a.y_dtype == QMM_BF16 ? f32_to_bf16_bits(v[h][r]) : f32_to_f16_bits(v[h][r]));
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int idx = q * 64 + lane, rl = idx >> 3, pc = idx & 7;
+      const int row = m0 + 32 * mt + rl, col = n0 + 64 * nh + pc * 8;
+      if (row < a.R && col < a.N)
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + (int64_t)row * a.N + col) =
+            *reinterpret_cast<const u32x4*>(o16 + rl * 64 + pc * 8);
+    }
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + 32 * mt + 8 * (r >> 2) + 4 * kh + (r & 3), col = n0 + 32 * (2 * nh + h) + li;
+        if (row < a.R && col < a.N) store_out(a.y, (int64_t)row * a.N + col, v[h][r], a.y_dtype);
+      }
+  }
+}
+
+}  // namespace
+
+// Rows of the split-activation workspace (row count rounded up to the tile).
+static int64_t mx_rows(int64_t R) { return ceil_div(R, TM) * TM; }
+
+bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K) {
+  if (getenv("QMM_NO_MXFP4_MFMA")) return false;
+  return K > 0 && K % 512 == 0 && N * (K / 2) < (1ll << 31) && mx_rows(R) * K * 3 / 2 < (1ll << 32) &&
+         mx_rows(R) * 4 * 8 < (1ll << 31);
+}
+
+size_t mxfp4_workspace_bytes(int64_t R, int64_t K) {
+  const int64_t rp = mx_rows(R);
+  return (size_t)(rp * K * 3 / 2 + (K / 512) * 32 * rp);
+}
+
+void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block) {
+  const int64_t tiles = ceil_div(R, TM) * ceil_div(N, TN);
+  *grid = (int)(ceil_div(tiles, 8) * 8);
+  *block = 256;
+}
+
+// x bf16 [R, K]; w uint8 [N, K/2]; s uint8 [N, K/32]; y [R, N]; workspace as sized above.
+void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, int y_dtype,
+                         int64_t R, int64_t N, int64_t K, void* workspace, hipStream_t st) {
+  const int64_t rp = mx_rows(R);
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  void* aq = ws;
+  void* as = ws + rp * K * 3 / 2;
+  const int64_t threads = rp * (K / 32);
+  hipLaunchKernelGGL(mx_split_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t*>(x), static_cast<u32x4*>(aq),
+                     static_cast<uint8_t*>(as), (int)R, (int)K, (int)rp);
+  MxArgs a;
+  a.aq = aq; a.as = as; a.w = w; a.s = s; a.y = y;
+  a.R = (int)R; a.N = (int)N; a.K = (int)K; a.Rp = (int)rp;
+  a.y_dtype = y_dtype;
+  a.m_tiles = (int)ceil_div(R, TM);
+  a.n_tiles = (int)ceil_div(N, TN);
+  int grid, block;
+  mxfp4_geometry(R, N, &grid, &block);
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mxfp4_mfma_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(mxfp4_mfma_kernel, dim3(grid), dim3(block), kLds, st, a);
+}
+
+}  // namespace qmm

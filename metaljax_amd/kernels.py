@@ -83,9 +83,12 @@ def quantized_matmul(x, w, scales, biases=None, transpose=True, group_size=64, b
     w, scales = w.contiguous(), scales.contiguous()
     biases = None if biases is None else biases.contiguous()
     tab = _dt(scales.dtype) if mode == "affine" else BF16
+    need = int(lib.qmm_workspace_bytes(batch, mrows, n, k, group_size, bits, _MODE[mode],
+                                       _dt(x2.dtype)))
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
     rc = lib.qmm_quantized_matmul(
         _ptr(x2), _dt(x2.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y), _dt(out_dtype),
-        batch, mrows, n, k, group_size, bits, _MODE[mode], None, 0, _stream(x))
+        batch, mrows, n, k, group_size, bits, _MODE[mode], _ptr(ws), need, _stream(x))
     _lib.check(rc)
     return y
 
@@ -230,11 +233,15 @@ class BoundQmm:
         for t in (x, w, scales, biases, y):
             if t is not None and not t.is_contiguous():
                 raise _lib.QmmError(1, "BoundQmm needs contiguous tensors")
-        self._keep = (x, w, scales, biases, y)
         self._lib = _lib.load()
         tab = _dt(scales.dtype) if mode == "affine" else BF16
+        need = int(self._lib.qmm_workspace_bytes(1, x.shape[0], n, k, group_size, bits,
+                                                 _MODE[mode], _dt(x.dtype)))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+        self._keep = (x, w, scales, biases, y, ws)
         self._args = (_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y),
-                      _dt(y.dtype), 1, x.shape[0], n, k, group_size, bits, _MODE[mode], None, 0)
+                      _dt(y.dtype), 1, x.shape[0], n, k, group_size, bits, _MODE[mode], _ptr(ws),
+                      need)
         self.y = y
 
     def launch(self, stream=None):

@@ -287,6 +287,92 @@ def test_gemm_mxfp4(m, n, k):
     assert O.rel_l2(y16, want) <= TOL_BF16_OUT
 
 
+@pytest.mark.parametrize("m,n,k", [(70, 200, 512), (64, 128, 2048), (300, 260, 1536), (33, 8, 1024)])
+def test_mxfp4_block_scaled_matrix_core_path(m, n, k):
+    """K % 512 == 0 and M > 16 runs on the block-scaled matrix cores: the weight
+    is exact there, the activations are split into two FP6 terms (about 3e-4
+    of |x| left over), so the float32 output must sit within 1e-3 of the oracle."""
+    from metaljax_amd import _lib
+    import ctypes
+    kern = ctypes.c_int()
+    assert _lib.load().qmm_plan(m, n, k, 32, 4, 1, kern, None, None) == 0
+    assert kern.value == _lib.KERNEL_MXFP4_MFMA
+    rng = np.random.default_rng(m * 7 + n)
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= TOL_F32_OUT, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4"))
+    assert O.rel_l2(y16, want) <= TOL_BF16_OUT
+
+
+def test_mxfp4_matrix_core_path_extreme_scales_and_zero_rows():
+    """E8M0 bytes over the whole legal range, an all-zero activation row and a
+    row of large magnitudes: no NaN/Inf, and the same tolerance row by row."""
+    rng = np.random.default_rng(99)
+    m, n, k = 40, 96, 512
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, lo=100, hi=150)
+    x, _ = make_x(rng, m, k)
+    x[3] = 0.0
+    x[5] = O.round_bf16(x[5] * 1.0e4)
+    x[7] = O.round_bf16(x[7] * 1.0e-6)
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                   out_dtype=torch.float32))
+    assert np.isfinite(y).all()
+    assert not y[3].any()
+    for r in (0, 5, 7, 39):
+        assert O.rel_l2(y[r], want[r]) <= TOL_F32_OUT, (r, O.rel_l2(y[r], want[r]))
+
+
+def test_mxfp4_matrix_core_path_batched():
+    rng = np.random.default_rng(5)
+    bsz, m, n, k = 3, 48, 72, 512
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(bsz,))
+    x = O.round_bf16(rng.standard_normal((bsz, m, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    y = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                   out_dtype=torch.float32))
+    for z in range(bsz):
+        want = O.qmm(x[z], words[z], sb[z], None, 32, 4, "mxfp4")
+        assert O.rel_l2(y[z], want) <= TOL_F32_OUT
+
+
+def test_mxfp4_missing_workspace_is_an_error():
+    from metaljax_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(1)
+    codes, words, sb, wd, sd = make_mxfp4(rng, 128, 512)
+    x, xd = make_x(rng, 64, 512)
+    y = torch.empty((64, 128), dtype=torch.bfloat16, device=DEV)
+    assert lib.qmm_workspace_bytes(1, 64, 128, 512, 32, 4, 1, _lib.BF16) > 0
+    rc = lib.qmm_quantized_matmul(xd.data_ptr(), _lib.BF16, wd.data_ptr(), sd.data_ptr(), None,
+                                  _lib.BF16, y.data_ptr(), _lib.BF16, 1, 64, 128, 512, 32, 4, 1,
+                                  None, 0, None)
+    assert rc == 4 and b"workspace" in lib.qmm_last_error()
+
+
+def test_c4_mxfp4_scaled_and_full_size():
+    wl = synth.make(4, scale=0.125)                      # N = 1024 rows of the same draw
+    x, w, s, b, _ = synth.to_device(wl)
+    want = C.qmm(wl.x, wl.w, wl.scales, None, 32, 4, "mxfp4", round_tile_bf16=False)
+    y32 = K.quantized_matmul(x, w, s, None, group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32)
+    assert O.rel_l2(out_f32(y32), want) <= TOL_F32_OUT, O.rel_l2(out_f32(y32), want)
+    # full size: against a float32 torch matmul on the device-dequantized (exact) weight
+    wl = synth.make(4)
+    x, w, s, b, _ = synth.to_device(wl)
+    y = K.quantized_matmul(x, w, s, None, group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32)
+    tile = K.dequantize(w, s, None, group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32)
+    ref = x.float() @ tile.T
+    rel = ((y - ref).norm() / ref.norm()).item()
+    assert rel <= TOL_F32_OUT, rel
+    yb = K.quantized_matmul(x, w, s, None, group_size=32, bits=4, mode="mxfp4")
+    assert ((yb.float() - ref).norm() / ref.norm()).item() <= TOL_BF16_OUT
+
+
 def test_c3_prefill_scaled_and_full_size_properties():
     wl = synth.make(3, scale=0.125, M=256)             # N = 512 rows of the same draw
     x, w, s, b, _ = synth.to_device(wl)
