@@ -115,15 +115,15 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
     const uint32_t tab_off = (uint32_t)((sl * CPS) >> GSHIFT) * 2;
     // ---- issue the global loads: the first tile (HBM, longest latency), the
     // activations (row blocks at or past M are not fetched), then the second tile
-    u32x4 wl[2][4], tv[2];
+    u32x4 wl[TMAX][4], tvs[TMAX], tvb[TMAX];
     // Table rows: lanes 0-15 fetch the 16 scale rows of a tile, lanes 16-31 the
     // bias rows (one 16-byte run each); they reach every lane through LDS.
     auto load_tables = [&](int t, int set) {
       const int64_t n = n_begin + t * 16 + r;
       const uint32_t to = (uint32_t)(n * ng * 2);
-      const u32x4 vs = __builtin_amdgcn_raw_buffer_load_b128(rs, lane < 16 && n < n_end ? to : kOutOfRange, tab_off, 0);
-      const u32x4 vb = __builtin_amdgcn_raw_buffer_load_b128(rb, (lane & 48) == 16 && n < n_end ? to : kOutOfRange, tab_off, 0);
-      tv[set] = vs | vb;                        // the lanes that miss read zeros
+      // (the two are merged where the tile is consumed, so that nothing waits here)
+      tvs[set] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane < 16 && n < n_end ? to : kOutOfRange, tab_off, 0);
+      tvb[set] = __builtin_amdgcn_raw_buffer_load_b128(rb, (lane & 48) == 16 && n < n_end ? to : kOutOfRange, tab_off, 0);
     };
     load_tile(wl[0], rw, n_begin, n_end, wpr, lrow, lpiece, slice_off);
     u32x4 xl[XR][4];
@@ -141,9 +141,12 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
       }
     }
     load_tables(0, 0);
-    if (TMAX > 1 && ntiles > 1) {
-      load_tile(wl[1], rw, n_begin + 16, n_end, wpr, lrow, lpiece, slice_off);
-      load_tables(1, 1);
+    // every other tile of the slice: all of this wavefront's weight bytes are in
+    // flight before the first one is consumed (tiles past the range read nothing)
+#pragma unroll
+    for (int t = 1; t < TMAX; ++t) {
+      load_tile(wl[t], rw, n_begin + t * 16, n_end, wpr, lrow, lpiece, slice_off);
+      load_tables(t, t);
     }
 
     // ---- activations: LDS round trip into operand layout, 128 codes a round
@@ -185,20 +188,15 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
       axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
     }
 
-    // ---- tiles: loads run two tiles ahead of the arithmetic
+    // ---- tiles
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
       if (t < ntiles) {
-        constexpr int kSetOf[4] = {0, 1, 0, 1};
-        const int set = kSetOf[t & 3];
+        const int set = t;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           *reinterpret_cast<u32x4*>(buf + st_off + i * 4 * kRowStride) = wl[set][i];
-        if (lane < 32) *reinterpret_cast<u32x4*>(tbuf + lane * 16) = tv[set];
-        if (t + 2 < TMAX && t + 2 < ntiles) {
-          load_tile(wl[set], rw, n_begin + (t + 2) * 16, n_end, wpr, lrow, lpiece, slice_off);
-          load_tables(t + 2, set);
-        }
+        if (lane < 32) *reinterpret_cast<u32x4*>(tbuf + lane * 16) = tvs[set] | tvb[set];   // the lanes that miss read zeros
         wave_lds_fence();
         // table rows as B operands over the chunk index (lane's row, entries of this slice)
         u32x4 svt = *reinterpret_cast<const u32x4*>(tbuf + r * 16);
