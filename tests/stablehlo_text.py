@@ -1,0 +1,271 @@
+"""Hand-written StableHLO modules in the shapes the reference's quantized test
+functions lower to (reference tests/test_qmm.py:179-234 `_unpack_nibbles`,
+`dense_sub`, `dense_perchannel`; tests/test_qmm_mxfp4.py:268-310
+`mxfp4_weight`, `dense_mxfp4`, `experts_mxfp4`), plus the seeded data
+generators of those tests restated with numpy alone.  jax is not available
+here, so the text is authored by hand: a nibble unpack out of and / shift /
+xor / concatenate, a `take` as a gather, a float subtract-and-scale, a dot.
+"""
+
+import numpy as np
+
+E2M1 = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
+
+
+def _t(shape, el):
+    return "tensor<" + "x".join([*map(str, shape), el]) + ">"
+
+
+def _unpack_nibbles(k, n):
+    """packed i8 [K, N/2] -> signed codes i8 [K, N]: lines defining %w."""
+    h = n // 2
+    a, b = _t((h, k), "i8"), _t((h, 1, k), "i8")
+    return f"""
+    %t = stablehlo.transpose %packed, dims = [1, 0] : ({_t((k, h), "i8")}) -> {a}
+    %c15 = stablehlo.constant dense<15> : tensor<i8>
+    %b15 = stablehlo.broadcast_in_dim %c15, dims = [] : (tensor<i8>) -> {a}
+    %c4 = stablehlo.constant dense<4> : tensor<i8>
+    %b4 = stablehlo.broadcast_in_dim %c4, dims = [] : (tensor<i8>) -> {a}
+    %c8 = stablehlo.constant dense<8> : tensor<i8>
+    %b8 = stablehlo.broadcast_in_dim %c8, dims = [] : (tensor<i8>) -> {a}
+    %low = stablehlo.and %t, %b15 : {a}
+    %sh = stablehlo.shift_right_arithmetic %t, %b4 : {a}
+    %high = stablehlo.and %sh, %b15 : {a}
+    %lx = stablehlo.xor %low, %b8 : {a}
+    %ls = stablehlo.subtract %lx, %b8 : {a}
+    %hx = stablehlo.xor %high, %b8 : {a}
+    %hs = stablehlo.subtract %hx, %b8 : {a}
+    %l3 = stablehlo.reshape %ls : ({a}) -> {b}
+    %h3 = stablehlo.reshape %hs : ({a}) -> {b}
+    %st = stablehlo.concatenate %l3, %h3, dim = 1 : ({b}, {b}) -> {_t((h, 2, k), "i8")}
+    %up = stablehlo.reshape %st : ({_t((h, 2, k), "i8")}) -> {_t((n, k), "i8")}
+    %cut = stablehlo.slice %up [0:{n}, 0:{k}] : ({_t((n, k), "i8")}) -> {_t((n, k), "i8")}
+    %w = stablehlo.transpose %cut, dims = [1, 0] : ({_t((n, k), "i8")}) -> {_t((k, n), "i8")}"""
+
+
+def _take_rows(name, table, ng, k, n, el):
+    """`jnp.take(table, g, axis=0)` with g [K] int32: negative indices wrap,
+    then a gather of whole rows."""
+    return f"""
+    %{name}_neg = stablehlo.compare LT, %g, %gz, SIGNED : ({_t((k,), "i32")}, {_t((k,), "i32")}) -> {_t((k,), "i1")}
+    %{name}_wrap = stablehlo.add %g, %gn : {_t((k,), "i32")}
+    %{name}_sel = stablehlo.select %{name}_neg, %{name}_wrap, %g : {_t((k,), "i1")}, {_t((k,), "i32")}
+    %{name}_idx = stablehlo.broadcast_in_dim %{name}_sel, dims = [0] : ({_t((k,), "i32")}) -> {_t((k, 1), "i32")}
+    %{name} = "stablehlo.gather"(%{table}, %{name}_idx) <{{dimension_numbers = #stablehlo.gather<offset_dims = [1], collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 1>, indices_are_sorted = false, slice_sizes = array<i64: 1, {n}>}}> : ({_t((ng, n), el)}, {_t((k, 1), "i32")}) -> {_t((k, n), el)}"""
+
+
+def dense_sub(k, n, ng, m, el="bf16", twice=False):
+    """x [M,K] @ ((unpack(packed) - zero[g]) * scale[g]); K rows, N columns.
+    `twice` adds a second consumer of the dequantized weight."""
+    out = _t((m, n), el)
+    extra, ret, res = "", "%y", out
+    if twice:
+        extra = f"""
+    %wsum = stablehlo.reduce(%wq init: %fz) applies stablehlo.add across dimensions = [0] : ({_t((k, n), el)}, tensor<{el}>) -> {_t((n,), el)}"""
+        ret, res = "%y, %wsum", f"({out}, {_t((n,), el)})"
+    return f"""
+module @jit_dense_sub {{
+  func.func public @main(%packed: {_t((k, n // 2), "i8")}, %scale: {_t((ng, n), el)}, %zero: {_t((ng, n), "i8")}, %gidx: {_t((k,), "f32")}, %x: {_t((m, k), el)}) -> {res} {{{_unpack_nibbles(k, n)}
+    %g = stablehlo.convert %gidx : ({_t((k,), "f32")}) -> {_t((k,), "i32")}
+    %gzs = stablehlo.constant dense<0> : tensor<i32>
+    %gz = stablehlo.broadcast_in_dim %gzs, dims = [] : (tensor<i32>) -> {_t((k,), "i32")}
+    %gns = stablehlo.constant dense<{ng}> : tensor<i32>
+    %gn = stablehlo.broadcast_in_dim %gns, dims = [] : (tensor<i32>) -> {_t((k,), "i32")}
+    %fz = stablehlo.constant dense<0.000000e+00> : tensor<{el}>{_take_rows("s", "scale", ng, k, n, el)}{_take_rows("z", "zero", ng, k, n, "i8")}
+    %wf = stablehlo.convert %w : ({_t((k, n), "i8")}) -> {_t((k, n), el)}
+    %zf = stablehlo.convert %z : ({_t((k, n), "i8")}) -> {_t((k, n), el)}
+    %d = stablehlo.subtract %wf, %zf : {_t((k, n), el)}
+    %wq = stablehlo.multiply %d, %s : {_t((k, n), el)}{extra}
+    %y = stablehlo.dot_general %x, %wq, contracting_dims = [1] x [0], precision = [DEFAULT, DEFAULT] : ({_t((m, k), el)}, {_t((k, n), el)}) -> {out}
+    return {ret} : {res.strip("()")}
+  }}
+}}
+"""
+
+
+def dense_i8_codes(k, n, ng, m, el="bf16"):
+    """dense_sub with the codes stored as plain i8 [K, N] (no nibble unpack)."""
+    text = dense_sub(k, n, ng, m, el)
+    head = text[:text.index("{", text.index("@main")) + 1].replace(_t((k, n // 2), "i8"), _t((k, n), "i8")).replace("%packed", "%w")
+    tail = text[text.index("    %g = stablehlo.convert %gidx"):]
+    return head + "\n" + tail
+
+
+def dense_int_sub(k, n, ng, m, el="bf16"):
+    """The same product with the zero point subtracted in INTEGER (i8)
+    arithmetic before the convert: the form that can wrap."""
+    return f"""
+func.func public @main(%packed: {_t((k, n // 2), "i8")}, %scale: {_t((ng, n), el)}, %zero: {_t((ng, n), "i8")}, %gidx: {_t((k,), "f32")}, %x: {_t((m, k), el)}) -> {_t((m, n), el)} {{{_unpack_nibbles(k, n)}
+  %g = stablehlo.convert %gidx : ({_t((k,), "f32")}) -> {_t((k,), "i32")}
+  %gzs = stablehlo.constant dense<0> : tensor<i32>
+  %gz = stablehlo.broadcast_in_dim %gzs, dims = [] : (tensor<i32>) -> {_t((k,), "i32")}
+  %gns = stablehlo.constant dense<{ng}> : tensor<i32>
+  %gn = stablehlo.broadcast_in_dim %gns, dims = [] : (tensor<i32>) -> {_t((k,), "i32")}{_take_rows("s", "scale", ng, k, n, el)}{_take_rows("z", "zero", ng, k, n, "i8")}
+  %di = stablehlo.subtract %w, %z : {_t((k, n), "i8")}
+  %d = stablehlo.convert %di : ({_t((k, n), "i8")}) -> {_t((k, n), el)}
+  %wq = stablehlo.multiply %d, %s : {_t((k, n), el)}
+  %y = stablehlo.dot_general %x, %wq, contracting_dims = [1] x [0] : ({_t((m, k), el)}, {_t((k, n), el)}) -> {_t((m, n), el)}
+  return %y : {_t((m, n), el)}
+}}
+"""
+
+
+def dense_perchannel(k, n, m, el="bf16"):
+    """(x @ convert(codes)) / scale[N]."""
+    return f"""
+func.func public @main(%packed: {_t((k, n // 2), "i8")}, %scale: {_t((n,), el)}, %x: {_t((m, k), el)}) -> {_t((m, n), el)} {{{_unpack_nibbles(k, n)}
+  %wf = stablehlo.convert %w : ({_t((k, n), "i8")}) -> {_t((k, n), el)}
+  %y0 = stablehlo.dot_general %x, %wf, contracting_dims = [1] x [0] : ({_t((m, k), el)}, {_t((k, n), el)}) -> {_t((m, n), el)}
+  %sb = stablehlo.broadcast_in_dim %scale, dims = [1] : ({_t((n,), el)}) -> {_t((m, n), el)}
+  %y = stablehlo.divide %y0, %sb : {_t((m, n), el)}
+  return %y : {_t((m, n), el)}
+}}
+"""
+
+
+def _e8m0_table_hex():
+    with np.errstate(over="ignore"):
+        t = np.ldexp(np.ones(256), np.arange(256) - 127).astype(np.float32)
+    t[255] = np.nan
+    return "0x" + t.tobytes().hex().upper()
+
+
+def _mxfp4_weight(lead, n, k, el, vtable=None):
+    """blocks ui8 [lead.., N, K/2] + E8M0 bytes [lead.., N, K/32] -> %wt [lead.., N, K]."""
+    L = tuple(lead)
+    vt = (list(E2M1) + [-v for v in E2M1]) if vtable is None else list(vtable)
+    vals = ", ".join(("-" if np.signbit(v) else "") + f"{abs(v):.6e}" for v in np.array(vt, np.float64))
+    cnt = int(np.prod(L + (n, k)))
+    sc = int(np.prod(L + (n, k // 32)))
+    bl, sb = _t(L + (n, k // 2), "ui8"), _t(L + (n, k // 32), "ui8")
+    r = len(L)
+    return f"""
+    %vt = stablehlo.constant dense<[{vals}]> : tensor<16x{el}>
+    %stab = stablehlo.constant dense<"{_e8m0_table_hex()}"> : tensor<256xf32>
+    %m15s = stablehlo.constant dense<15> : tensor<ui8>
+    %m15 = stablehlo.broadcast_in_dim %m15s, dims = [] : (tensor<ui8>) -> {bl}
+    %s4s = stablehlo.constant dense<4> : tensor<ui8>
+    %s4 = stablehlo.broadcast_in_dim %s4s, dims = [] : (tensor<ui8>) -> {bl}
+    %lo = stablehlo.and %blocks, %m15 : {bl}
+    %hi = stablehlo.shift_right_logical %blocks, %s4 : {bl}
+    %lo3 = stablehlo.reshape %lo : ({bl}) -> {_t(L + (n, k // 2, 1), "ui8")}
+    %hi3 = stablehlo.reshape %hi : ({bl}) -> {_t(L + (n, k // 2, 1), "ui8")}
+    %nb = stablehlo.concatenate %lo3, %hi3, dim = {r + 2} : ({_t(L + (n, k // 2, 1), "ui8")}, {_t(L + (n, k // 2, 1), "ui8")}) -> {_t(L + (n, k // 2, 2), "ui8")}
+    %nib = stablehlo.reshape %nb : ({_t(L + (n, k // 2, 2), "ui8")}) -> {_t((cnt, 1), "ui8")}
+    %ni = stablehlo.convert %nib : ({_t((cnt, 1), "ui8")}) -> {_t((cnt, 1), "i32")}
+    %vflat = "stablehlo.gather"(%vt, %ni) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 1>, slice_sizes = array<i64: 1>}}> : (tensor<16x{el}>, {_t((cnt, 1), "i32")}) -> {_t((cnt,), el)}
+    %sbi0 = stablehlo.reshape %scales : ({sb}) -> {_t((sc, 1), "ui8")}
+    %sbi = stablehlo.convert %sbi0 : ({_t((sc, 1), "ui8")}) -> {_t((sc, 1), "i32")}
+    %sflat = "stablehlo.gather"(%stab, %sbi) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 1>, slice_sizes = array<i64: 1>}}> : (tensor<256xf32>, {_t((sc, 1), "i32")}) -> {_t((sc,), "f32")}
+    %sc32 = stablehlo.reshape %sflat : ({_t((sc,), "f32")}) -> {_t(L + (n, k // 32), "f32")}
+    %scd = stablehlo.convert %sc32 : ({_t(L + (n, k // 32), "f32")}) -> {_t(L + (n, k // 32), el)}
+    %scb = stablehlo.broadcast_in_dim %scd, dims = [{", ".join(map(str, range(r + 2)))}] : ({_t(L + (n, k // 32), el)}) -> {_t(L + (n, k // 32, 32), el)}
+    %v3 = stablehlo.reshape %vflat : ({_t((cnt,), el)}) -> {_t(L + (n, k // 32, 32), el)}
+    %w3 = stablehlo.multiply %v3, %scb : {_t(L + (n, k // 32, 32), el)}
+    %wt = stablehlo.reshape %w3 : ({_t(L + (n, k // 32, 32), el)}) -> {_t(L + (n, k), el)}"""
+
+
+def dense_mxfp4(n, k, t, el="bf16", vtable=None):
+    """`th,nh->tn` over an in-graph MXFP4 reconstruction."""
+    return f"""
+module @jit_dense_mxfp4 {{
+  func.func public @main(%blocks: {_t((n, k // 2), "ui8")}, %scales: {_t((n, k // 32), "ui8")}, %x: {_t((t, k), el)}) -> {_t((t, n), el)} {{{_mxfp4_weight((), n, k, el, vtable)}
+    %y = stablehlo.dot_general %x, %wt, contracting_dims = [1] x [1] : ({_t((t, k), el)}, {_t((n, k), el)}) -> {_t((t, n), el)}
+    return %y : {_t((t, n), el)}
+  }}
+}}
+"""
+
+
+def experts_mxfp4(e, n, k, t, el="bf16"):
+    """`etm,ehm->eth`: one weight per expert, a BATCHED dot."""
+    return f"""
+func.func public @main(%blocks: {_t((e, n, k // 2), "ui8")}, %scales: {_t((e, n, k // 32), "ui8")}, %x: {_t((e, t, k), el)}) -> {_t((e, t, n), el)} {{{_mxfp4_weight((e,), n, k, el)}
+  %y = stablehlo.dot_general %x, %wt, batching_dims = [0] x [0], contracting_dims = [2] x [2] : ({_t((e, t, k), el)}, {_t((e, n, k), el)}) -> {_t((e, t, n), el)}
+  return %y : {_t((e, t, n), el)}
+}}
+"""
+
+
+def float_dot(k, n, m, el="bf16"):
+    """An ordinary float projection with a per-row scale: nothing to recognize."""
+    return f"""
+func.func public @main(%w: {_t((k, n), el)}, %r: {_t((k,), el)}, %x: {_t((m, k), el)}) -> {_t((m, n), el)} {{
+  %rb = stablehlo.broadcast_in_dim %r, dims = [0] : ({_t((k,), el)}) -> {_t((k, n), el)}
+  %ws = stablehlo.multiply %w, %rb : {_t((k, n), el)}
+  %y = stablehlo.dot_general %x, %ws, contracting_dims = [1] x [0] : ({_t((m, k), el)}, {_t((k, n), el)}) -> {_t((m, n), el)}
+  return %y : {_t((m, n), el)}
+}}
+"""
+
+
+def decode_loop(k, ng, m, steps, el="bf16"):
+    """A while loop whose weights arrive as carries returned unchanged (how jax
+    lowers a loop's closed-over constants); the body is one dense_sub with
+    N == K so the result feeds the next step."""
+    n = k
+    pk, sc, zr, gi, xx = (_t((k, n // 2), "i8"), _t((ng, n), el), _t((ng, n), "i8"),
+                          _t((k,), "f32"), _t((m, k), el))
+    body = dense_sub(k, n, ng, m, el)
+    lines = body[body.index("{", body.index("@main")) + 1:body.rindex("%y = stablehlo.dot_general")]
+    lines = (lines.replace("%packed", "%cp").replace("%scale,", "%cs,").replace("(%scale", "(%cs")
+             .replace("%zero,", "%cz,").replace("(%zero", "(%cz").replace("%gidx", "%cg"))
+    return f"""
+func.func public @main(%packed: {pk}, %scale: {sc}, %zero: {zr}, %gidx: {gi}, %x0: {xx}) -> {xx} {{
+  %i0 = stablehlo.constant dense<0> : tensor<i32>
+  %r:6 = stablehlo.while(%i = %i0, %cx = %x0, %cp = %packed, %cs = %scale, %cz = %zero, %cg = %gidx) : tensor<i32>, {xx}, {pk}, {sc}, {zr}, {gi}
+   cond {{
+    %lim = stablehlo.constant dense<{steps}> : tensor<i32>
+    %p = stablehlo.compare LT, %i, %lim, SIGNED : (tensor<i32>, tensor<i32>) -> tensor<i1>
+    stablehlo.return %p : tensor<i1>
+  }} do {{{lines}
+    %y = stablehlo.dot_general %cx, %wq, contracting_dims = [1] x [0] : ({xx}, {_t((k, n), el)}) -> {xx}
+    %one = stablehlo.constant dense<1> : tensor<i32>
+    %ni = stablehlo.add %i, %one : tensor<i32>
+    stablehlo.return %ni, %y, %cp, %cs, %cz, %cg : tensor<i32>, {xx}, {pk}, {sc}, {zr}, {gi}
+  }}
+  return %r#1 : {xx}
+}}
+"""
+
+
+# ------------------------------------------------------------ seeded data ----
+
+def bf16_round(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    r = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint32) << 16
+    return r.view(np.float32).reshape(np.shape(x))
+
+
+def quantize(rows, cols, block, seed=0, bits=4, g_idx=None, bf16=True):
+    """Codes + scale/zero maps in the keras storage layout: the generator of
+    reference tests/test_qmm.py:237-252 (same draws, same order)."""
+    rng = np.random.default_rng(seed)
+    lo, hi = -(1 << (bits - 1)), (1 << (bits - 1)) - 1
+    q = rng.integers(lo, hi + 1, size=(rows, cols)).astype(np.int8)
+    bsz = rows if block < 0 else block
+    ng = rows // bsz
+    scale = ((rng.random((ng, cols)).astype(np.float32) + 0.5) * 0.05)
+    zero = (np.zeros((ng, cols), np.int8) if block < 0 else
+            rng.integers(-3, 4, size=(ng, cols)).astype(np.int8))
+    if g_idx is None:
+        g_idx = (np.arange(rows) // bsz).astype(np.float32)
+    packed = ((q[:, 0::2] & 0x0F) | (q[:, 1::2] << 4)).astype(np.int8)
+    if bf16:
+        scale = bf16_round(scale)
+    gi = g_idx.astype(np.int32)
+    ref = scale[gi] * (q.astype(np.float32) - zero[gi].astype(np.float32))
+    return q, packed, scale, zero, g_idx, ref
+
+
+def random_mxfp4(shape_nk, seed=0, lo=117, hi=127):
+    """blocks ui8 [.., N, K/2], E8M0 bytes [.., N, K/32] and the exact float32
+    weight (reference tests/test_qmm_mxfp4.py:100-108)."""
+    rng = np.random.default_rng(seed)
+    *lead, n, k = shape_nk
+    codes = rng.integers(0, 16, size=(*lead, n, k), dtype=np.uint8)
+    blocks = (codes[..., 0::2] | (codes[..., 1::2] << 4)).astype(np.uint8)
+    sb = rng.integers(lo, hi + 1, size=(*lead, n, k // 32), dtype=np.uint8)
+    grid = np.array(list(E2M1) + [-v for v in E2M1], np.float32)
+    w = grid[codes] * np.repeat(np.ldexp(np.float32(1), sb.astype(np.int32) - 127), 32, axis=-1)
+    return codes, blocks, sb, w.astype(np.float32)

@@ -1,0 +1,152 @@
+"""Recognized programs executed for real: StableHLO text -> recognizer ->
+pack -> the HIP kernels through `emit`, against the literal interpretation of
+the same program and the exact float32 product (the comparison of reference
+tests/test_qmm.py:261-282: the fused result must be no worse than the literal
+chain, and within rtol 2e-2 / atol 1e-2*max of it)."""
+
+import numpy as np
+import pytest
+import torch
+
+import stablehlo_text as T
+from metaljax_amd import engine, interpreter as I, moe, qmm
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _fresh():
+    qmm.reset_stats()
+    moe.reset_stats()
+    qmm._BUILT.clear()
+    qmm._SHARED.clear()
+    yield
+
+
+def compare(text, args, exact, packs=1):
+    lit = I.Interpreter(text)
+    want = I.host(lit.run(args)[0]).a.astype(np.float32)
+    ex = engine.compile_program(text)
+    (y,) = engine.execute(ex, args)
+    assert isinstance(y, torch.Tensor) and y.is_cuda          # the fused op ran on the device
+    got = y.float().cpu().numpy()
+    assert qmm.stats()["packs"] == packs and qmm.stats()["fallbacks"] == 0
+    scale = np.abs(exact).max()
+    err_fused = np.abs(got - exact).max() / scale
+    err_lit = np.abs(want - exact).max() / scale
+    assert got.shape == want.shape
+    assert err_fused <= err_lit * 1.5 + 1e-6, (err_fused, err_lit)
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=1e-2 * scale)
+    return ex
+
+
+def dense_args(packed, scale, zero, g_idx, x):
+    return [I.from_numpy(packed), I.from_numpy(scale, "bf16"), I.from_numpy(zero),
+            I.from_numpy(g_idx), I.from_numpy(x, "bf16")]
+
+
+@pytest.mark.parametrize("m,block", [(4, 128), (1, 64), (40, 32), (16, -1)])
+def test_dense_subchannel(m, block):
+    k, n = 256, 128
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, block, seed=m)
+    x = T.bf16_round(np.random.default_rng(3).standard_normal((m, k)).astype(np.float32) * 0.5)
+    compare(T.dense_sub(k, n, scale.shape[0], m), dense_args(packed, scale, zero, g_idx, x), x @ wref)
+
+
+def test_dense_int8_codes():
+    k, n, m = 128, 64, 24
+    q, _, scale, zero, g_idx, wref = T.quantize(k, n, 64, seed=5, bits=8)
+    x = T.bf16_round(np.random.default_rng(3).standard_normal((m, k)).astype(np.float32) * 0.5)
+    compare(T.dense_i8_codes(k, n, 2, m), dense_args(q, scale, zero, g_idx, x), x @ wref)
+
+
+def test_perchannel():
+    k, n, m = 128, 64, 3
+    q, packed, _, _, _, _ = T.quantize(k, n, -1, seed=2)
+    scale = T.bf16_round(np.random.default_rng(9).uniform(8.0, 40.0, n).astype(np.float32))
+    x = T.bf16_round(np.random.default_rng(4).standard_normal((m, k)).astype(np.float32))
+    args = [I.from_numpy(packed), I.from_numpy(scale, "bf16"), I.from_numpy(x, "bf16")]
+    compare(T.dense_perchannel(k, n, m), args, (x @ q.astype(np.float32)) / scale)
+
+
+def test_interleaved_groups_run_through_the_permutation():
+    k, n, m, ng = 256, 64, 4, 2
+    g_idx = (np.arange(k) % ng).astype(np.float32)
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, k // ng, seed=11, g_idx=g_idx)
+    x = T.bf16_round(np.random.default_rng(3).standard_normal((m, k)).astype(np.float32))
+    compare(T.dense_sub(k, n, ng, m), dense_args(packed, scale, zero, g_idx, x), x @ wref)
+    assert qmm.stats()["perms"] == 1
+
+
+@pytest.mark.parametrize("t,k", [(5, 128), (40, 512)])
+def test_dense_mxfp4(t, k):
+    n = 48
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=1)
+    x = T.bf16_round(np.random.default_rng(2).standard_normal((t, k)).astype(np.float32))
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")]
+    compare(T.dense_mxfp4(n, k, t), args, x @ w.T)
+    assert qmm.stats()["mxfp4"] == 1
+
+
+def test_batched_experts_mxfp4():
+    e, n, k, t = 3, 32, 64, 4
+    codes, blocks, sb, w = T.random_mxfp4((e, n, k), seed=7)
+    x = T.bf16_round(np.random.default_rng(2).standard_normal((e, t, k)).astype(np.float32))
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")]
+    compare(T.experts_mxfp4(e, n, k, t), args, np.einsum("etk,enk->etn", x, w))
+    assert qmm.stats()["batched"] == 1
+
+
+def test_decode_loop_packs_once_across_steps_and_calls():
+    k, m, steps = 128, 2, 3
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, k, 64, seed=10)
+    scale = T.bf16_round(scale * 0.2)
+    wref = wref * 0.0 + scale[g_idx.astype(np.int32)] * (q.astype(np.float32) - zero[g_idx.astype(np.int32)])
+    x = T.bf16_round(np.random.default_rng(1).standard_normal((m, k)).astype(np.float32))
+    text = T.decode_loop(k, 2, m, steps)
+    args = dense_args(packed, scale, zero, g_idx, x)
+    want = I.host(I.Interpreter(text).run(args)[0]).a
+    ex = engine.compile_program(text)
+    for _ in range(2):
+        (y,) = engine.execute(ex, args)
+    got = I.host(y).a
+    assert qmm.stats()["packs"] == 1
+    np.testing.assert_allclose(got, want, rtol=4e-2, atol=2e-2 * np.abs(want).max())
+    # new weight buffers repack, and the result follows the new weights
+    args2 = dense_args(packed.copy(), T.bf16_round(scale * 0.5), zero, g_idx, x)
+    (y2,) = engine.execute(ex, args2)
+    want2 = I.host(I.Interpreter(text).run(args2)[0]).a
+    assert qmm.stats()["packs"] == 2
+    np.testing.assert_allclose(I.host(y2).a, want2, rtol=4e-2, atol=2e-2 * np.abs(want2).max())
+
+
+def test_gathered_expert_dispatch_over_a_recognized_pack():
+    """Top-2 routing over experts whose weights the recognizer packed: the
+    expert-indexed product + weighted sum against the dense reference
+    (reference tests/test_moe.py:514-557)."""
+    e, n, k, t, topk = 4, 64, 128, 12, 2
+    codes, blocks, sb, w = T.random_mxfp4((e, n, k), seed=21)
+    xe = T.bf16_round(np.random.default_rng(2).standard_normal((e, 1, k)).astype(np.float32))
+    ex = engine.compile_program(T.experts_mxfp4(e, n, k, 1))
+    st = qmm.analyze(ex.interp)
+    qmm.prologue(ex.interp, [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(xe, "bf16")])
+    mt = st.matches[0]
+    dot = moe.Dot(mt)
+    assert mt.absorbed
+    rng = np.random.default_rng(5)
+    x = T.bf16_round(rng.standard_normal((t, k)).astype(np.float32))
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    idx = np.argsort(-logits, axis=1)[:, :topk]
+    p = np.exp(logits - logits.max(1, keepdims=True))
+    p = p / p.sum(1, keepdims=True)
+    wts = np.take_along_axis(p, idx, 1)
+    xd = qmm.to_device(I.from_numpy(x, "bf16"))
+    y = moe.expert_dispatch(ex.interp, dot.match, xd, torch.from_numpy(idx).cuda(),
+                            torch.from_numpy(wts).cuda())
+    want = np.zeros((t, n), np.float32)
+    for i in range(t):
+        for j in range(topk):
+            want[i] += wts[i, j] * (x[i] @ w[idx[i, j]].T)
+    got = y.float().cpu().numpy()
+    assert moe.stats() == {"gather_qmm": 1, "dispatches": 1}
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-2
