@@ -12,6 +12,7 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
                    int y_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int gs, int bits,
                    int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st);
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
+void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
@@ -153,14 +154,24 @@ size_t qmm_gather_workspace_bytes(int64_t P, int64_t E) {
   return P <= kGatherGemvMaxPairs ? 0 : route_bytes(P, E);
 }
 
-int qmm_plan(int64_t M, int64_t N, int64_t K, int, int, int mode, int* kernel, int* grid,
-             int* block) {
+int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode, int* kernel,
+             int* grid, int* block) {
   if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K)) {
     int g, b;
     mxfp4_geometry(M, N, &g, &b);
     if (kernel) *kernel = QMM_KERNEL_MXFP4_MFMA;
     if (grid) *grid = g;
     if (block) *block = b;
+    return QMM_OK;
+  }
+  if (M <= kGemvMaxM && mode == QMM_MODE_AFFINE && (group_size == 64 || group_size == 128) &&
+      (bits == 4 || bits == 8) && K % (2048 / bits) == 0) {
+    // the staged decode kernel (bf16 tables assumed): contiguous row ranges
+    int waves, rows;
+    skinny_geometry(N, K, bits, &waves, &rows);
+    if (kernel) *kernel = QMM_KERNEL_GEMV;
+    if (grid) *grid = (int)ceil_div(N, rows);
+    if (block) *block = 64 * waves;
     return QMM_OK;
   }
   if (M <= kGemvMaxM) {
