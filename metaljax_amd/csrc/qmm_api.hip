@@ -18,6 +18,12 @@ void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, i
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
                    int64_t K, int gs, int bits, int mode, hipStream_t st);
 int64_t gemm_row_tile(int64_t R, int64_t E);
+bool gemm2_supported(int64_t R, int64_t N, int64_t K);
+size_t gemm2_workspace_bytes(int64_t R, int64_t K);
+void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
+                    const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
+                    int bits, int mode, int row_tile, void* workspace, hipStream_t st);
 bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K);
 size_t mxfp4_workspace_bytes(int64_t R, int64_t K);
 void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block);
@@ -147,6 +153,7 @@ const char* qmm_last_error(void) { return g_err; }
 size_t qmm_workspace_bytes(int64_t, int64_t M, int64_t N, int64_t K, int, int, int mode, int) {
   if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K))
     return mxfp4_workspace_bytes(M, K);
+  if (M > kGemvMaxM && gemm2_supported(M, N, K)) return gemm2_workspace_bytes(M, K);
   return 0;
 }
 
@@ -232,6 +239,26 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
     }
     return QMM_OK;
   }
+  if (gemm2_supported(M, N, K)) {
+    const size_t need = gemm2_workspace_bytes(M, K);
+    if (!workspace || workspace_bytes < need)
+      return fail(QMM_ERR_WORKSPACE, "the prefill kernel needs %zu workspace bytes, got %zu", need,
+                  workspace ? workspace_bytes : (size_t)0);
+    if (!aligned16(workspace) || !aligned16(scales))
+      return fail(QMM_ERR_BAD_ARGUMENT, "workspace / table pointer not 16-byte aligned");
+    const int bm = (int)gemm_row_tile(M, 1);
+    for (int64_t z = 0; z < batch; ++z) {
+      gemm2_dispatch(static_cast<const char*>(x) + z * M * K * 2,
+                     static_cast<const uint32_t*>(w) + z * N * wpr,
+                     static_cast<const char*>(scales) + z * N * ng * tabsz,
+                     biases ? static_cast<const char*>(biases) + z * N * ng * tabsz : nullptr,
+                     table_dtype, static_cast<char*>(y) + z * M * N * ysz, y_dtype, nullptr, nullptr,
+                     nullptr, M, 1, N, K, group_size, bits, mode, bm, workspace, st);
+      rc = check_launch("gemm launch");
+      if (rc) return rc;
+    }
+    return QMM_OK;
+  }
   for (int64_t z = 0; z < batch; ++z) {
     gemm_dispatch(static_cast<const char*>(x) + z * M * K * 2,
                   static_cast<const uint32_t*>(w) + z * N * wpr,
@@ -248,7 +275,8 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
 int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scales,
                     const void* biases, int table_dtype, void* y, int y_dtype,
                     const int32_t* row_offsets, int64_t R, int64_t E, int64_t N, int64_t K,
-                    int group_size, int bits, int mode, void*, size_t, void* stream) {
+                    int group_size, int bits, int mode, void* workspace, size_t workspace_bytes,
+                    void* stream) {
   if (R < 0 || E < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
   if (R == 0 || N == 0 || E == 0) return QMM_OK;
   if (!row_offsets) return fail(QMM_ERR_BAD_ARGUMENT, "null row_offsets");
@@ -258,6 +286,14 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   if (rc) return rc;
   if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535 || R * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  if (gemm2_supported(R, N, K) && workspace && workspace_bytes >= gemm2_workspace_bytes(R, K) &&
+      aligned16(workspace)) {
+    gemm2_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
+                   E, N, K, group_size, bits, mode, (int)gemm_row_tile(R, E), workspace,
+                   static_cast<hipStream_t>(stream));
+    return check_launch("grouped gemm launch");
+  }
+  // without a workspace the grouped product runs on the LDS-staged kernel
   gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
                 R, E, N, K, group_size, bits, mode, static_cast<hipStream_t>(stream));
   return check_launch("grouped gemm launch");

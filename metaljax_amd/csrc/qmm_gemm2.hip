@@ -1,0 +1,504 @@
+// Prefill-regime quantized matmul (M > 16) and the grouped (per-expert) form
+// for gfx950, second generation: activations reach the matrix cores straight
+// from global memory, only the dequantized weight tile goes through LDS.
+//
+// Why.  With both operand tiles in LDS a 256 x 128 x 64 step moves 144 KB
+// through LDS (48 KB of writes, 96 KB of fragment reads) for 1024 clocks of
+// v_mfma_f32_32x32x16_bf16 work per SIMD: more than the 128 B/clk the LDS can
+// deliver, so the matrix cores wait.  The activation fragments have no reuse
+// inside a wavefront row block, so they do not need LDS at all, provided a
+// lane's 16 bytes (row i, 8 consecutive k) can be fetched coalesced.  A short
+// pre-pass therefore re-lays x once per call:
+//     ax[k/8][row]   16 bytes each (8 consecutive k of one row), rows contiguous
+// so the lanes of a fragment load (32 rows x 2 k-halves) read two 512-byte
+// runs, for any first row (grouped tiles start at arbitrary rows).  The row
+// gather of the expert-sorted form (lhs_idx) is folded into the same pass.
+//
+// Main kernel.  Workgroup tile BM x 128, BK = 64, four wavefronts stacked in M
+// (each (BM/4) x 128: MT x 4 MFMA tiles of 32 x 32).  Per K-tile:
+//   * every thread loads 32 packed codes of one weight row (row tid/2, k-half
+//     tid%2), dequantizes them with the row's scale/bias of that 32-group
+//     (float32 fma, one round-to-nearest-even to bf16: the reference's tile
+//     semantics, bit for bit) and writes four 16-byte pieces of the bf16 tile
+//     to LDS (piece p of row r at p ^ (r & 7));
+//   * every wavefront reads the whole weight tile back as B fragments and
+//     multiplies it with its own activation fragments (registers).
+// Schedule: the packed words of tile t+4 (they come from HBM and are consumed
+// three K-tiles later) and the activation fragments of tile t+2 (from L2) are
+// loaded while tile t is multiplied; tile t+1 is dequantized between the MFMAs
+// of tile t; three LDS stages, one LDS-only barrier per K-tile.
+#include <type_traits>
+
+#include "qmm_common.hpp"
+
+namespace qmm {
+
+namespace {
+
+constexpr int BN = 128, BK = 64;
+constexpr int kRowBytes = BK * 2;                 // bf16 tile row
+constexpr int kStage = BN * kRowBytes;            // 16 KB
+constexpr int kStages = 3;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
+  const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
+}
+
+__device__ __forceinline__ void lds_barrier() {   // orders LDS traffic only; global loads stay in flight
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__device__ __forceinline__ int swz(int row, int piece) { return row * kRowBytes + ((piece ^ (row & 7)) << 4); }
+
+// ---------------------------------------------------------------------------
+// x [x_rows, K] bf16 (rows optionally gathered through lhs_idx) -> ax[K/8][Rp]
+// One thread = one row's 64 bytes (4 pieces); consecutive threads = consecutive rows.
+__global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* __restrict__ x,
+                                                        const int32_t* __restrict__ lhs_idx,
+                                                        u32x4* __restrict__ ax, int R, int K, int Rp) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int row = (int)(idx % Rp);
+  const int chunk = (int)(idx / Rp);               // 32 elements = 4 pieces
+  if (chunk >= K / 32 || row >= R) return;
+  const int64_t src = lhs_idx ? (int64_t)lhs_idx[row] : (int64_t)row;
+  const u32x4* p = reinterpret_cast<const u32x4*>(x + src * K + chunk * 32);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ax[((int64_t)chunk * 4 + j) * Rp + row] = p[j];
+}
+
+// ---------------------------------------------------------------------------
+struct Gemm2Args {
+  const void* ax;        // re-laid activations
+  const uint32_t* w;     // [E, N, K*bits/32]
+  const void* s;         // [E, N, K/gs]
+  const void* b;
+  void* y;               // [R, N]
+  const int32_t* row_offsets;   // [E+1] or null
+  const int32_t* out_idx;       // optional row scatter for y
+  int R, N, K, E, Rp;
+  int gs, tab, y_dtype;
+  int m_tiles;
+  int tabfast;           // table rows are dword-aligned: fetch them as 16-byte windows
+};
+
+// 32 codes (one row, one 32-group) -> four 16-byte pieces of bf16 weights
+template <int MODE, int BITS>
+__device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float sc, float bi) {
+  float f[8];
+  if constexpr (MODE == 1) {
+    // exact: the converter widens the two codes of a byte and applies the power-of-two scale
+    const uint32_t w = q[pc];
+    return u32x4{__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 0)),
+                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 1)),
+                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 2)),
+                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 3))};
+  } else if constexpr (BITS == 8) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t w = q[2 * pc + h];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[4 * h + j] = fmaf(sc, (float)((w >> (8 * j)) & 255u), bi);
+    }
+  } else {
+    const uint32_t w = q[pc];
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;     // even / odd codes as bytes
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = fmaf(sc, (float)((lo >> (8 * j)) & 255u), bi);
+      f[2 * j + 1] = fmaf(sc, (float)((hi >> (8 * j)) & 255u), bi);
+    }
+  }
+  return u32x4{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+               pack_bf16x2(f[6], f[7])};
+}
+
+// MT x NT MFMA tiles (32 x 32) per wavefront; WMW wavefronts stacked in M and
+// 4 / WMW side by side in N, which always spans the 128 weight rows of a tile:
+//   MT=2 NT=4 WMW=4: 256 x 128 workgroup tile (every wavefront reads the whole
+//                    weight tile, activations are private);
+//   MT=2 NT=2 WMW=2: 128 x 128 (for short row groups: half the LDS reads a
+//                    wavefront, the two wavefronts of a row block fetch the
+//                    same activation fragments).
+// NWAVES = 8 puts two wavefronts on every SIMD (one's vector ALU and load issue
+// fill the other's MFMA shadow) at half the work each.
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
+  constexpr int WNW = NWAVES / WMW;
+  static_assert(WNW * NT * 32 == BN, "the wavefronts must span the weight tile");
+  constexpr int WM = MT * 32;                      // rows per wavefront
+  constexpr int BM = WMW * WM;                     // rows per workgroup
+  constexpr int WBITS = (MODE == 1) ? 4 : BITS;
+  constexpr int TPR = NWAVES / 2;                  // threads per weight row: 2 | 4
+  constexpr int CPT = BK / TPR;                    // codes per thread per K-tile: 32 | 16
+  constexpr int PPT = CPT / 8;                     // 16-byte bf16 pieces per thread: 4 | 2
+  constexpr int WPT = CPT * WBITS / 32;            // packed words per thread per K-tile
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WNW, wn = wave % WNW;
+  const int li = lane & 31, kh = lane >> 5;
+
+  // ---- which tile?  XCD x (workgroups are dealt round-robin) gets a
+  // contiguous run of tiles, column tile fastest, so the workgroups sharing an
+  // L2 share activation row blocks.
+  const int n_tiles = (a.N + BN - 1) / BN;
+  const int total = n_tiles * a.m_tiles;
+  const int per = (total + 7) / 8;
+  const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if (tile >= total) return;
+  const int tile_n = tile % n_tiles, tile_m = tile / n_tiles;
+  int e = 0, row_lo = 0, row_hi = a.R, mt_idx = tile_m;
+  if (a.row_offsets) {
+    int t = tile_m;
+    bool found = false;
+    for (int i = 0; i < a.E; ++i) {
+      const int lo = a.row_offsets[i], hi = a.row_offsets[i + 1];
+      const int tiles = (hi - lo + BM - 1) / BM;
+      if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
+      t -= tiles;
+    }
+    if (!found) return;
+  }
+  const int m0 = row_lo + mt_idx * BM;
+  if (m0 >= row_hi) return;
+  const int n0 = tile_n * BN;
+
+  const int64_t wpr = (int64_t)a.K * WBITS / 32;
+  const int gs = (MODE == 1) ? 32 : a.gs;
+  const int64_t ng = a.K / gs;
+  const int tabsz = (MODE == 1) ? 1 : (a.tab == QMM_F32 ? 4 : 2);
+  const uint32_t* wb = a.w + (int64_t)e * a.N * wpr;
+  const char* sb = static_cast<const char*>(a.s) + (int64_t)e * a.N * ng * tabsz;
+  const char* bb = (MODE == 1) ? nullptr : static_cast<const char*>(a.b) + (int64_t)e * a.N * ng * tabsz;
+
+  // ---- activation fragments: lane (row li, k-half kh) of row tile i, k-step ks
+  // reads ax[(kt*8 + ks*2 + kh) * Rp + m0 + wm*WM + i*32 + li]
+  const auto ra = make_rsrc(a.ax, (int64_t)(a.K / 8) * a.Rp * 16);
+  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * WM + li) * 16);
+  typedef u32x4 AFrag[4][MT];
+  auto load_a_part = [&](int kt, AFrag& dst, int ks) {       // the fragments of one k-step
+    const uint32_t so = (uint32_t)((kt * 8 + ks * 2) * 16) * (uint32_t)a.Rp;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      dst[ks][i] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo + i * 512, so, 0);
+  };
+  auto load_a = [&](int kt, AFrag& dst) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) load_a_part(kt, dst, ks);
+  };
+
+  // ---- weight staging: thread -> (row tid/TPR, k-part tid%TPR): CPT codes a K-tile
+  const int wrow = tid / TPR, whalf = tid % TPR;
+  int64_t wn_row = n0 + wrow;
+  if (wn_row >= a.N) wn_row = a.N - 1;             // rows past N are computed and never stored
+  const auto rw = make_rsrc(wb, (int64_t)a.N * wpr * 4);
+  const uint32_t wvo = (uint32_t)((wn_row * wpr + whalf * WPT) * 4);
+  const int64_t trow = wn_row * ng;
+  struct WRegs { uint32_t q[WPT]; };
+  auto load_w = [&](int kt, WRegs& r) {
+    const uint32_t so = (uint32_t)kt * (BK * WBITS / 8);
+    if constexpr (WPT == 2) {
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rw, wvo, so, 0);
+      r.q[0] = v[0]; r.q[1] = v[1];
+    } else {
+#pragma unroll
+      for (int j = 0; j < WPT; j += 4) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rw, wvo + j * 4, so, 0);
+        r.q[j] = v[0]; r.q[j + 1] = v[1]; r.q[j + 2] = v[2]; r.q[j + 3] = v[3];
+      }
+    }
+  };
+
+  // ---- scale / bias entries.  A window = the entries of four K-tiles of this
+  // thread's row (32 bytes a table, fetched once per four K-tiles); the entry
+  // of K-tile t' = kt & 3 is picked out of it with per-thread constants.
+  struct TabWin { u32x4 s[2], b[2]; };
+  const auto rs = make_rsrc(sb, (int64_t)a.N * ng * tabsz);
+  const auto rb = make_rsrc(MODE == 1 ? sb : bb, (int64_t)a.N * ng * tabsz);
+  const uint32_t tvo = (uint32_t)(trow * tabsz);
+  const int gshift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+  auto load_win = [&](int quad, TabWin& tw) {
+    const uint32_t so = (uint32_t)(((quad * 4 * BK) >> gshift) * tabsz);
+    tw.s[0] = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo, so, 0);
+    if (tabsz == 4) tw.s[1] = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo + 16, so, 0);
+    if constexpr (MODE == 0) {
+      tw.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo, so, 0);
+      if (tabsz == 4) tw.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo + 16, so, 0);
+    }
+  };
+  // entry index of K-tile t' inside its window, for this thread's k-half
+  uint32_t eidx[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) eidx[t] = (uint32_t)((t * BK + whalf * CPT) >> gshift);
+  auto pick = [&](const u32x4 (&w)[2], uint32_t e) -> float {
+    // entry e (0..7) of a window of 1-, 2- or 4-byte entries
+    const uint32_t byte = e * (uint32_t)tabsz;
+    const uint32_t d = byte >> 2;
+    uint32_t v = w[0][0];
+    v = d == 1 ? w[0][1] : v;
+    v = d == 2 ? w[0][2] : v;
+    v = d == 3 ? w[0][3] : v;
+    if (tabsz == 4) {
+      v = d == 4 ? w[1][0] : v;
+      v = d == 5 ? w[1][1] : v;
+      v = d == 6 ? w[1][2] : v;
+      v = d == 7 ? w[1][3] : v;
+      return __uint_as_float(v);
+    }
+    v >>= (byte & 3u) * 8u;
+    if constexpr (MODE == 1) return e8m0_to_f32(v & 255u);
+    return a.tab == QMM_BF16 ? bf16_bits_to_f32(v & 0xFFFFu) : f16_bits_to_f32(v & 0xFFFFu);
+  };
+  // (scale, bias) of K-tile kt for this thread
+  auto entry = [&](int kt, const TabWin& tw, float& sc, float& bi) {
+    if (a.tabfast) {
+      sc = pick(tw.s, eidx[kt & 3]);
+      bi = MODE == 1 ? 0.f : pick(tw.b, eidx[kt & 3]);
+    } else {
+      const int64_t ti = trow + ((kt * BK + whalf * CPT) >> gshift);
+      if constexpr (MODE == 1) {
+        sc = e8m0_to_f32(reinterpret_cast<const uint8_t*>(sb)[ti]);
+        bi = 0.f;
+      } else {
+        sc = load_table_rt(sb, ti, a.tab);
+        bi = load_table_rt(bb, ti, a.tab);
+      }
+    }
+  };
+  auto store_piece = [&](int stage, const WRegs& r, int pc, float sc, float bi) {
+    *reinterpret_cast<u32x4*>(smem + stage * kStage + swz(wrow, whalf * PPT + pc)) =
+        dequant_piece<MODE, BITS>(r.q, pc, sc, bi);
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int KT = a.K / BK;
+  AFrag af[4];                                    // K-tile t lives in af[t & 3]
+  WRegs wr[4];                                    // words of K-tile t live in wr[t & 3]
+  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
+
+  // prologue: tile 0 dequantized, tiles 0..1 of the activations and the words
+  // of tile 1 in flight
+  TabWin tw_cur, tw_nxt;
+  if (a.tabfast) load_win(0, tw_cur);
+  load_w(0, wr[0]);
+  load_a(0, af[0]);
+  load_w(clampk(1), wr[1]);
+  load_a(clampk(1), af[1]);
+  load_w(clampk(2), wr[2]);
+  load_w(clampk(3), wr[3]);
+  {
+    float sc, bi;
+    entry(0, tw_cur, sc, bi);
+#pragma unroll
+    for (int pc = 0; pc < PPT; ++pc) store_piece(0, wr[0], pc, sc, bi);
+  }
+  lds_barrier();
+
+  bf16x8 fb[2][NT];                               // B fragments: k-step ks in set ks & 1
+  auto read_b = [&](const unsigned char* pbase, int ks, int set) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      fb[set][j] = *reinterpret_cast<const bf16x8*>(pbase + swz(wn * (NT * 32) + j * 32 + li, ks * 2 + kh));
+  };
+  read_b(smem, 0, 0);
+
+  // One K-tile.  A single wavefront per SIMD has to keep its matrix core busy
+  // by itself, and both a vector-memory instruction (about 64 clocks to issue
+  // 1 KB) and a run of vector ALU work stall the next MFMA if they sit in one
+  // lump; so each k-step's eight MFMAs are interleaved, instruction by
+  // instruction, with a quarter of everything else the tile needs: the loads
+  // of tile kt+2, one piece of tile kt+1's dequantization, the fragment reads
+  // of the next k-step.
+  auto step = [&](int kt, auto tc) {
+    constexpr int t = decltype(tc)::value;         // kt & 3
+    const unsigned char* pb = smem + (kt % kStages) * kStage;
+    const int nstage = (kt + 1) % kStages;
+    const bool has_next = kt + 1 < KT;             // uniform
+    const int kt2 = clampk(kt + 2), kt4 = clampk(kt + 4);
+    float sc, bi;                                  // of tile kt+1 (the first tile of the next quad at t == 3)
+    entry(kt + 1, t == 3 ? tw_nxt : tw_cur, sc, bi);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1);
+      load_a_part(kt2, af[(t + 2) & 3], ks);
+      if (ks == 0) load_w(kt4, wr[t & 3]);          // three K-tiles ahead of its dequantization
+      if (ks == 1 && t == 0 && a.tabfast) {        // next quad's table window (clamped at the end)
+        const int q = (kt >> 2) + 1;
+        load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][i]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[i][j], 0, 0, 0);
+      }
+      // (after the last tile this writes a stage nobody reads: cheaper than a branch,
+      // which would split the scheduling region)
+      if (PPT == 4 || (ks & 1) == 0) store_piece(nstage, wr[(t + 1) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
+      // order inside the k-step: fragment reads first, then MFMA / ALU / load slots
+      __builtin_amdgcn_sched_group_barrier(0x100, NT, 0);      // ds reads
+#pragma unroll
+      for (int m = 0; m < MT * NT; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 32 / (MT * NT), 0);   // a few vector ALU instructions
+        if (m < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one vector-memory load
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (t == 3) tw_cur = tw_nxt;
+    lds_barrier();
+    if (has_next) read_b(smem + nstage * kStage, 0, 0);
+  };
+  int kt = 0;
+  for (; kt + 4 <= KT; kt += 4) {
+    step(kt, std::integral_constant<int, 0>{});
+    step(kt + 1, std::integral_constant<int, 1>{});
+    step(kt + 2, std::integral_constant<int, 2>{});
+    step(kt + 3, std::integral_constant<int, 3>{});
+  }
+  if (kt < KT) { step(kt, std::integral_constant<int, 0>{}); ++kt; }
+  if (kt < KT) { step(kt, std::integral_constant<int, 1>{}); ++kt; }
+  if (kt < KT) { step(kt, std::integral_constant<int, 2>{}); ++kt; }
+
+  // ---- epilogue.  D[i][j] of a 32x32 tile: lane holds column lane % 32 and
+  // rows (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5), r = 0..15.
+  const bool wide = a.y_dtype != QMM_F32 && (a.N & 7) == 0 &&
+                    (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;
+  if (wide) {
+    // 16-bit outputs: transpose each 32 x (NT*32) block through this wavefront's
+    // share of LDS (free after the last barrier), store 16 bytes a lane
+    constexpr int WC = NT * 32;                    // columns per wavefront
+    uint16_t* o16 = reinterpret_cast<uint16_t*>(smem) + wave * (32 * WC);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rl = (r & 3) + 8 * (r >> 2) + 4 * kh;
+          const float v = acc[i][j][r];
+          o16[rl * WC + j * 32 + li] =
+              (uint16_t)(a.y_dtype == QMM_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+        }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int q = 0; q < WC / 16; ++q) {          // 32 rows x WC/8 pieces over 64 lanes
+        const int idx = q * 64 + lane, rl = idx / (WC / 8), pc = idx % (WC / 8);
+        const int m = m0 + wm * WM + i * 32 + rl, n = n0 + wn * WC + pc * 8;
+        if (m < row_hi && n < a.N) {
+          const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
+          *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + n) =
+              *reinterpret_cast<const u32x4*>(o16 + rl * WC + pc * 8);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int n = n0 + wn * (NT * 32) + j * 32 + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * WM + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          if (m < row_hi && n < a.N) {
+            const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
+            store_out(a.y, orow * a.N + n, acc[i][j][r], a.y_dtype);
+          }
+        }
+      }
+  }
+}
+
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
+void launch2(const Gemm2Args& a0, hipStream_t st) {
+  constexpr int BM = WMW * MT * 32;
+  Gemm2Args a = a0;
+  a.m_tiles = (int)(a.row_offsets ? ceil_div(a.R, BM) + a.E : ceil_div(a.R, BM));
+  const int64_t total = ceil_div(a.N, BN) * a.m_tiles;
+  dim3 grid((unsigned)(ceil_div(total, 8) * 8));
+  const size_t lds = kStages * kStage;            // 48 KB (the epilogue reuses 32 KB of it)
+  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES>;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(64 * NWAVES), lds, st, a);
+}
+
+template <int MODE, int BITS>
+void launch2_mt(const Gemm2Args& a, int mt, hipStream_t st) {
+  static const int variant = getenv("QMM_G2_VARIANT") ? atoi(getenv("QMM_G2_VARIANT")) : 0;
+  if (mt == 2) {
+    if (variant == 1) launch2<MODE, BITS, 2, 2, 4, 8>(a, st);      // 256 x 128, eight wavefronts
+    else launch2<MODE, BITS, 2, 4, 4, 4>(a, st);                   // 256 x 128, four wavefronts
+  } else {
+    if (variant == 2) launch2<MODE, BITS, 2, 2, 2, 4>(a, st);      // 128 x 128, four wavefronts
+    else launch2<MODE, BITS, 1, 2, 4, 8>(a, st);                   // 128 x 128, eight wavefronts
+  }
+}
+
+int64_t prep_rows(int64_t R) { return ceil_div(R + 256, 64) * 64; }   // a tile may start at any row
+
+}  // namespace
+
+bool gemm2_supported(int64_t R, int64_t N, int64_t K) {
+  if (getenv("QMM_GEMM_V1")) return false;
+  return K > 0 && K % 64 == 0 && prep_rows(R) * K * 2 < (1ll << 32) && N * K < (1ll << 31);
+}
+
+size_t gemm2_workspace_bytes(int64_t R, int64_t K) { return (size_t)(prep_rows(R) * K * 2); }
+
+// x bf16 [x_rows, K] (rows gathered through lhs_idx when given); the rest as gemm_dispatch.
+void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
+                    const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
+                    int bits, int mode, int row_tile, void* workspace, hipStream_t st) {
+  if (R == 0 || N == 0) return;
+  const int64_t rp = prep_rows(R);
+  const int64_t threads = rp * (K / 32);
+  hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t*>(x), lhs_idx, static_cast<u32x4*>(workspace),
+                     (int)R, (int)K, (int)rp);
+  Gemm2Args a;
+  a.ax = workspace;
+  a.w = static_cast<const uint32_t*>(w);
+  a.s = s;
+  a.b = b;
+  a.y = y;
+  a.row_offsets = row_offsets;
+  a.out_idx = out_idx;
+  a.R = (int)R; a.N = (int)N; a.K = (int)K; a.E = (int)E; a.Rp = (int)rp;
+  a.gs = gs; a.tab = tab; a.y_dtype = y_dtype;
+  a.m_tiles = 0;
+  {
+    const int esz = mode == QMM_MODE_MXFP4 ? 1 : (tab == QMM_F32 ? 4 : 2);
+    const int g = mode == QMM_MODE_MXFP4 ? 32 : gs;
+    const bool aligned = ((K / g) * esz) % 4 == 0 && (reinterpret_cast<uintptr_t>(s) & 3u) == 0 &&
+                         (mode == QMM_MODE_MXFP4 || (reinterpret_cast<uintptr_t>(b) & 3u) == 0);
+    a.tabfast = aligned && K % 256 == 0 && N * (K / g) * esz < (1ll << 31) && !getenv("QMM_G2_NOTABFAST");
+  }
+  const int mt = row_tile >= 256 ? 2 : 1;
+  if (mode == QMM_MODE_MXFP4) launch2_mt<1, 4>(a, mt, st);
+  else if (bits == 4) launch2_mt<0, 4>(a, mt, st);
+  else launch2_mt<0, 8>(a, mt, st);
+}
+
+}  // namespace qmm

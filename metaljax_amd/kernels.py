@@ -108,9 +108,11 @@ def grouped_qmm(x, w, scales, biases, row_offsets, group_size=64, bits=4, mode="
     biases = None if biases is None else biases.contiguous()
     ro = row_offsets.to(torch.int32).contiguous()
     tab = _dt(scales.dtype) if mode == "affine" else BF16
+    need = int(lib.qmm_workspace_bytes(1, r, n, k, group_size, bits, _MODE[mode], _dt(x.dtype)))
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
     rc = lib.qmm_grouped_qmm(_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab,
                              _ptr(y), _dt(out_dtype), _ptr(ro), r, e, n, k, group_size, bits,
-                             _MODE[mode], None, 0, _stream(x))
+                             _MODE[mode], _ptr(ws), need, _stream(x))
     _lib.check(rc)
     return y
 
