@@ -137,6 +137,22 @@ def cpu_baseline(wl, budget_s=4.0):
                       f"{sec * 1e3:.1f} ms per pass, unpack + dequantize to a bf16 tile + f32-accumulate dot"}
 
 
+def committed_traffic():
+    """HBM bytes per launch of the decode kernel on C2, as measured by the
+    FETCH_SIZE / WRITE_SIZE counter runs whose summary is committed under
+    profiles/ (a counter run cannot happen inside this program); None when
+    that summary is absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                        "decode_qmm_C2_int4_g64_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +160,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-extra", action="store_true", help="skip the other named shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--m16-only", action="store_true", help="run the headline decode leg only")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a 64 MiB read + 64 MiB write elementwise kernel five times, "
+                         "for scaling FETCH_SIZE / WRITE_SIZE counter readings")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU; --gpus {args.gpus} is not supported "
@@ -155,6 +175,12 @@ def main():
         return 3
     from metaljax_amd import kernels as K
 
+    if args.calibration_copy:
+        src = torch.arange(1 << 24, dtype=torch.int32, device="cuda")      # 64 MiB
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.bitwise_not(src, out=dst)
+        torch.cuda.synchronize()
     wl, ms, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
     us = ms * 1e3 / args.steps
     gbs = wl.algorithmic_bytes / us / 1e3
@@ -171,9 +197,13 @@ def main():
                    "algorithmic_bytes": wl.algorithmic_bytes, "flops": wl.flops,
                    "kernel": "decode (M<=16)" if kern == 1 else "prefill", "grid": grid, "block": block},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": committed_traffic()},
         "TFLOP/s": round(wl.flops / us / 1e6, 2),
     }
+    if args.m16_only:
+        print(json.dumps(out))
+        return 0
     # second decode point: the same weight at M = 1
     wl1, ms1, _, _ = bench_decode(2, 1, max(args.steps // 4, 50), max(args.warmup // 4, 5))
     us1 = ms1 * 1e3 / max(args.steps // 4, 50)
