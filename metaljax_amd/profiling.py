@@ -40,7 +40,12 @@ def counter_stats(path: str):
 
 
 def _short(name: str) -> str:
-    return name.replace("void qmm::(anonymous namespace)::", "").split("(")[0][:64]
+    name = name.replace("(anonymous namespace)::", "")
+    if name.startswith("void "):
+        name = name[5:]
+    if name.startswith("qmm::"):
+        name = name[5:]
+    return name.split("(")[0][:64]
 
 
 def main(argv):
