@@ -71,9 +71,11 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
 size_t qmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int group_size,
                            int bits, int mode, int x_dtype);
 
-/* Scratch bytes qmm_gather_qmm needs for P pairs over E experts (0 when the
- * pairs are few enough to run as independent decode products). */
-size_t qmm_gather_workspace_bytes(int64_t P, int64_t E);
+/* Scratch bytes qmm_gather_qmm wants for P pairs over E experts of [N, K]
+ * weights (0 when the pairs are few enough to run as independent decode
+ * products): the expert sort's arrays plus the re-laid activation copy of the
+ * fast kernel.  With only the sort's share the call still runs, slower. */
+size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K);
 
 /* The kernel family and launch geometry the dispatcher would choose. */
 int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode,

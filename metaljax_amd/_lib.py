@@ -65,7 +65,7 @@ def load():
                                          ci, ci, ci, vp, sz, vp]
     lib.qmm_workspace_bytes.argtypes = [i64, i64, i64, i64, ci, ci, ci, ci]
     lib.qmm_workspace_bytes.restype = sz
-    lib.qmm_gather_workspace_bytes.argtypes = [i64, i64]
+    lib.qmm_gather_workspace_bytes.argtypes = [i64, i64, i64, i64]
     lib.qmm_gather_workspace_bytes.restype = sz
     lib.qmm_plan.argtypes = [i64, i64, i64, ci, ci, ci, ip, ip, ip]
     lib.qmm_gather_qmm.argtypes = [vp, ci, vp, vp, vp, ci, vp, ci, vp, vp, i64, i64, i64, i64,

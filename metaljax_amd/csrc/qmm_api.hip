@@ -22,8 +22,9 @@ bool gemm2_supported(int64_t R, int64_t N, int64_t K);
 size_t gemm2_workspace_bytes(int64_t R, int64_t K);
 void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                     int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
-                    const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
-                    int bits, int mode, int row_tile, void* workspace, hipStream_t st);
+                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
+                    int64_t K, int gs, int bits, int mode, int row_tile, void* workspace,
+                    hipStream_t st);
 bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K);
 size_t mxfp4_workspace_bytes(int64_t R, int64_t K);
 void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block);
@@ -109,6 +110,11 @@ __global__ __launch_bounds__(1024) void route_kernel(const int32_t* __restrict__
     row_offsets[e] = 0;
     if (e < E) cursor[e] = 0;
   }
+  // slots that no valid pair lands in (pairs naming an expert outside [0, E)) gather nothing
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    src_row[p] = -1;
+    out_row[p] = -1;
+  }
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
     const int e = rhs_idx[p];
@@ -135,8 +141,8 @@ __global__ __launch_bounds__(1024) void route_kernel(const int32_t* __restrict__
   }
 }
 
-size_t route_bytes(int64_t P, int64_t E) {
-  return (size_t)(2 * E + 1 + 2 * P) * sizeof(int32_t) + 64;
+size_t route_bytes(int64_t P, int64_t E) {     // a multiple of 256: what follows stays aligned
+  return ((size_t)(2 * E + 1 + 2 * P) * sizeof(int32_t) + 255) / 256 * 256;
 }
 
 }  // namespace
@@ -157,8 +163,11 @@ size_t qmm_workspace_bytes(int64_t, int64_t M, int64_t N, int64_t K, int, int, i
   return 0;
 }
 
-size_t qmm_gather_workspace_bytes(int64_t P, int64_t E) {
-  return P <= kGatherGemvMaxPairs ? 0 : route_bytes(P, E);
+size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K) {
+  if (P <= kGatherGemvMaxPairs) return 0;
+  // the expert sort's arrays, then (when the register-operand kernel serves
+  // the shape) the re-laid copy of the gathered activation rows
+  return route_bytes(P, E) + (gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0);
 }
 
 int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode, int* kernel,
@@ -253,7 +262,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
                      static_cast<const char*>(scales) + z * N * ng * tabsz,
                      biases ? static_cast<const char*>(biases) + z * N * ng * tabsz : nullptr,
                      table_dtype, static_cast<char*>(y) + z * M * N * ysz, y_dtype, nullptr, nullptr,
-                     nullptr, M, 1, N, K, group_size, bits, mode, bm, workspace, st);
+                     nullptr, M, M, 1, N, K, group_size, bits, mode, bm, workspace, st);
       rc = check_launch("gemm launch");
       if (rc) return rc;
     }
@@ -289,7 +298,7 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   if (gemm2_supported(R, N, K) && workspace && workspace_bytes >= gemm2_workspace_bytes(R, K) &&
       aligned16(workspace)) {
     gemm2_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
-                   E, N, K, group_size, bits, mode, (int)gemm_row_tile(R, E), workspace,
+                   R, E, N, K, group_size, bits, mode, (int)gemm_row_tile(R, E), workspace,
                    static_cast<hipStream_t>(stream));
     return check_launch("grouped gemm launch");
   }
@@ -331,6 +340,14 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
                      ro, cursor, src_row, out_row);
   rc = check_launch("route launch");
   if (rc) return rc;
+  if (gemm2_supported(P, N, K) && workspace_bytes >= need + gemm2_workspace_bytes(P, K) &&
+      aligned16(workspace)) {
+    // rows gathered in expert order into the re-laid copy, results scattered back to pair order
+    gemm2_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
+                   group_size, bits, mode, (int)gemm_row_tile(P, E),
+                   static_cast<char*>(workspace) + need, st);
+    return check_launch("gather gemm launch");
+  }
   gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
                 group_size, bits, mode, st);
   return check_launch("gather gemm launch");

@@ -56,15 +56,18 @@ __device__ __forceinline__ int swz(int row, int piece) { return row * kRowBytes 
 // One thread = one row's 64 bytes (4 pieces); consecutive threads = consecutive rows.
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* __restrict__ x,
                                                         const int32_t* __restrict__ lhs_idx,
-                                                        u32x4* __restrict__ ax, int R, int K, int Rp) {
+                                                        u32x4* __restrict__ ax, int R, int x_rows,
+                                                        int K, int Rp) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int row = (int)(idx % Rp);
   const int chunk = (int)(idx / Rp);               // 32 elements = 4 pieces
   if (chunk >= K / 32 || row >= R) return;
   const int64_t src = lhs_idx ? (int64_t)lhs_idx[row] : (int64_t)row;
-  const u32x4* p = reinterpret_cast<const u32x4*>(x + src * K + chunk * 32);
+  const bool ok = src >= 0 && src < x_rows;        // an index outside x gathers a zero row
+  const u32x4* p = reinterpret_cast<const u32x4*>(x + (ok ? src : 0) * K + chunk * 32);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) ax[((int64_t)chunk * 4 + j) * Rp + row] = p[j];
+  for (int j = 0; j < 4; ++j)
+    ax[((int64_t)chunk * 4 + j) * Rp + row] = ok ? p[j] : u32x4{0u, 0u, 0u, 0u};
 }
 
 // ---------------------------------------------------------------------------
@@ -469,14 +472,15 @@ size_t gemm2_workspace_bytes(int64_t R, int64_t K) { return (size_t)(prep_rows(R
 // x bf16 [x_rows, K] (rows gathered through lhs_idx when given); the rest as gemm_dispatch.
 void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                     int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
-                    const int32_t* out_idx, int64_t R, int64_t E, int64_t N, int64_t K, int gs,
-                    int bits, int mode, int row_tile, void* workspace, hipStream_t st) {
+                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
+                    int64_t K, int gs, int bits, int mode, int row_tile, void* workspace,
+                    hipStream_t st) {
   if (R == 0 || N == 0) return;
   const int64_t rp = prep_rows(R);
   const int64_t threads = rp * (K / 32);
   hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
                      static_cast<const uint16_t*>(x), lhs_idx, static_cast<u32x4*>(workspace),
-                     (int)R, (int)K, (int)rp);
+                     (int)R, (int)x_rows, (int)K, (int)rp);
   Gemm2Args a;
   a.ax = workspace;
   a.w = static_cast<const uint32_t*>(w);

@@ -142,7 +142,7 @@ def gather_qmm(x, w, scales, biases=None, lhs_indices=None, rhs_indices=None, tr
     y = torch.empty((p, n), dtype=out_dtype, device=x.device)
     x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
     biases = None if biases is None else biases.contiguous()
-    nbytes = int(lib.qmm_gather_workspace_bytes(p, e))
+    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
     tab = _dt(scales.dtype) if mode == "affine" else BF16
     rc = lib.qmm_gather_qmm(_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab,

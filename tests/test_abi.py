@@ -68,9 +68,9 @@ def test_plan_picks_the_regime(lib):
 
 def test_workspace_queries_need_no_device(lib):
     assert lib.qmm_workspace_bytes(1, 16, 14336, 4096, 64, 4, 0, _lib.BF16) == 0
-    need = lib.qmm_gather_workspace_bytes(1024, 8)
+    need = lib.qmm_gather_workspace_bytes(1024, 8, 14336, 4096)
     assert need > 0 and need % 4 == 0
-    assert lib.qmm_gather_workspace_bytes(0, 8) >= 0
+    assert lib.qmm_gather_workspace_bytes(0, 8, 64, 64) >= 0
 
 
 def test_argument_errors_are_reported_before_any_launch(lib):

@@ -424,6 +424,85 @@ def test_gather_qmm_unsorted_pairs(pairs):
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
 
 
+@pytest.mark.parametrize("bits,mode", [(4, "affine"), (8, "affine"), (4, "mxfp4")])
+def test_gather_qmm_many_pairs_skewed_experts(bits, mode):
+    """Prefill-sized pair lists: one expert takes most pairs, one takes none,
+    and the rows come back in pair order whatever the sort inside did."""
+    rng = np.random.default_rng(100 + bits + len(mode))
+    e, n, k, t = 6, 200, 512, 700
+    if mode == "affine":
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, 64, lead=(e,))
+        gs = 64
+    else:
+        _, words, s, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+        b, bd, gs = None, None, 32
+    x, xd = make_x(rng, t, k)
+    p = 2 * t
+    lhs = rng.permutation(np.repeat(np.arange(t), 2)).astype(np.int32)
+    rhs = rng.choice(e, size=p, p=[0.7, 0.1, 0.0, 0.1, 0.05, 0.05]).astype(np.int32)
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, gs, bits, mode,
+                        weight_rounding="bf16")[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV),
+                             torch.from_numpy(rhs).to(DEV), group_size=gs, bits=bits, mode=mode,
+                             out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+    # bf16 results, identity lhs (pair p reads row p)
+    want2 = O.gather_qmm(x[:, None, :], words, s, b, np.arange(t), rhs[:t], gs, bits, mode,
+                         weight_rounding="bf16")[:, 0]
+    y2 = out_f32(K.gather_qmm(xd, wd, sd, bd, None, torch.from_numpy(rhs[:t]).to(DEV),
+                              group_size=gs, bits=bits, mode=mode))
+    assert O.rel_l2(y2, want2) <= 1e-2, O.rel_l2(y2, want2)
+
+
+def test_gather_qmm_pairs_naming_no_expert_are_skipped():
+    """An expert index outside [0, E) selects nothing: the pair's row is left
+    as it was and every other row is right."""
+    rng = np.random.default_rng(77)
+    e, n, k, t = 3, 72, 256, 90
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = np.arange(t).astype(np.int32)
+    rhs = rng.integers(0, e, size=t).astype(np.int32)
+    bad = np.array([4, 17, 60])
+    rhs_dev = rhs.copy()
+    rhs_dev[bad] = [e, -1, 1000]
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, weight_rounding="bf16")[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV),
+                             torch.from_numpy(rhs_dev).to(DEV), group_size=64, bits=4,
+                             out_dtype=torch.float32))
+    good = np.setdiff1d(np.arange(t), bad)
+    assert O.rel_l2(y[good], want[good]) <= 2e-5
+
+
+def test_gather_qmm_with_only_the_sort_workspace_still_runs():
+    """The C entry point accepts the smaller workspace (the expert sort's arrays
+    alone) and serves the call on the general kernel."""
+    from metaljax_amd import _lib
+    from metaljax_amd.kernels import _ptr, _dt, _stream
+    lib = _lib.load()
+    rng = np.random.default_rng(5)
+    e, n, k, t = 4, 64, 256, 150
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    rhs = rng.integers(0, e, size=t).astype(np.int32)
+    rd = torch.from_numpy(rhs).to(DEV)
+    full = int(lib.qmm_gather_workspace_bytes(t, e, n, k))
+    small = ((2 * e + 1 + 2 * t) * 4 + 255) // 256 * 256
+    assert full > small
+    ws = torch.empty(small, dtype=torch.uint8, device=DEV)
+    y = torch.empty((t, n), dtype=torch.float32, device=DEV)
+    rc = lib.qmm_gather_qmm(_ptr(xd), _lib.BF16, _ptr(wd), _ptr(sd), _ptr(bd), _lib.BF16, _ptr(y),
+                            _dt(torch.float32), None, _ptr(rd), t, t, e, n, k, 64, 4, 0, _ptr(ws),
+                            small, _stream(xd))
+    assert rc == 0, lib.qmm_last_error()
+    want = O.gather_qmm(x[:, None, :], words, s, b, np.arange(t), rhs, weight_rounding="bf16")[:, 0]
+    assert O.rel_l2(out_f32(y), want) <= 2e-5
+    rc = lib.qmm_gather_qmm(_ptr(xd), _lib.BF16, _ptr(wd), _ptr(sd), _ptr(bd), _lib.BF16, _ptr(y),
+                            _dt(torch.float32), None, _ptr(rd), t, t, e, n, k, 64, 4, 0, _ptr(ws),
+                            small - 256, _stream(xd))
+    assert rc == 4 and _lib.ERR_NAMES[rc] == "WORKSPACE"
+
+
 def test_c5_moe_scaled():
     wl = synth.make(5, scale=1 / 56)                  # N = 256, 18 tokens... of the same draw
     x, w, s, b, ro = synth.to_device(wl)
