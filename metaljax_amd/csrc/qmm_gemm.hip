@@ -363,7 +363,12 @@ int env_int(const char* name) {
 int64_t gemm_row_tile(int64_t R, int64_t E) {
   static const int env_bm = env_int("QMM_GEMM_BM");
   if (env_bm) return env_bm;
+  // Grouped rows are ragged around R / E: once the mean nears 128 many experts
+  // spill into a second 128-row tile that is almost empty, while a 256-row
+  // tile takes each of them in one (and runs its short main loop for the
+  // experts that fill at most half of it).
   const int64_t per_group = E > 0 ? R / E : R;
+  if (E > 1) return per_group > 96 ? 256 : 128;
   return per_group >= 512 ? 256 : 128;
 }
 

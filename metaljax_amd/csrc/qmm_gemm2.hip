@@ -85,6 +85,14 @@ struct Gemm2Args {
   int tabfast;           // table rows are dword-aligned: fetch them as 16-byte windows
 };
 
+// Rows [lo, hi) of expert i, forced into [0, R] and hi >= lo whatever the offsets hold.
+__device__ __forceinline__ void group_rows(const Gemm2Args& a, int i, int& lo, int& hi) {
+  lo = a.row_offsets[i];
+  hi = a.row_offsets[i + 1];
+  lo = lo < 0 ? 0 : (lo > a.R ? a.R : lo);
+  hi = hi < lo ? lo : (hi > a.R ? a.R : hi);
+}
+
 // 32 codes (one row, one 32-group) -> four 16-byte pieces of bf16 weights
 template <int MODE, int BITS>
 __device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float sc, float bi) {
@@ -117,15 +125,19 @@ __device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float 
 }
 
 // MT x NT MFMA tiles (32 x 32) per wavefront; WMW wavefronts stacked in M and
-// 4 / WMW side by side in N, which always spans the 128 weight rows of a tile:
-//   MT=2 NT=4 WMW=4: 256 x 128 workgroup tile (every wavefront reads the whole
-//                    weight tile, activations are private);
-//   MT=2 NT=2 WMW=2: 128 x 128 (for short row groups: half the LDS reads a
-//                    wavefront, the two wavefronts of a row block fetch the
-//                    same activation fragments).
-// NWAVES = 8 puts two wavefronts on every SIMD (one's vector ALU and load issue
-// fill the other's MFMA shadow) at half the work each.
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
+// NWAVES / WMW side by side in N, which always spans the 128 weight rows of a tile:
+//   MT=2 NT=4 WMW=4 NWAVES=4: 256 x 128 workgroup tile, one wavefront a SIMD
+//                    (every wavefront reads the whole weight tile, activations
+//                    are private);
+//   MT=1 NT=2 WMW=4 NWAVES=8: 128 x 128 for short row groups, two wavefronts a
+//                    SIMD (one's vector ALU and load issue fill the other's
+//                    MFMA shadow) at a quarter of the work each.
+//
+// RAG (ragged row groups: the grouped launches) deals a wavefront's row blocks
+// round-robin (block wm + i*WMW instead of wm*MT + i), so that a tile whose
+// rows end in its first half leaves every wavefront's second block empty and
+// runs a main loop without it.
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG>
 __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   constexpr int WNW = NWAVES / WMW;
   static_assert(WNW * NT * 32 == BN, "the wavefronts must span the weight tile");
@@ -136,6 +148,8 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   constexpr int CPT = BK / TPR;                    // codes per thread per K-tile: 32 | 16
   constexpr int PPT = CPT / 8;                     // 16-byte bf16 pieces per thread: 4 | 2
   constexpr int WPT = CPT * WBITS / 32;            // packed words per thread per K-tile
+  constexpr int RB0 = RAG ? 1 : MT;                // row block of (wm, i) = wm*RB0 + i*RBI
+  constexpr int RBI = RAG ? WMW : 1;
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -143,21 +157,43 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   const int wm = wave / WNW, wn = wave % WNW;
   const int li = lane & 31, kh = lane >> 5;
 
-  // ---- which tile?  XCD x (workgroups are dealt round-robin) gets a
-  // contiguous run of tiles, column tile fastest, so the workgroups sharing an
-  // L2 share activation row blocks.
+  // ---- which tile?  Workgroups are dealt round-robin over the 8 XCDs.
+  // Dense: XCD x gets a contiguous run of tiles, column tile fastest, so the
+  // workgroups sharing an L2 share activation row blocks.
+  // Grouped: XCD x gets a band of column tiles of every expert, expert after
+  // expert.  Experts differ in rows (a tile that is at most half full runs the
+  // short main loop), and this way every XCD sees the same mix, while the
+  // workgroups in flight on one XCD still share an expert's rows.
   const int n_tiles = (a.N + BN - 1) / BN;
-  const int total = n_tiles * a.m_tiles;
-  const int per = (total + 7) / 8;
-  const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  if (tile >= total) return;
-  const int tile_n = tile % n_tiles, tile_m = tile / n_tiles;
+  int tile_n, tile_m;
+  if (a.row_offsets) {
+    // the grid is provisioned for the worst raggedness: count the row tiles that exist
+    int m_tiles = 0;
+    for (int i = 0; i < a.E; ++i) {
+      int lo, hi;
+      group_rows(a, i, lo, hi);
+      m_tiles += (hi - lo + BM - 1) / BM;
+    }
+    const int band = (n_tiles + 7) / 8;
+    const int l = blockIdx.x >> 3;
+    tile_m = l / band;
+    tile_n = (blockIdx.x & 7) * band + l % band;
+    if (tile_m >= m_tiles || tile_n >= n_tiles) return;
+  } else {
+    const int total = n_tiles * a.m_tiles;
+    const int per = (total + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    if (tile >= total) return;
+    tile_n = tile % n_tiles;
+    tile_m = tile / n_tiles;
+  }
   int e = 0, row_lo = 0, row_hi = a.R, mt_idx = tile_m;
   if (a.row_offsets) {
     int t = tile_m;
     bool found = false;
     for (int i = 0; i < a.E; ++i) {
-      const int lo = a.row_offsets[i], hi = a.row_offsets[i + 1];
+      int lo, hi;
+      group_rows(a, i, lo, hi);
       const int tiles = (hi - lo + BM - 1) / BM;
       if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
       t -= tiles;
@@ -177,19 +213,20 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   const char* bb = (MODE == 1) ? nullptr : static_cast<const char*>(a.b) + (int64_t)e * a.N * ng * tabsz;
 
   // ---- activation fragments: lane (row li, k-half kh) of row tile i, k-step ks
-  // reads ax[(kt*8 + ks*2 + kh) * Rp + m0 + wm*WM + i*32 + li]
+  // reads ax[(kt*8 + ks*2 + kh) * Rp + m0 + (wm*RB0 + i*RBI)*32 + li]
   const auto ra = make_rsrc(a.ax, (int64_t)(a.K / 8) * a.Rp * 16);
-  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * WM + li) * 16);
+  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * (RB0 * 32) + li) * 16);
   typedef u32x4 AFrag[4][MT];
-  auto load_a_part = [&](int kt, AFrag& dst, int ks) {       // the fragments of one k-step
+  auto load_a_part = [&](int kt, AFrag& dst, int ks, auto ac) __attribute__((always_inline)) {   // the fragments of one k-step
+    constexpr int ACT = decltype(ac)::value;
     const uint32_t so = (uint32_t)((kt * 8 + ks * 2) * 16) * (uint32_t)a.Rp;
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-      dst[ks][i] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo + i * 512, so, 0);
+    for (int i = 0; i < ACT; ++i)
+      dst[ks][i] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo + i * (RBI * 512), so, 0);
   };
-  auto load_a = [&](int kt, AFrag& dst) {
+  auto load_a = [&](int kt, AFrag& dst, auto ac) __attribute__((always_inline)) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_a_part(kt, dst, ks);
+    for (int ks = 0; ks < 4; ++ks) load_a_part(kt, dst, ks, ac);
   };
 
   // ---- weight staging: thread -> (row tid/TPR, k-part tid%TPR): CPT codes a K-tile
@@ -292,10 +329,13 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // of tile 1 in flight
   TabWin tw_cur, tw_nxt;
   if (a.tabfast) load_win(0, tw_cur);
+  const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;   // uniform over the workgroup
   load_w(0, wr[0]);
-  load_a(0, af[0]);
+  if (half_tile) load_a(0, af[0], std::integral_constant<int, 1>{});
+  else load_a(0, af[0], std::integral_constant<int, MT>{});
   load_w(clampk(1), wr[1]);
-  load_a(clampk(1), af[1]);
+  if (half_tile) load_a(clampk(1), af[1], std::integral_constant<int, 1>{});
+  else load_a(clampk(1), af[1], std::integral_constant<int, MT>{});
   load_w(clampk(2), wr[2]);
   load_w(clampk(3), wr[3]);
   {
@@ -321,8 +361,9 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // instruction, with a quarter of everything else the tile needs: the loads
   // of tile kt+2, one piece of tile kt+1's dequantization, the fragment reads
   // of the next k-step.
-  auto step = [&](int kt, auto tc) {
+  auto step = [&](int kt, auto tc, auto ac) __attribute__((always_inline)) {
     constexpr int t = decltype(tc)::value;         // kt & 3
+    constexpr int ACT = decltype(ac)::value;       // row blocks this wavefront multiplies
     const unsigned char* pb = smem + (kt % kStages) * kStage;
     const int nstage = (kt + 1) % kStages;
     const bool has_next = kt + 1 < KT;             // uniform
@@ -332,14 +373,14 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1);
-      load_a_part(kt2, af[(t + 2) & 3], ks);
+      load_a_part(kt2, af[(t + 2) & 3], ks, ac);
       if (ks == 0) load_w(kt4, wr[t & 3]);          // three K-tiles ahead of its dequantization
       if (ks == 1 && t == 0 && a.tabfast) {        // next quad's table window (clamped at the end)
         const int q = (kt >> 2) + 1;
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
       }
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
+      for (int i = 0; i < ACT; ++i) {
         const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][i]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
@@ -351,9 +392,9 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
       // order inside the k-step: fragment reads first, then MFMA / ALU / load slots
       __builtin_amdgcn_sched_group_barrier(0x100, NT, 0);      // ds reads
 #pragma unroll
-      for (int m = 0; m < MT * NT; ++m) {
+      for (int m = 0; m < ACT * NT; ++m) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 32 / (MT * NT), 0);   // a few vector ALU instructions
+        __builtin_amdgcn_sched_group_barrier(0x002, 32 / (ACT * NT), 0);   // a few vector ALU instructions
         if (m < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one vector-memory load
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -362,16 +403,24 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     lds_barrier();
     if (has_next) read_b(smem + nstage * kStage, 0, 0);
   };
-  int kt = 0;
-  for (; kt + 4 <= KT; kt += 4) {
-    step(kt, std::integral_constant<int, 0>{});
-    step(kt + 1, std::integral_constant<int, 1>{});
-    step(kt + 2, std::integral_constant<int, 2>{});
-    step(kt + 3, std::integral_constant<int, 3>{});
+  auto run = [&](auto ac) __attribute__((always_inline)) {
+    int kt = 0;
+    for (; kt + 4 <= KT; kt += 4) {
+      step(kt, std::integral_constant<int, 0>{}, ac);
+      step(kt + 1, std::integral_constant<int, 1>{}, ac);
+      step(kt + 2, std::integral_constant<int, 2>{}, ac);
+      step(kt + 3, std::integral_constant<int, 3>{}, ac);
+    }
+    if (kt < KT) { step(kt, std::integral_constant<int, 0>{}, ac); ++kt; }
+    if (kt < KT) { step(kt, std::integral_constant<int, 1>{}, ac); ++kt; }
+    if (kt < KT) { step(kt, std::integral_constant<int, 2>{}, ac); ++kt; }
+  };
+  if constexpr (RAG && MT == 2) {
+    if (half_tile) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, MT>{});
+  } else {
+    run(std::integral_constant<int, MT>{});
   }
-  if (kt < KT) { step(kt, std::integral_constant<int, 0>{}); ++kt; }
-  if (kt < KT) { step(kt, std::integral_constant<int, 1>{}); ++kt; }
-  if (kt < KT) { step(kt, std::integral_constant<int, 2>{}); ++kt; }
 
   // ---- epilogue.  D[i][j] of a 32x32 tile: lane holds column lane % 32 and
   // rows (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5), r = 0..15.
@@ -399,7 +448,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
 #pragma unroll
       for (int q = 0; q < WC / 16; ++q) {          // 32 rows x WC/8 pieces over 64 lanes
         const int idx = q * 64 + lane, rl = idx / (WC / 8), pc = idx % (WC / 8);
-        const int m = m0 + wm * WM + i * 32 + rl, n = n0 + wn * WC + pc * 8;
+        const int m = m0 + (wm * RB0 + i * RBI) * 32 + rl, n = n0 + wn * WC + pc * 8;
         if (m < row_hi && n < a.N) {
           const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
           *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + n) =
@@ -418,7 +467,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
         const int n = n0 + wn * (NT * 32) + j * 32 + li;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * WM + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          const int m = m0 + (wm * RB0 + i * RBI) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
           if (m < row_hi && n < a.N) {
             const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
             store_out(a.y, orow * a.N + n, acc[i][j][r], a.y_dtype);
@@ -428,15 +477,17 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   }
 }
 
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
-void launch2(const Gemm2Args& a0, hipStream_t st) {
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG>
+void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   constexpr int BM = WMW * MT * 32;
   Gemm2Args a = a0;
   a.m_tiles = (int)(a.row_offsets ? ceil_div(a.R, BM) + a.E : ceil_div(a.R, BM));
-  const int64_t total = ceil_div(a.N, BN) * a.m_tiles;
-  dim3 grid((unsigned)(ceil_div(total, 8) * 8));
+  // dense: tiles rounded up to the 8 XCDs; grouped: 8 bands of column tiles x provisioned row tiles
+  const int64_t total = a.row_offsets ? ceil_div(ceil_div(a.N, BN), 8) * 8 * a.m_tiles
+                                      : ceil_div(ceil_div(a.N, BN) * a.m_tiles, 8) * 8;
+  dim3 grid((unsigned)total);
   const size_t lds = kStages * kStage;            // 48 KB (the epilogue reuses 32 KB of it)
-  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES>;
+  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG>;
   static bool configured = false;
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -446,16 +497,16 @@ void launch2(const Gemm2Args& a0, hipStream_t st) {
   hipLaunchKernelGGL(kern, grid, dim3(64 * NWAVES), lds, st, a);
 }
 
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
+void launch2(const Gemm2Args& a, hipStream_t st) {
+  if (a.row_offsets) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, true>(a, st);
+  else launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, false>(a, st);
+}
+
 template <int MODE, int BITS>
 void launch2_mt(const Gemm2Args& a, int mt, hipStream_t st) {
-  static const int variant = getenv("QMM_G2_VARIANT") ? atoi(getenv("QMM_G2_VARIANT")) : 0;
-  if (mt == 2) {
-    if (variant == 1) launch2<MODE, BITS, 2, 2, 4, 8>(a, st);      // 256 x 128, eight wavefronts
-    else launch2<MODE, BITS, 2, 4, 4, 4>(a, st);                   // 256 x 128, four wavefronts
-  } else {
-    if (variant == 2) launch2<MODE, BITS, 2, 2, 2, 4>(a, st);      // 128 x 128, four wavefronts
-    else launch2<MODE, BITS, 1, 2, 4, 8>(a, st);                   // 128 x 128, eight wavefronts
-  }
+  if (mt == 2) launch2<MODE, BITS, 2, 4, 4, 4>(a, st);     // 256 x 128, four wavefronts
+  else launch2<MODE, BITS, 1, 2, 4, 8>(a, st);             // 128 x 128, eight wavefronts
 }
 
 int64_t prep_rows(int64_t R) { return ceil_div(R + 256, 64) * 64; }   // a tile may start at any row
