@@ -137,7 +137,15 @@ __device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float 
 // round-robin (block wm + i*WMW instead of wm*MT + i), so that a tile whose
 // rows end in its first half leaves every wavefront's second block empty and
 // runs a main loop without it.
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG>
+//
+// TF selects how scales / biases are fetched.  1..3: as 16-byte windows (four
+// K-tiles of a row at once), with the entry type fixed at compile time --
+// 1 = two-byte bf16 (one-byte E8M0 for MXFP4), 2 = float32, 3 = float16 -- so
+// that picking an entry is a handful of selects and the K loop has no branch
+// in it (a branch would end the region the MFMAs are interleaved in).
+// 0: any layout, one load per entry, types read at run time (unaligned or
+// short tables).
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF>
 __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   constexpr int WNW = NWAVES / WMW;
   static_assert(WNW * NT * 32 == BN, "the wavefronts must span the weight tile");
@@ -207,7 +215,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   const int64_t wpr = (int64_t)a.K * WBITS / 32;
   const int gs = (MODE == 1) ? 32 : a.gs;
   const int64_t ng = a.K / gs;
-  const int tabsz = (MODE == 1) ? 1 : (a.tab == QMM_F32 ? 4 : 2);
+  const int tabsz = (MODE == 1) ? 1 : (TF == 2 ? 4 : TF != 0 ? 2 : (a.tab == QMM_F32 ? 4 : 2));
   const uint32_t* wb = a.w + (int64_t)e * a.N * wpr;
   const char* sb = static_cast<const char*>(a.s) + (int64_t)e * a.N * ng * tabsz;
   const char* bb = (MODE == 1) ? nullptr : static_cast<const char*>(a.b) + (int64_t)e * a.N * ng * tabsz;
@@ -262,10 +270,10 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   auto load_win = [&](int quad, TabWin& tw) {
     const uint32_t so = (uint32_t)(((quad * 4 * BK) >> gshift) * tabsz);
     tw.s[0] = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo, so, 0);
-    if (tabsz == 4) tw.s[1] = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo + 16, so, 0);
+    if constexpr (TF == 2) tw.s[1] = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo + 16, so, 0);
     if constexpr (MODE == 0) {
       tw.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo, so, 0);
-      if (tabsz == 4) tw.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo + 16, so, 0);
+      if constexpr (TF == 2) tw.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo + 16, so, 0);
     }
   };
   // entry index of K-tile t' inside its window, for this thread's k-half
@@ -273,14 +281,15 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
 #pragma unroll
   for (int t = 0; t < 4; ++t) eidx[t] = (uint32_t)((t * BK + whalf * CPT) >> gshift);
   auto pick = [&](const u32x4 (&w)[2], uint32_t e) -> float {
-    // entry e (0..7) of a window of 1-, 2- or 4-byte entries
-    const uint32_t byte = e * (uint32_t)tabsz;
+    // entry e (0..7) of a window of 1-, 2- or 4-byte entries (TF != 0 only)
+    constexpr uint32_t TS = (MODE == 1) ? 1u : (TF == 2 ? 4u : 2u);
+    const uint32_t byte = e * TS;
     const uint32_t d = byte >> 2;
     uint32_t v = w[0][0];
     v = d == 1 ? w[0][1] : v;
     v = d == 2 ? w[0][2] : v;
     v = d == 3 ? w[0][3] : v;
-    if (tabsz == 4) {
+    if constexpr (TF == 2) {
       v = d == 4 ? w[1][0] : v;
       v = d == 5 ? w[1][1] : v;
       v = d == 6 ? w[1][2] : v;
@@ -289,11 +298,12 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     }
     v >>= (byte & 3u) * 8u;
     if constexpr (MODE == 1) return e8m0_to_f32(v & 255u);
-    return a.tab == QMM_BF16 ? bf16_bits_to_f32(v & 0xFFFFu) : f16_bits_to_f32(v & 0xFFFFu);
+    if constexpr (TF == 3) return f16_bits_to_f32(v & 0xFFFFu);
+    return __uint_as_float(v << 16);
   };
   // (scale, bias) of K-tile kt for this thread
   auto entry = [&](int kt, const TabWin& tw, float& sc, float& bi) {
-    if (a.tabfast) {
+    if constexpr (TF != 0) {
       sc = pick(tw.s, eidx[kt & 3]);
       bi = MODE == 1 ? 0.f : pick(tw.b, eidx[kt & 3]);
     } else {
@@ -325,57 +335,77 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   WRegs wr[4];                                    // words of K-tile t live in wr[t & 3]
   auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
-  // prologue: tile 0 dequantized, tiles 0..1 of the activations and the words
-  // of tile 1 in flight
+  // prologue: tiles 0 and 1 dequantized, tiles 0..1 of the activations and the
+  // words of tiles 2..3 in flight
   TabWin tw_cur, tw_nxt;
-  if (a.tabfast) load_win(0, tw_cur);
+  if constexpr (TF != 0) load_win(0, tw_cur);
   const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;   // uniform over the workgroup
+  // Issue order matters: a wait counts the loads issued after the one it needs,
+  // and the waits inside the loop must also hold on its first pass.  The words
+  // that the loop dequantizes first (tiles 2, 3) therefore go out before the
+  // sixteen activation loads, as they do in steady state.
   load_w(0, wr[0]);
-  if (half_tile) load_a(0, af[0], std::integral_constant<int, 1>{});
-  else load_a(0, af[0], std::integral_constant<int, MT>{});
   load_w(clampk(1), wr[1]);
-  if (half_tile) load_a(clampk(1), af[1], std::integral_constant<int, 1>{});
-  else load_a(clampk(1), af[1], std::integral_constant<int, MT>{});
   load_w(clampk(2), wr[2]);
   load_w(clampk(3), wr[3]);
+  if (half_tile) {
+    load_a(0, af[0], std::integral_constant<int, 1>{});
+    load_a(clampk(1), af[1], std::integral_constant<int, 1>{});
+  } else {
+    load_a(0, af[0], std::integral_constant<int, MT>{});
+    load_a(clampk(1), af[1], std::integral_constant<int, MT>{});
+  }
   {
     float sc, bi;
     entry(0, tw_cur, sc, bi);
 #pragma unroll
     for (int pc = 0; pc < PPT; ++pc) store_piece(0, wr[0], pc, sc, bi);
+    entry(clampk(1), tw_cur, sc, bi);
+#pragma unroll
+    for (int pc = 0; pc < PPT; ++pc) store_piece(1, wr[1], pc, sc, bi);
   }
   lds_barrier();
 
-  bf16x8 fb[2][NT];                               // B fragments: k-step ks in set ks & 1
+  bf16x8 fb[4][NT];                               // B fragments: k-step ks of a tile in set ks
   auto read_b = [&](const unsigned char* pbase, int ks, int set) {
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       fb[set][j] = *reinterpret_cast<const bf16x8*>(pbase + swz(wn * (NT * 32) + j * 32 + li, ks * 2 + kh));
   };
   read_b(smem, 0, 0);
+  read_b(smem, 1, 1);
 
   // One K-tile.  A single wavefront per SIMD has to keep its matrix core busy
   // by itself, and both a vector-memory instruction (about 64 clocks to issue
   // 1 KB) and a run of vector ALU work stall the next MFMA if they sit in one
   // lump; so each k-step's eight MFMAs are interleaved, instruction by
   // instruction, with a quarter of everything else the tile needs: the loads
-  // of tile kt+2, one piece of tile kt+1's dequantization, the fragment reads
-  // of the next k-step.
+  // of tile kt+2, one piece of tile kt+2's dequantization, the fragment reads
+  // of the k-step after next.
+  //
+  // Stages: step kt multiplies out of stage kt % 3, fills stage (kt+2) % 3 and,
+  // in its last two k-steps, already reads the first fragments of tile kt+1
+  // (complete since the barrier that ended step kt-1): the four wavefronts
+  // read their fragments at the same moment, so a read issued one k-step
+  // ahead arrives late, and one issued right after the barrier stalls the
+  // first MFMAs of every tile.  One barrier a tile still orders everything:
+  // stage (kt+2) % 3 == (kt-1) % 3 was last read in step kt-1.
   auto step = [&](int kt, auto tc, auto ac) __attribute__((always_inline)) {
     constexpr int t = decltype(tc)::value;         // kt & 3
     constexpr int ACT = decltype(ac)::value;       // row blocks this wavefront multiplies
     const unsigned char* pb = smem + (kt % kStages) * kStage;
-    const int nstage = (kt + 1) % kStages;
-    const bool has_next = kt + 1 < KT;             // uniform
+    const unsigned char* pb1 = smem + ((kt + 1) % kStages) * kStage;
+    const int wstage = (kt + 2) % kStages;
     const int kt2 = clampk(kt + 2), kt4 = clampk(kt + 4);
-    float sc, bi;                                  // of tile kt+1 (the first tile of the next quad at t == 3)
-    entry(kt + 1, t == 3 ? tw_nxt : tw_cur, sc, bi);
+    float sc, bi;                                  // of tile kt+2 (in the next quad's window at t >= 2)
+    entry(kt2, t >= 2 ? tw_nxt : tw_cur, sc, bi);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1);
+      if (ks < 2) read_b(pb, ks + 2, ks + 2);
+      else read_b(pb1, ks - 2, ks - 2);
       load_a_part(kt2, af[(t + 2) & 3], ks, ac);
-      if (ks == 0) load_w(kt4, wr[t & 3]);          // three K-tiles ahead of its dequantization
-      if (ks == 1 && t == 0 && a.tabfast) {        // next quad's table window (clamped at the end)
+      if (ks == 0) load_w(kt4, wr[t & 3]);          // two K-tiles ahead of its dequantization
+      if (TF != 0 && ks == 1 && t == 0) {          // next quad's table window (clamped at the end)
         const int q = (kt >> 2) + 1;
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
       }
@@ -384,11 +414,11 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
         const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][i]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks][j], acc[i][j], 0, 0, 0);
       }
       // (after the last tile this writes a stage nobody reads: cheaper than a branch,
       // which would split the scheduling region)
-      if (PPT == 4 || (ks & 1) == 0) store_piece(nstage, wr[(t + 1) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
+      if (PPT == 4 || (ks & 1) == 0) store_piece(wstage, wr[(t + 2) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
       // order inside the k-step: fragment reads first, then MFMA / ALU / load slots
       __builtin_amdgcn_sched_group_barrier(0x100, NT, 0);      // ds reads
 #pragma unroll
@@ -401,7 +431,6 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     }
     if (t == 3) tw_cur = tw_nxt;
     lds_barrier();
-    if (has_next) read_b(smem + nstage * kStage, 0, 0);
   };
   auto run = [&](auto ac) __attribute__((always_inline)) {
     int kt = 0;
@@ -477,7 +506,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   }
 }
 
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG>
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF>
 void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   constexpr int BM = WMW * MT * 32;
   Gemm2Args a = a0;
@@ -486,8 +515,10 @@ void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   const int64_t total = a.row_offsets ? ceil_div(ceil_div(a.N, BN), 8) * 8 * a.m_tiles
                                       : ceil_div(ceil_div(a.N, BN) * a.m_tiles, 8) * 8;
   dim3 grid((unsigned)total);
-  const size_t lds = kStages * kStage;            // 48 KB (the epilogue reuses 32 KB of it)
-  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG>;
+  // three weight stages; the epilogue transposes 32 x NT*32 sixteen-bit results per wavefront there
+  const size_t epi = (size_t)NWAVES * 32 * NT * 32 * 2;
+  const size_t lds = epi > (size_t)(kStages * kStage) ? epi : (size_t)(kStages * kStage);
+  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG, TF>;
   static bool configured = false;
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -497,10 +528,22 @@ void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   hipLaunchKernelGGL(kern, grid, dim3(64 * NWAVES), lds, st, a);
 }
 
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG>
+void launch2_tf(const Gemm2Args& a, hipStream_t st) {
+  if (!a.tabfast) return launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 0>(a, st);
+  if constexpr (MODE == 1) {
+    launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1>(a, st);
+  } else {
+    if (a.tab == QMM_BF16) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1>(a, st);
+    else if (a.tab == QMM_F32) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 2>(a, st);
+    else launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 3>(a, st);
+  }
+}
+
 template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES>
 void launch2(const Gemm2Args& a, hipStream_t st) {
-  if (a.row_offsets) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, true>(a, st);
-  else launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, false>(a, st);
+  if (a.row_offsets) launch2_tf<MODE, BITS, MT, NT, WMW, NWAVES, true>(a, st);
+  else launch2_tf<MODE, BITS, MT, NT, WMW, NWAVES, false>(a, st);
 }
 
 template <int MODE, int BITS>
