@@ -335,14 +335,14 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   WRegs wr[4];                                    // words of K-tile t live in wr[t & 3]
   auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
-  // prologue: tiles 0 and 1 dequantized, tiles 0..1 of the activations and the
-  // words of tiles 2..3 in flight
+  // prologue: tile 0 dequantized, tiles 0..1 of the activations and the words
+  // of tiles 1..3 in flight
   TabWin tw_cur, tw_nxt;
   if constexpr (TF != 0) load_win(0, tw_cur);
   const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;   // uniform over the workgroup
   // Issue order matters: a wait counts the loads issued after the one it needs,
   // and the waits inside the loop must also hold on its first pass.  The words
-  // that the loop dequantizes first (tiles 2, 3) therefore go out before the
+  // that the loop dequantizes first (tiles 1, 2, 3) therefore go out before the
   // sixteen activation loads, as they do in steady state.
   load_w(0, wr[0]);
   load_w(clampk(1), wr[1]);
@@ -360,51 +360,39 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     entry(0, tw_cur, sc, bi);
 #pragma unroll
     for (int pc = 0; pc < PPT; ++pc) store_piece(0, wr[0], pc, sc, bi);
-    entry(clampk(1), tw_cur, sc, bi);
-#pragma unroll
-    for (int pc = 0; pc < PPT; ++pc) store_piece(1, wr[1], pc, sc, bi);
   }
   lds_barrier();
 
-  bf16x8 fb[4][NT];                               // B fragments: k-step ks of a tile in set ks
+  bf16x8 fb[2][NT];                               // B fragments: k-step ks in set ks & 1
   auto read_b = [&](const unsigned char* pbase, int ks, int set) {
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       fb[set][j] = *reinterpret_cast<const bf16x8*>(pbase + swz(wn * (NT * 32) + j * 32 + li, ks * 2 + kh));
   };
   read_b(smem, 0, 0);
-  read_b(smem, 1, 1);
 
   // One K-tile.  A single wavefront per SIMD has to keep its matrix core busy
   // by itself, and both a vector-memory instruction (about 64 clocks to issue
   // 1 KB) and a run of vector ALU work stall the next MFMA if they sit in one
   // lump; so each k-step's eight MFMAs are interleaved, instruction by
   // instruction, with a quarter of everything else the tile needs: the loads
-  // of tile kt+2, one piece of tile kt+2's dequantization, the fragment reads
-  // of the k-step after next.
-  //
-  // Stages: step kt multiplies out of stage kt % 3, fills stage (kt+2) % 3 and,
-  // in its last two k-steps, already reads the first fragments of tile kt+1
-  // (complete since the barrier that ended step kt-1): the four wavefronts
-  // read their fragments at the same moment, so a read issued one k-step
-  // ahead arrives late, and one issued right after the barrier stalls the
-  // first MFMAs of every tile.  One barrier a tile still orders everything:
-  // stage (kt+2) % 3 == (kt-1) % 3 was last read in step kt-1.
+  // of tile kt+2, one piece of tile kt+1's dequantization, the fragment reads
+  // of the next k-step.  (Dequantizing two tiles ahead and reading fragments
+  // two k-steps ahead was measured too: no faster, more registers.)
   auto step = [&](int kt, auto tc, auto ac) __attribute__((always_inline)) {
     constexpr int t = decltype(tc)::value;         // kt & 3
     constexpr int ACT = decltype(ac)::value;       // row blocks this wavefront multiplies
     const unsigned char* pb = smem + (kt % kStages) * kStage;
-    const unsigned char* pb1 = smem + ((kt + 1) % kStages) * kStage;
-    const int wstage = (kt + 2) % kStages;
+    const int nstage = (kt + 1) % kStages;
+    const bool has_next = kt + 1 < KT;             // uniform
     const int kt2 = clampk(kt + 2), kt4 = clampk(kt + 4);
-    float sc, bi;                                  // of tile kt+2 (in the next quad's window at t >= 2)
-    entry(kt2, t >= 2 ? tw_nxt : tw_cur, sc, bi);
+    float sc, bi;                                  // of tile kt+1 (the first tile of the next quad at t == 3)
+    entry(clampk(kt + 1), t == 3 ? tw_nxt : tw_cur, sc, bi);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      if (ks < 2) read_b(pb, ks + 2, ks + 2);
-      else read_b(pb1, ks - 2, ks - 2);
+      if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1);
       load_a_part(kt2, af[(t + 2) & 3], ks, ac);
-      if (ks == 0) load_w(kt4, wr[t & 3]);          // two K-tiles ahead of its dequantization
+      if (ks == 0) load_w(kt4, wr[t & 3]);          // three K-tiles ahead of its dequantization
       if (TF != 0 && ks == 1 && t == 0) {          // next quad's table window (clamped at the end)
         const int q = (kt >> 2) + 1;
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
@@ -414,11 +402,11 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
         const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][i]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[i][j], 0, 0, 0);
       }
       // (after the last tile this writes a stage nobody reads: cheaper than a branch,
       // which would split the scheduling region)
-      if (PPT == 4 || (ks & 1) == 0) store_piece(wstage, wr[(t + 2) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
+      if (PPT == 4 || (ks & 1) == 0) store_piece(nstage, wr[(t + 1) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
       // order inside the k-step: fragment reads first, then MFMA / ALU / load slots
       __builtin_amdgcn_sched_group_barrier(0x100, NT, 0);      // ds reads
 #pragma unroll
@@ -431,6 +419,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     }
     if (t == 3) tw_cur = tw_nxt;
     lds_barrier();
+    if (has_next) read_b(smem + nstage * kStage, 0, 0);
   };
   auto run = [&](auto ac) __attribute__((always_inline)) {
     int kt = 0;
