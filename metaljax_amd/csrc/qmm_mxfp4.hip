@@ -275,43 +275,54 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   };
   auto quad_of = [&](int qi) { return wave + 4 * (qi < nq - 1 ? qi : nq - 1); };
 
+  // Loads retire in order, so a wait can only say "all but the newest n have
+  // landed": the order of issue has to be the order of use.  A K-step i uses
+  // its activation terms A(i) and its weight codes W(i); step i issues A(i+2)
+  // during its first two MFMA groups and W(i+3) during its last two, and
+  // before its last group waits for W(i+1) and reads its fragments, so that a
+  // step starts with its weight operands already in registers.  The prologue issues in the same
+  // order (W0 A0 W1 A1 W2), which keeps every count in the loop valid on its
+  // first pass.  A step issues 20 loads, the first of a quad 10 more (its
+  // activation scales and the next quad's weight scales).
+  i32x8 bfq[2][2][4];                             // [step parity][u][nt] weight fragments
+  auto read_bf = [&](int stage, i32x8 (&dst)[2][4]) {
+    const unsigned char* st = wbase + stage * kStageBytes;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        dst[u][nt] = as_fp4_operand(*reinterpret_cast<const u32x4*>(st + rd_off[u] + nt * 2048));
+  };
+  auto read_sbq = [&](int par) {
+    const unsigned char* sq = sbase + par * kScaleBytes + li * 16;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) sbq[nt] = *reinterpret_cast<const u32x4*>(sq + nt * 512);
+  };
   if (nq > 0) {
     issue_sa(quad_of(0), sa);
     dma_s(quad_of(0), 0);
-    issue_a(kstep_of(0), areg[0]);
     dma_w(kstep_of(0), 0);
-    issue_a(kstep_of(1), areg[1]);
+    issue_a(kstep_of(0), areg[0]);
     dma_w(kstep_of(1), 1);
+    issue_a(kstep_of(1), areg[1]);
     dma_w(kstep_of(2), 2);
-    auto step = [&](int qi, auto tc) {
+    wait_vmcnt<40>();                              // W0 and the first scales
+    read_bf(0, bfq[0]);
+    read_sbq(0);
+    auto step = [&](int qi, auto tc) __attribute__((always_inline)) {
       constexpr int t = decltype(tc)::value;
       const int i = 4 * qi + t;
-      // Landed by now: everything but the loads issued during the previous
-      // step and the two weight loads that ended the step before it, i.e. this
-      // step's activation terms, codes and scales.
-      wait_vmcnt<(t == 1 ? 32 : 22)>();
+      // A(i) has landed once at most W(i+1) and the previous step's loads are out
+      wait_vmcnt<(t == 1 ? 38 : 28)>();
       const int ks_a = kstep_of(i + 2), ks_w = kstep_of(i + 3);
-
-      const unsigned char* st = wbase + t * kStageBytes;
-      if (t == 0) {
-        const unsigned char* sq = sbase + (qi & 1) * kScaleBytes + li * 16;
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt) sbq[nt] = *reinterpret_cast<const u32x4*>(sq + nt * 512);
-      }
-      i32x8 bf[2][4];
       int sb[2][4];
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
-          bf[u][nt] = as_fp4_operand(*reinterpret_cast<const u32x4*>(st + rd_off[u] + nt * 2048));
-          sb[u][nt] = (int)(sbq[nt][t] >> sh[u]);
-        }
-      // Four groups of 8 MFMAs; after each, a quarter of the loads for later
-      // steps (activation terms two steps ahead, weight codes three steps
-      // ahead), so that load issue hides under the matrix-core work of this
-      // single wavefront per SIMD.  Loads retire in order: the activation part
-      // goes first in each quarter.
+        for (int nt = 0; nt < 4; ++nt) sb[u][nt] = (int)(sbq[nt][t] >> sh[u]);
+      // Four groups of 8 MFMAs, each followed by a share of the loads for later
+      // steps, so that load issue hides under the matrix-core work of this
+      // single wavefront per SIMD.
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int u = g >> 1, term = g & 1;
@@ -321,13 +332,27 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
 #pragma unroll
           for (int nt = 0; nt < 4; ++nt)
             acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                af, bf[u][nt], acc[mt][nt], kFp6, kFp4, t, (int)sa[u][mt][term], 0, sb[u][nt]);
+                af, bfq[t & 1][u][nt], acc[mt][nt], kFp6, kFp4, t, (int)sa[u][mt][term], 0, sb[u][nt]);
         }
         __builtin_amdgcn_sched_barrier(0);
-        issue_a_part(ks_a, areg[(t + 2) & 3], g);
-        if (t == 0 && g == 0) issue_sa(quad_of(qi + 1), sa_nxt);
-        dma_w_part(ks_w, (t + 3) & 3, g);
-        if (t == 0 && g == 0) dma_s(quad_of(qi + 1), (qi + 1) & 1);
+        if (g < 2) {
+          issue_a_part(ks_a, areg[(t + 2) & 3], 2 * g);
+          issue_a_part(ks_a, areg[(t + 2) & 3], 2 * g + 1);
+          if (t == 0 && g == 0) {
+            issue_sa(quad_of(qi + 1), sa_nxt);
+            dma_s(quad_of(qi + 1), (qi + 1) & 1);
+          }
+        } else {
+          dma_w_part(ks_w, (t + 3) & 3, 2 * (g - 2));
+          dma_w_part(ks_w, (t + 3) & 3, 2 * (g - 2) + 1);
+        }
+        if (g == 2) {
+          // W(i+1): everything but the previous step's loads and this step's so far;
+          // the fragment reads then run under the last MFMA group
+          wait_vmcnt<(t <= 1 ? 46 : 36)>();
+          read_bf((t + 1) & 3, bfq[(t + 1) & 1]);
+          if (t == 3) read_sbq((qi + 1) & 1);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       if (t == 3) {
