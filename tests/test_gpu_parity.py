@@ -274,6 +274,36 @@ def test_gemm_affine(bits, gs, m, n, k):
     assert O.rel_l2(y16, want_exact) <= TOL_BF16_OUT
 
 
+@pytest.mark.parametrize("tab", ["f32", "f16"])
+@pytest.mark.parametrize("gs,bits", [(32, 4), (64, 8), (128, 4)])
+@pytest.mark.parametrize("k", [512, 320])
+def test_gemm_table_dtypes(tab, gs, bits, k):
+    """float32 / float16 scale and bias tables on the prefill kernel: K = 512
+    fetches them as 16-byte windows, K = 320 entry by entry."""
+    if k % gs:
+        pytest.skip("K must be a multiple of the group size")
+    rng = np.random.default_rng(gs + bits + k)
+    m, n = 40, 136
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, s, b, gs, bits, weight_rounding="bf16")
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+def test_grouped_qmm_float32_tables_and_eight_bit_codes():
+    rng = np.random.default_rng(23)
+    e, n, k = 3, 200, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 8, 64, "f32", lead=(e,))
+    sizes = np.array([150, 20, 131])
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    x, xd = make_x(rng, int(ro[-1]), k)
+    want = O.grouped_qmm(x, words, s, b, ro, 64, 8, weight_rounding="bf16")
+    y = out_f32(K.grouped_qmm(xd, wd, sd, bd, torch.from_numpy(ro).to(DEV), group_size=64, bits=8,
+                              out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
 @pytest.mark.parametrize("m,n,k", [(17, 40, 128), (256, 136, 1024)])
 def test_gemm_mxfp4(m, n, k):
     rng = np.random.default_rng(m + n)
