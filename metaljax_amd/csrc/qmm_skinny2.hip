@@ -1,0 +1,413 @@
+// Decode-regime affine quantized matmul (M <= 16) with loader wavefronts.
+//
+// Same arithmetic as qmm_skinny.hip (codes exact in bf16, two
+// v_mfma_f32_16x16x32_bf16 per 64-code chunk, scale applied to the chunk's
+// dot, the code-independent terms as small MFMAs over the chunk index); what
+// differs is who moves the bytes.
+//
+// A compute unit cannot keep its whole share of the weight (about 130 KB for
+// the 4096 x 14336 case) in flight: vector-memory instructions are accepted at
+// the pace the memory system returns data, and a wavefront that issues all its
+// loads first spends most of the streaming time blocked in issue, computing
+// only afterwards.  Here NL loader wavefronts do nothing but issue
+// direct-to-LDS loads (they are the ones that block), and CW compute
+// wavefronts never touch global memory until the final store: they consume
+// "items" from a three-slot LDS ring as the loaders complete them.
+//
+// Items of one pass (a pass = CW consecutive K-slices, one per compute
+// wavefront; a slice = 256 packed bytes per row):
+//   XR activation rounds  [CW slices][16 rows m][256 bytes = 128 codes of x]
+//   TMAX weight tiles     [CW slices][16 rows n][256 packed bytes] + table rows
+// Every item is CW * 4 KB.  Inside a slice's 4 KB, row r holds its 16-byte
+// piece p at position p ^ (r & 7): the loader lane that fills position
+// (r, lp) fetches global piece lp ^ (r & 7), so the global access stays inside
+// the same 128-byte segments (coalesced) and the operand-order readback
+// (lane = row l % 16) is spread over the banks without padding.
+//
+// Synchronisation is one workgroup barrier per item: a loader wavefront
+// arrives after its share of item i has landed, a compute wavefront after it
+// has finished item i-1; past the barrier the loaders refill the slot of item
+// i-1.  Every wavefront executes the same number of barriers whatever its
+// role, the tile count or the slice count.
+//
+// Order of issue.  The first byte of a kernel arrives 2-3 us after it starts
+// and the weight stream is what bounds the kernel, so the first weight tile is
+// requested at once, between the activation rounds: x0 x1 t0 x2 (the four
+// slots), then one item per freed slot: x3 t1 t2 t3.  Loads retire in order,
+// so "item i has landed" is a wait on the number of loads issued after it; the
+// schedule and those counts are worked out at compile time (struct Sched).
+#include <type_traits>
+#include <utility>
+
+#include "qmm_gemv_common.hpp"
+
+namespace qmm {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {    // s_waitcnt vmcnt(N) only; also a compiler barrier
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+  asm volatile("" ::: "memory");
+}
+
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, unsigned char* dst, uint32_t voff,
+                                      uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, voff, soff, 0, 0);
+}
+
+// all LDS traffic of this wavefront done, then the workgroup barrier
+__device__ __forceinline__ void item_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__device__ __forceinline__ void split3(float v, float& hi, float& mid, float& lo) {
+  hi = __uint_as_float(__float_as_uint(v) & 0xFFFF0000u);
+  const float r1 = v - hi;
+  mid = __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
+  lo = r1 - mid;                              // at most 8 significant bits: exact in bf16
+}
+
+__device__ __forceinline__ uint32_t hi16_pair(float a, float b) {      // (bf16(a), bf16(b)), truncating
+  return byte_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+
+// The static schedule of one pass: XR activation rounds (items 0 .. XR-1) and
+// TMAX weight tiles (items XR ..), consumed in that order, issued in the order
+// x0 x1 t0 x2 .. t1 ..; LX / LT loads per loader wavefront per item.
+template <int XR, int TMAX, int LX, int LT>
+struct Sched {
+  static constexpr int NI = XR + TMAX;
+  static constexpr int B = NI < 4 ? NI : 4;                 // ring slots = items issued up front
+  static constexpr int item_at(int j) {                     // the item issued j-th
+    if (j < 2) return j;
+    if (j == 2) return XR;
+    if (j < XR + 1) return j - 1;
+    return j;
+  }
+  static constexpr int pos(int item) {
+    for (int j = 0; j < NI; ++j)
+      if (item_at(j) == item) return j;
+    return -1;
+  }
+  static constexpr int loads(int item) { return item < XR ? LX : LT; }
+  // the issue at position j >= B happens after barrier j-B+1 and takes the slot of item j-B
+  static constexpr int slot_at(int j) { return j < B ? j : slot_at(pos(j - B)); }
+  static constexpr int slot(int item) { return slot_at(pos(item)); }
+  // loads that may still be outstanding when item k is declared landed
+  static constexpr int allowed(int k) {
+    int issued = B + (k >= 1 ? k - 1 : 0);
+    if (issued > NI) issued = NI;
+    int n = 0;
+    for (int j = pos(k) + 1; j < issued; ++j) n += loads(item_at(j));
+    return n > 63 ? 63 : n;
+  }
+};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int BITS, int CW, int NL, int TMAX, int GSHIFT>
+__global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, int rows_per_wg) {
+  constexpr int KS = 2048 / BITS;                 // codes per slice: 512 | 256
+  constexpr int CPS = KS / 64;                    // 64-code chunks per slice: 8 | 4
+  constexpr int XR = KS / 128;                    // activation rounds per slice: 4 | 2
+  constexpr int NI = XR + TMAX;                   // items per pass
+  constexpr int kItem = CW * 4096;
+  constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;   // scale rows | bias rows of one tile
+  constexpr int kTab = 2 * kTabKind;
+  constexpr int NTAB = 2 * (CW >= 4 ? CW / 4 : 1);      // table load instructions per tile
+  static_assert((CW * 4) % NL == 0 && NTAB % NL == 0, "loader shares must be whole");
+  constexpr int QI = CW * 4 / NL;                 // code / activation loads per loader wavefront per item
+  constexpr int QT = NTAB / NL;                   // table loads per loader wavefront per tile
+  constexpr int LX = QI, LT = QI + QT;            // loads per loader wavefront: activation item | tile item
+  typedef Sched<XR, TMAX, LX, LT> S;
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* ring = smem;
+  unsigned char* tabs = smem + S::B * kItem;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t bz = blockIdx.y;
+  const int64_t n_begin = (int64_t)blockIdx.x * rows_per_wg;
+  const int64_t n_end = n_begin + rows_per_wg < a.N ? n_begin + rows_per_wg : a.N;
+  const int ntiles = (int)((n_end - n_begin + 15) / 16);        // uniform, <= TMAX
+  const int64_t wpr = (int64_t)a.K * BITS / 8;                  // bytes per weight row
+  const int64_t ng = (int64_t)(a.K / 64) >> GSHIFT;             // table entries per row
+  const int slices = a.K / KS;
+  const int passes = (slices + CW - 1) / CW;
+
+  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+
+  f32x4 acc[TMAX];
+#pragma unroll
+  for (int t = 0; t < TMAX; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (wave >= CW) {
+    // ------------------------------------------------------------ loaders ----
+    const int lw = wave - CW;
+    const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+    const auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
+    const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * 2, a.N * ng * 2);
+    const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * 2, a.N * ng * 2);
+    const int lrow = lane >> 4, lp = lane & 15;
+    // Load q of this wavefront is instruction j = lw + q*NL of the item: slice
+    // j / 4, row quad j % 4 = (lw + o) % 4 with o = q*NL % 4 known at compile
+    // time, so the lane offsets are kept per o.
+    uint32_t wv[4], xv[4];
+    int wrow[4];
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      const int rq = (lw + o) & 3;
+      const int row = 4 * rq + lrow;
+      const uint32_t gp = (uint32_t)(lp ^ (row & 7));
+      wrow[o] = row;
+      wv[o] = (uint32_t)((n_begin + row) * wpr) + gp * 16;
+      xv[o] = row < a.M ? (uint32_t)((int64_t)row * a.K * 2) + gp * 16 : kOutOfRange;
+    }
+    const int trow = lane & 15, tsl = lane >> 4;  // table loads: lane = (slice within four, row)
+
+    // item `i` (compile-time kind) of pass `p` into ring slot `slot`
+    auto issue_item = [&](int p, auto ic, int slot) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      unsigned char* base = ring + slot * kItem;
+      static_for<QI>([&](auto qc) __attribute__((always_inline)) {
+        constexpr int q = decltype(qc)::value;
+        constexpr int o = (q * NL) & 3;
+        const int j = lw + q * NL;                // uniform
+        const int sloc = j >> 2, rq = j & 3;
+        const int sl = p * CW + sloc;
+        const bool ok = sl < slices;              // also false for passes past the last
+        unsigned char* dst = base + sloc * 4096 + rq * 1024;
+        if constexpr (i < XR) {
+          const uint32_t so = ok ? (uint32_t)(sl * KS + i * 128) * 2u : 0u;
+          dma16(rx, dst, ok ? xv[o] : kOutOfRange, so);
+        } else {
+          constexpr int t = i - XR;
+          const bool rok = ok && n_begin + t * 16 + wrow[o] < n_end;
+          const uint32_t so = ok ? (uint32_t)sl * 256u + (uint32_t)(t * 16 * wpr) : 0u;
+          dma16(rw, dst, rok ? wv[o] : kOutOfRange, so);
+        }
+      });
+      if constexpr (i >= XR) {
+        constexpr int t = i - XR;
+        unsigned char* tb = tabs + slot * kTab;
+#pragma unroll
+        for (int q = 0; q < QT; ++q) {
+          const int jt = lw + q * NL;             // uniform
+          const int kind = jt / (NTAB / 2), h = jt % (NTAB / 2);
+          const int sloc = 4 * h + tsl;
+          const int sl = p * CW + sloc;
+          const int64_t n = n_begin + t * 16 + trow;
+          const bool ok = sloc < CW && sl < slices && n < n_end;
+          const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> GSHIFT) * 2u : kOutOfRange;
+          dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
+        }
+      }
+    };
+    // The K slices of tile t meet here: after the barrier that follows the
+    // tile's consumption the loaders (otherwise idle) add up the compute
+    // wavefronts' partial sums and store the 16 x 16 results, under the next
+    // item's arithmetic.  Lane l, component e of an accumulator is output row
+    // 4*(l/16) + e, column l % 16 of the tile.
+    auto reduce_tile = [&](int p, auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;
+      if (p != passes - 1 || t >= ntiles) return;
+      const float* part = reinterpret_cast<const float*>(ring + S::slot(XR + t) * kItem);
+#pragma unroll
+      for (int e = lw; e < 4; e += NL) {
+        float v = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < CW; ++wv) v += part[wv * 1024 + e * kWave + lane];
+        const int m = 4 * (lane >> 4) + e;
+        const int64_t n = n_begin + t * 16 + (lane & 15);
+        if (m < a.M && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+      }
+    };
+    for (int p = 0; p < passes; ++p) {
+      static_for<S::B>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value;
+        issue_item(p, std::integral_constant<int, S::item_at(j)>{}, S::slot_at(j));
+      });
+      static_for<NI>([&](auto kc) __attribute__((always_inline)) {
+        constexpr int k = decltype(kc)::value;
+        wait_vmcnt<S::allowed(k)>();              // item k has landed
+        item_barrier();
+        constexpr int j = S::B + k - 1;           // the slot of item k-1 is free now
+        if constexpr (k >= 1 && j < NI)
+          issue_item(p, std::integral_constant<int, S::item_at(j)>{}, S::slot_at(j));
+        if constexpr (k >= XR + 1) reduce_tile(p, std::integral_constant<int, k - 1 - XR>{});
+      });
+      item_barrier();                             // the pass is consumed: its slots may be refilled
+      reduce_tile(p, std::integral_constant<int, TMAX - 1>{});
+    }
+  } else {
+    // ----------------------------------------------------- compute wavefronts
+    const int r = lane & 15, kg = lane >> 4;
+    const uint32_t swz = (uint32_t)(r & 7);
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t one = pin_vgpr(kOnesBf16x2);
+    const bf16x8 ones = as_bf16x8(one, one, one, one);
+    const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
+    const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
+    for (int p = 0; p < passes; ++p) {
+      const bool active = p * CW + wave < slices;               // uniform
+      bf16x8 xa[CPS][2];
+      bf16x8 axh, axm, axo;
+      auto consume = [&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        item_barrier();
+        const unsigned char* base = ring + S::slot(i) * kItem + rowb;
+        if constexpr (i < XR) {
+          // activations of chunks 2i, 2i+1 into operand layout
+          if (active) {
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+              for (int j = 0; j < 2; ++j) {
+                const uint32_t pc = (uint32_t)(cc * 8 + kg * 2 + j);
+                const u32x4 v = *reinterpret_cast<const u32x4*>(base + ((pc ^ swz) << 4));
+                if constexpr (BITS == 4) xa[i * 2 + cc][j] = pair_stride4(v);
+                else xa[i * 2 + cc][j] = __builtin_bit_cast(bf16x8, v);
+              }
+          }
+          if constexpr (i == XR - 1) {
+            // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
+            // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
+            if (active) {
+              float xh[8], xm[8], xo[8];
+#pragma unroll
+              for (int c = 0; c < 8; ++c) {
+                float xs = 0.f;
+                if (c < CPS) {
+                  f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
+                  t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
+                  xs = kg == 0 ? t4[0] : 0.f;
+                }
+                split3(xs, xh[c], xm[c], xo[c]);
+              }
+              axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
+              axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
+              axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
+            }
+          }
+        } else {
+          constexpr int t = i - XR;
+          if (active && t < ntiles) {
+            const unsigned char* tb = tabs + S::slot(i) * kTab + wave * 256 + r * 16;
+            u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
+            u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
+            if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
+              svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
+                          byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
+              bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
+                          byte_perm(bvt[1], bvt[1], 0x01000100u), byte_perm(bvt[1], bvt[1], 0x03020302u)};
+            }
+            const bf16x8 bop = __builtin_bit_cast(bf16x8, bvt);
+            f32x4 accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, bop, acc[t], 0, 0, 0);
+            accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, bop, accb, 0, 0, 0);
+            accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, bop, accb, 0, 0, 0);
+            f32x4 accs = zero;
+            if constexpr (BITS == 4) {
+              const bf16x8 sop = __builtin_bit_cast(bf16x8, svt);
+              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, sop, zero, 0, 0, 0);
+              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, sop, accs, 0, 0, 0);
+              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, sop, accs, 0, 0, 0);
+            }
+            f32x4 at = accb;
+#pragma unroll
+            for (int c = 0; c < CPS; ++c) {
+              f32x4 d;
+              if constexpr (BITS == 4) {
+                const uint32_t pc = (uint32_t)(2 * c + (kg >> 1));
+                const u32x2 q = *reinterpret_cast<const u32x2*>(base + ((pc ^ swz) << 4) + (kg & 1) * 8);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int4(q[0], nib, magic), zero, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int4(q[1], nib, magic), d, 0, 0, 0);
+              } else {
+                const uint32_t pc = (uint32_t)(4 * c + kg);
+                const u32x4 q = *reinterpret_cast<const u32x4*>(base + ((pc ^ swz) << 4));
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int8(q[0], q[1]), zero, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int8(q[2], q[3]), d, 0, 0, 0);
+              }
+              const uint32_t sw = svt[c >> 1];
+              const float sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
+            }
+            if constexpr (BITS == 4) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) at[e] = fmaf(-128.f, accs[e], at[e]);
+            }
+            acc[t] = at;
+          }
+          // Last pass: this wavefront's partial sums of tile t go where its own
+          // slice of the tile was (nobody else reads that region, and a tile's
+          // slot is not refilled within a pass); the loaders add the slices up.
+          if (p == passes - 1 && t < ntiles) {
+            float* part = reinterpret_cast<float*>(ring + S::slot(i) * kItem + wave * 4096);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) part[e * kWave + lane] = acc[t][e];
+          }
+        }
+      };
+      static_for<NI>(consume);
+      item_barrier();                             // pass consumed
+    }
+  }
+}
+
+template <int BITS, int CW, int NL, int TMAX, int GSHIFT>
+void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
+  dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch);
+  constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
+  constexpr int XR = 2048 / BITS / 128;
+  const size_t lds = (size_t)(XR + TMAX < 4 ? XR + TMAX : 4) * (CW * 4096 + 2 * kTabKind);
+  auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT>;
+  static bool configured = false;                 // one flag per instantiation
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);
+}
+
+template <int BITS, int CW, int NL, int TMAX>
+void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
+  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1>(a, batch, rows_per_wg, st);
+  else launch_one<BITS, CW, NL, TMAX, 0>(a, batch, rows_per_wg, st);
+}
+
+template <int BITS>
+void launch_g(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
+  if (rows_per_wg <= 32) launch_k<BITS, 8, 4, 2>(a, batch, rows_per_wg, st);
+  else launch_k<BITS, 8, 4, 4>(a, batch, rows_per_wg, st);
+}
+
+}  // namespace
+
+// The loader-wavefront kernel pays off where a workgroup streams several
+// tiles over eight K-slices (the big decode weights); eight compute and four
+// loader wavefronts.  Smaller problems stay on the self-loading kernel, which
+// has fewer barriers.
+bool skinny2_supported(int waves, int rows_per_wg) { return waves == 8 && rows_per_wg > 16 && rows_per_wg <= 64; }
+
+void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {
+  GemvArgs a = a0;
+  a.gshift = gs == 128 ? 1 : 0;
+  if (bits == 4) launch_g<4>(a, batch, rows, st);
+  else launch_g<8>(a, batch, rows, st);
+}
+
+}  // namespace qmm

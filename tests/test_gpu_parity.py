@@ -233,6 +233,48 @@ def test_gemv_batched():
         assert O.rel_l2(y[z], O.qmm(x[z], words[z], s[z], b[z], 64, 4)) <= 2e-5
 
 
+@pytest.mark.parametrize("bits,gs,m,n,k", [
+    (4, 64, 16, 7000, 4096),     # 28 rows a workgroup: two tiles, the second ragged
+    (4, 128, 5, 9000, 4096),     # group 128, three tiles a workgroup
+    (8, 64, 3, 6001, 4096),      # eight-bit codes: 16 K-slices = two passes, N odd
+    (8, 128, 16, 12000, 2048),   # eight-bit codes, one pass
+    (4, 64, 2, 5000, 8192),      # two passes of four-bit slices
+    (4, 64, 1, 16384, 6144),     # 12 slices: the second pass is half empty
+])
+def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
+    """Shapes big enough for the decode kernel whose loader wavefronts stream
+    the operands through LDS (eight K-slices, more than one tile a workgroup):
+    several passes, ragged last tiles, both code widths and group sizes."""
+    rng = np.random.default_rng(bits * 1000 + gs + m + n)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits))
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
+def test_decode_big_weights_batched_and_gathered():
+    rng = np.random.default_rng(99)
+    e, n, k = 3, 6000, 4096
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x = O.round_bf16(rng.standard_normal((e, 4, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=64, bits=4, out_dtype=torch.float32))
+    for z in range(e):
+        assert O.rel_l2(y[z], O.qmm(x[z], words[z], s[z], b[z], 64, 4)) <= 2e-5
+    # a few (token, expert) pairs: one decode product each
+    lhs = np.array([2, 0, 1, 1, 3], dtype=np.int32)
+    rhs = np.array([1, 2, 0, 2, 1], dtype=np.int32)
+    xt = x[0]
+    xtd = bf16_dev(O.f32_to_bf16_bits(xt))
+    want = O.gather_qmm(xt[:, None, :], words, s, b, lhs, rhs)[:, 0]
+    yg = out_f32(K.gather_qmm(xtd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                              group_size=64, bits=4, out_dtype=torch.float32))
+    assert O.rel_l2(yg, want) <= 2e-5
+
+
 def test_c1_decode_gemv_full_size():
     wl = synth.make(1)
     x, w, s, b, _ = synth.to_device(wl)
