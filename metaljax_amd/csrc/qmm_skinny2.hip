@@ -391,17 +391,20 @@ void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st)
 
 template <int BITS>
 void launch_g(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  if (rows_per_wg <= 32) launch_k<BITS, 8, 4, 2>(a, batch, rows_per_wg, st);
-  else launch_k<BITS, 8, 4, 4>(a, batch, rows_per_wg, st);
+  launch_k<BITS, 8, 4, 4>(a, batch, rows_per_wg, st);
 }
 
 }  // namespace
 
-// The loader-wavefront kernel pays off where a workgroup streams several
-// tiles over eight K-slices (the big decode weights); eight compute and four
-// loader wavefronts.  Smaller problems stay on the self-loading kernel, which
-// has fewer barriers.
-bool skinny2_supported(int waves, int rows_per_wg) { return waves == 8 && rows_per_wg > 16 && rows_per_wg <= 64; }
+// The loader-wavefront kernel pays off where a workgroup streams three or
+// four tiles over exactly eight K-slices, i.e. one pass (measured: 3-5 % faster
+// on 4096 x 14336 and 4096 x 28672 four-bit weights; with two passes the ring
+// drains between them and it is 13 % slower, as it is with two tiles).  Eight
+// compute and four loader wavefronts.  Everything else stays on the
+// self-loading kernel.
+bool skinny2_supported(int64_t K, int bits, int waves, int rows_per_wg) {
+  return waves == 8 && K == 8 * (2048 / bits) && rows_per_wg > 32 && rows_per_wg <= 64;
+}
 
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {
   GemvArgs a = a0;

@@ -257,7 +257,7 @@ def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
 
 def test_decode_big_weights_batched_and_gathered():
     rng = np.random.default_rng(99)
-    e, n, k = 3, 6000, 4096
+    e, n, k = 3, 9000, 4096
     _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
     x = O.round_bf16(rng.standard_normal((e, 4, k)).astype(np.float32))
     xd = bf16_dev(O.f32_to_bf16_bits(x))
