@@ -584,6 +584,55 @@ def test_c5_moe_scaled():
     assert O.rel_l2(out_f32(y), want) <= 2e-5
 
 
+# ------------------------------------------------- checkpoint-side layouts ----
+
+def test_hf_mxfp4_checkpoint_tensors_feed_the_kernels_as_they_are():
+    """`_blocks` [E, N, K/32, 16] / `_scales` [E, N, K/32] uint8 straight from a
+    checkpoint (reference scripts/model_bench/mxfp4_gpt_oss.py:211-258): the
+    flattened blocks are the packed weight, no repack on either side."""
+    from metaljax_amd import checkpoint as CK
+    rng = np.random.default_rng(31)
+    e, n, k = 3, 96, 1024
+    codes = rng.integers(0, 16, size=(e, n, k), dtype=np.uint8)
+    blocks = (codes[..., 0::2] | (codes[..., 1::2] << 4)).astype(np.uint8).reshape(e, n, k // 32, 16)
+    sb = rng.integers(118, 132, size=(e, n, k // 32)).astype(np.uint8)
+    w, sc = CK.mxfp4_from_hf_blocks(torch.from_numpy(blocks).to(DEV), torch.from_numpy(sb).to(DEV))
+    assert tuple(w.shape) == (e, n, k // 2) and sc.dtype == torch.uint8
+    x, xd = make_x(rng, 40, k)
+    words = O.pack_codes(codes, 4)
+    # one expert as a plain product (prefill and decode), all of them as a gathered product
+    want = O.qmm(x, words[1], sb[1], None, 32, 4, "mxfp4")
+    y = out_f32(K.quantized_matmul(xd, w[1], sc[1], None, group_size=32, bits=4, mode="mxfp4",
+                                   out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= TOL_F32_OUT
+    y1 = out_f32(K.quantized_matmul(xd[:2], w[1], sc[1], None, group_size=32, bits=4, mode="mxfp4",
+                                    out_dtype=torch.float32))
+    assert O.rel_l2(y1, want[:2]) <= 2e-5
+    rhs = rng.integers(0, e, size=40).astype(np.int32)
+    wantg = O.gather_qmm(x[:, None, :], words, sb, None, np.arange(40), rhs, 32, 4, "mxfp4")[:, 0]
+    yg = out_f32(K.gather_qmm(xd, w, sc, None, None, torch.from_numpy(rhs).to(DEV), group_size=32, bits=4,
+                              mode="mxfp4", out_dtype=torch.float32))
+    assert O.rel_l2(yg, wantg) <= TOL_F32_OUT
+
+
+def test_keras_int4_kernel_repacked_once_then_multiplied():
+    from metaljax_amd import checkpoint as CK
+    rng = np.random.default_rng(32)
+    k, n = 512, 72
+    wq = rng.integers(-8, 8, size=(k, n)).astype(np.int8)
+    packed = ((wq[:, 0::2] & 15) | ((wq[:, 1::2] & 15) << 4)).astype(np.int8)
+    words, offset = CK.keras_int4_kernel_to_packed(packed, n)
+    s = O.round_bf16(rng.uniform(0.005, 0.02, (n, k // 64)).astype(np.float32))
+    z = rng.integers(-2, 3, (n, k // 64)).astype(np.float32)
+    ss, bb, kind = O.scale_bias(s, z, offset, "bf16")
+    x, xd = make_x(rng, 3, k)
+    want = x @ ((wq.T.astype(np.float32) - np.repeat(z, 64, axis=1)) * np.repeat(s, 64, axis=1)).T
+    tab = (lambda v: bf16_dev(O.f32_to_bf16_bits(v))) if kind == "bf16" else (lambda v: torch.from_numpy(v).to(DEV))
+    y = out_f32(K.quantized_matmul(xd, CK.to_device(words), tab(ss), tab(bb), group_size=64, bits=4,
+                                   out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
 # ------------------------------------------------------------ error paths ----
 
 def test_unsupported_and_bad_shapes_raise_without_launching():
