@@ -53,21 +53,26 @@ __device__ __forceinline__ int swz(int row, int piece) { return row * kRowBytes 
 
 // ---------------------------------------------------------------------------
 // x [x_rows, K] bf16 (rows optionally gathered through lhs_idx) -> ax[K/8][Rp]
-// One thread = one row's 64 bytes (4 pieces); consecutive threads = consecutive rows.
+// One thread = one 16-byte piece.  A wavefront covers 8 rows x 8 pieces, so
+// that both sides move whole 128-byte lines: 8 lanes read one row's line, and
+// the 8 rows of one piece are written as one 128-byte run.  A workgroup is
+// four such wavefronts side by side along K (512 contiguous bytes a row).
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* __restrict__ x,
                                                         const int32_t* __restrict__ lhs_idx,
                                                         u32x4* __restrict__ ax, int R, int x_rows,
                                                         int K, int Rp) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int row = (int)(idx % Rp);
-  const int chunk = (int)(idx / Rp);               // 32 elements = 4 pieces
-  if (chunk >= K / 32 || row >= R) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pieces = K / 8;
+  const int pblocks = (pieces + 31) / 32;
+  const int rb = blockIdx.x / pblocks, pb = blockIdx.x % pblocks;
+  const int row = rb * 8 + (lane >> 3);
+  const int piece = pb * 32 + wave * 8 + (lane & 7);
+  if (row >= R || piece >= pieces) return;
   const int64_t src = lhs_idx ? (int64_t)lhs_idx[row] : (int64_t)row;
   const bool ok = src >= 0 && src < x_rows;        // an index outside x gathers a zero row
-  const u32x4* p = reinterpret_cast<const u32x4*>(x + (ok ? src : 0) * K + chunk * 32);
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    ax[((int64_t)chunk * 4 + j) * Rp + row] = ok ? p[j] : u32x4{0u, 0u, 0u, 0u};
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (ok) v = reinterpret_cast<const u32x4*>(x + src * K)[piece];
+  ax[(int64_t)piece * Rp + row] = v;
 }
 
 // ---------------------------------------------------------------------------
@@ -560,8 +565,8 @@ void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, 
                     hipStream_t st) {
   if (R == 0 || N == 0) return;
   const int64_t rp = prep_rows(R);
-  const int64_t threads = rp * (K / 32);
-  hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
+  const int64_t prep_blocks = ceil_div(R, 8) * ceil_div(K / 8, 32);
+  hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)prep_blocks), dim3(256), 0, st,
                      static_cast<const uint16_t*>(x), lhs_idx, static_cast<u32x4*>(workspace),
                      (int)R, (int)x_rows, (int)K, (int)rp);
   Gemm2Args a;
