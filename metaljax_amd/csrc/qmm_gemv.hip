@@ -1,8 +1,14 @@
-// Decode-regime quantized matmul (M <= 16) for gfx950.
+// Decode-regime quantized matmul (M <= 16) for gfx950: the general kernel.
 //
 // y[m, n] = sum_k x[m, k] * w[n, k],  w = scales*q + biases (affine) or
-// E2M1[q] * 2^(e-127) (mxfp4).  The kernel is HBM-bound: every packed weight
-// byte is read exactly once with vector loads and unpacked in registers.
+// E2M1[q] * 2^(e-127) (mxfp4).  Every packed weight byte is read exactly once,
+// straight into the matrix-core operand layout, and unpacked in registers.
+// That layout makes each lane its own L1 request (lane = weight row), which
+// bounds this kernel by L1 tag lookups rather than by HBM; the common layouts
+// (group 64 / 128, bf16 tables, K a multiple of a slice) therefore run on the
+// LDS-staged kernels of qmm_skinny.hip / qmm_skinny2.hip, and this one serves
+// everything else: group 32, float32 / float16 tables, odd K, MXFP4.  The
+// dispatcher at the end of the file chooses.
 //
 // Mapping.  One workgroup owns 16*T consecutive weight rows over the whole K;
 // its WAVES wavefronts split K into contiguous slices and their partial sums
