@@ -1,0 +1,110 @@
+"""Seeded random sweep of the C ABI against the oracle: shapes, group sizes,
+code widths, table types and output types drawn at random, so that every
+kernel family and its edge handling (ragged tiles, short K, odd N, unaligned
+table pitches) is hit by inputs nobody chose by hand."""
+import numpy as np
+import pytest
+import torch
+
+from metaljax_amd import kernels as K
+from oracle import qmm_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _bf16_dev(v):
+    return torch.from_numpy(np.ascontiguousarray(O.f32_to_bf16_bits(v)).view(np.int16)).to(DEV).view(torch.bfloat16)
+
+
+def _tab_dev(v, tab):
+    if tab == "bf16":
+        return _bf16_dev(v)
+    if tab == "f16":
+        return torch.from_numpy(v.astype(np.float16)).to(DEV)
+    return torch.from_numpy(v.astype(np.float32)).to(DEV)
+
+
+def _draw_affine(rng):
+    regime = rng.choice(["decode", "prefill", "prefill_big"])
+    m = int(rng.integers(1, 17)) if regime == "decode" else int(rng.integers(17, 300 if regime == "prefill" else 700))
+    n = int(rng.integers(1, 700))
+    gs = int(rng.choice([32, 64, 128]))
+    k = gs * int(rng.integers(1, 2048 // gs + 1))
+    bits = int(rng.choice([4, 8]))
+    tab = str(rng.choice(["bf16", "bf16", "f32", "f16"]))
+    return m, n, k, gs, bits, tab
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_affine_random_case(seed):
+    rng = np.random.default_rng(7000 + seed)
+    m, n, k, gs, bits, tab = _draw_affine(rng)
+    codes = rng.integers(0, 1 << bits, size=(n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    s = rng.uniform(0.005, 0.02, (n, k // gs)).astype(np.float32)
+    b = (-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s).astype(np.float32)
+    if tab == "bf16":
+        s, b = O.round_bf16(s), O.round_bf16(b)
+    elif tab == "f16":
+        s, b = s.astype(np.float16).astype(np.float32), b.astype(np.float16).astype(np.float32)
+    x = O.round_bf16(rng.standard_normal((m, k)).astype(np.float32))
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    y = K.quantized_matmul(_bf16_dev(x), wd, _tab_dev(s, tab), _tab_dev(b, tab), group_size=gs, bits=bits,
+                           out_dtype=torch.float32).float().cpu().numpy()
+    rounding = "f32" if m <= 16 else "bf16"          # prefill stages a bf16 weight tile
+    want = O.qmm(x, words, s, b, gs, bits, weight_rounding=rounding)
+    err = O.rel_l2(y, want)
+    assert err <= 2e-5, (m, n, k, gs, bits, tab, err)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_mxfp4_random_case(seed):
+    rng = np.random.default_rng(9000 + seed)
+    m = int(rng.choice([int(rng.integers(1, 17)), int(rng.integers(17, 400))]))
+    n = int(rng.integers(1, 500))
+    k = 32 * int(rng.integers(1, 65))
+    codes = rng.integers(0, 16, size=(n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, 4)
+    sb = rng.integers(112, 140, size=(n, k // 32)).astype(np.uint8)
+    x = O.round_bf16(rng.standard_normal((m, k)).astype(np.float32))
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    y = K.quantized_matmul(_bf16_dev(x), wd, torch.from_numpy(sb).to(DEV), None, group_size=32, bits=4,
+                           mode="mxfp4", out_dtype=torch.float32).float().cpu().numpy()
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    # K % 512 == 0 and M > 16 runs on the block-scaled matrix cores (two FP6 activation terms)
+    tol = 1e-3 if (m > 16 and k % 512 == 0) else 2e-5
+    err = O.rel_l2(y, want)
+    assert err <= tol, (m, n, k, err)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_and_gathered_random_case(seed):
+    rng = np.random.default_rng(11000 + seed)
+    e = int(rng.integers(1, 7))
+    n = int(rng.integers(8, 300))
+    gs = int(rng.choice([32, 64, 128]))
+    k = gs * int(rng.integers(1, 1024 // gs + 1))
+    bits = int(rng.choice([4, 8]))
+    sizes = rng.integers(0, 200, size=e)
+    sizes[rng.integers(0, e)] += 70                   # never all empty; total well past the decode regime
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    codes = rng.integers(0, 1 << bits, size=(e, n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    s = O.round_bf16(rng.uniform(0.005, 0.02, (e, n, k // gs)).astype(np.float32))
+    b = O.round_bf16(-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s)
+    x = O.round_bf16(rng.standard_normal((r, k)).astype(np.float32))
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    sd, bd, xd = _bf16_dev(s), _bf16_dev(b), _bf16_dev(x)
+    want = O.grouped_qmm(x, words, s, b, ro, gs, bits, weight_rounding="bf16")
+    y = K.grouped_qmm(xd, wd, sd, bd, torch.from_numpy(ro).to(DEV), group_size=gs, bits=bits,
+                      out_dtype=torch.float32).float().cpu().numpy()
+    assert O.rel_l2(y, want) <= 2e-5, (e, n, k, gs, bits, sizes, O.rel_l2(y, want))
+    # the same rows as shuffled (row, expert) pairs
+    rhs = np.repeat(np.arange(e), sizes).astype(np.int32)
+    perm = rng.permutation(r)
+    yg = K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(perm.astype(np.int32)).to(DEV),
+                      torch.from_numpy(rhs[perm]).to(DEV), group_size=gs, bits=bits,
+                      out_dtype=torch.float32).float().cpu().numpy()
+    assert O.rel_l2(yg, want[perm]) <= 2e-5, (e, n, k, gs, bits, O.rel_l2(yg, want[perm]))
