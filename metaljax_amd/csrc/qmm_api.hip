@@ -30,7 +30,9 @@ bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K);
 size_t mxfp4_workspace_bytes(int64_t R, int64_t K);
 void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block);
 void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, int y_dtype,
-                         int64_t R, int64_t N, int64_t K, void* workspace, hipStream_t st);
+                         const int32_t* row_offsets, const int32_t* lhs_idx,
+                         const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
+                         int64_t K, void* workspace, hipStream_t st);
 void unpack_dispatch(const void* w, void* codes, int64_t rows, int64_t K, int bits, hipStream_t st);
 void pack_dispatch(const void* codes, void* w, int64_t rows, int64_t K, int bits, hipStream_t st);
 void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void* out,
@@ -168,7 +170,10 @@ size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K) {
   if (P <= kGatherGemvMaxPairs) return 0;
   // the expert sort's arrays, then (when the register-operand kernel serves
   // the shape) the re-laid copy of the gathered activation rows
-  return route_bytes(P, E) + (gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0);
+  size_t relaid = gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0;
+  if (mxfp4_mfma_supported(P, N, K) && mxfp4_workspace_bytes(P, K) > relaid)
+    relaid = mxfp4_workspace_bytes(P, K);          // the mode is not known here: the larger of the two
+  return route_bytes(P, E) + relaid;
 }
 
 int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode, int* kernel,
@@ -244,7 +249,8 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
       mxfp4_mfma_dispatch(static_cast<const char*>(x) + z * M * K * 2,
                           static_cast<const uint32_t*>(w) + z * N * wpr,
                           static_cast<const char*>(scales) + z * N * ng,
-                          static_cast<char*>(y) + z * M * N * ysz, y_dtype, M, N, K, workspace, st);
+                          static_cast<char*>(y) + z * M * N * ysz, y_dtype, nullptr, nullptr,
+                          nullptr, M, M, 1, N, K, workspace, st);
       rc = check_launch("mxfp4 launch");
       if (rc) return rc;
     }
@@ -297,6 +303,13 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   if (rc) return rc;
   if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535 || R * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(R, N, K) && workspace &&
+      workspace_bytes >= mxfp4_workspace_bytes(R, K) && aligned16(workspace) && aligned16(scales)) {
+    // MXFP4 experts on the block-scaled matrix cores
+    mxfp4_mfma_dispatch(x, w, scales, y, y_dtype, row_offsets, nullptr, nullptr, R, R, E, N, K,
+                        workspace, static_cast<hipStream_t>(stream));
+    return check_launch("grouped mxfp4 launch");
+  }
   if (gemm2_supported(R, N, K) && workspace && workspace_bytes >= gemm2_workspace_bytes(R, K) &&
       aligned16(workspace)) {
     gemm2_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, row_offsets, nullptr, nullptr, R,
@@ -342,6 +355,13 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
                      ro, cursor, src_row, out_row);
   rc = check_launch("route launch");
   if (rc) return rc;
+  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(P, N, K) &&
+      workspace_bytes >= need + mxfp4_workspace_bytes(P, K) && aligned16(workspace) &&
+      aligned16(scales)) {
+    mxfp4_mfma_dispatch(x, w, scales, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
+                        static_cast<char*>(workspace) + need, st);
+    return check_launch("gather mxfp4 launch");
+  }
   if (gemm2_supported(P, N, K) && workspace_bytes >= need + gemm2_workspace_bytes(P, K) &&
       aligned16(workspace)) {
     // rows gathered in expert order into the re-laid copy, results scattered back to pair order

@@ -89,21 +89,25 @@ __device__ __forceinline__ uint32_t block_scale_byte(uint32_t e) {
 }
 
 // ---------------------------------------------------------------------------
-// x [R, K] bf16 -> two FP6 terms + scales in matrix-core operand order.
+// x [x_rows, K] bf16 (rows optionally gathered through lhs_idx) -> two FP6
+// terms + scales in matrix-core operand order.
 // One thread = one (row, 32-block); consecutive threads = consecutive rows.
 __global__ __launch_bounds__(256) void mx_split_kernel(const uint16_t* __restrict__ x,
+                                                       const int32_t* __restrict__ lhs_idx,
                                                        u32x4* __restrict__ aq,
-                                                       uint8_t* __restrict__ as, int R, int K,
-                                                       int Rp) {
+                                                       uint8_t* __restrict__ as, int R, int x_rows,
+                                                       int K, int Rp) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int row = (int)(idx % Rp);
   const int blk = (int)(idx / Rp);
   if (blk >= K / 32 || row >= R) return;
-  const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)row * K + blk * 32);
+  const int64_t srow = lhs_idx ? (int64_t)lhs_idx[row] : (int64_t)row;
+  const bool ok = srow >= 0 && srow < x_rows;      // an index outside x gathers a zero row
+  const u32x4* src = reinterpret_cast<const u32x4*>(x + (ok ? srow : 0) * K + blk * 32);
   u32x16 raw;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const u32x4 v = src[i];
+    const u32x4 v = ok ? src[i] : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int j = 0; j < 4; ++j) raw[4 * i + j] = v[j];
   }
@@ -153,10 +157,20 @@ struct MxArgs {
   const void* w;         // uint8 [N, K/2]
   const void* s;         // uint8 [N, K/32]
   void* y;               // [R, N]
-  int R, N, K, Rp;
+  const int32_t* row_offsets;   // [E+1] or null: rows [o[e], o[e+1]) use expert e's weight
+  const int32_t* out_idx;       // optional row scatter for y
+  int R, N, K, Rp, E;
   int y_dtype;
-  int m_tiles, n_tiles;
+  int m_tiles, n_tiles;  // provisioned row tiles (>= the tiles that exist when grouped)
 };
+
+// Rows [lo, hi) of expert i, forced into [0, R] and hi >= lo whatever the offsets hold.
+__device__ __forceinline__ void mx_group_rows(const MxArgs& a, int i, int& lo, int& hi) {
+  lo = a.row_offsets[i];
+  hi = a.row_offsets[i + 1];
+  lo = lo < 0 ? 0 : (lo > a.R ? a.R : lo);
+  hi = hi < lo ? lo : (hi > a.R ? a.R : hi);
+}
 
 // The two FP6 terms of a lane's 48 bytes (three 16-byte planes, hi | lo).
 __device__ __forceinline__ i32x8 fp6_term(const u32x4 (&p)[3], int term) {
@@ -177,11 +191,36 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   // Workgroups are dealt to the 8 XCDs round-robin in launch order; XCD x is
   // handed a contiguous run of tiles, row-tile fastest, so the workgroups that
   // share one L2 share weight column tiles.
-  const int total = a.m_tiles * a.n_tiles;
+  // Grouped: the grid is provisioned for the worst raggedness; the row tiles
+  // that exist are counted first and only those are dealt; a tile never
+  // straddles two experts.
+  int m_tiles = a.m_tiles;
+  if (a.row_offsets) {
+    m_tiles = 0;
+    for (int i = 0; i < a.E; ++i) {
+      int lo, hi;
+      mx_group_rows(a, i, lo, hi);
+      m_tiles += (hi - lo + TM - 1) / TM;
+    }
+  }
+  const int total = m_tiles * a.n_tiles;
   const int per = (total + 7) / 8;
   const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  if (tile >= total) return;
-  const int m0 = (tile % a.m_tiles) * TM, n0 = (tile / a.m_tiles) * TN;
+  if ((int)(blockIdx.x >> 3) >= per || tile >= total) return;
+  int e = 0, row_hi = a.R, m0 = (tile % m_tiles) * TM;
+  const int n0 = (tile / m_tiles) * TN;
+  if (a.row_offsets) {
+    int t = tile % m_tiles;
+    bool found = false;
+    for (int i = 0; i < a.E; ++i) {
+      int lo, hi;
+      mx_group_rows(a, i, lo, hi);
+      const int tiles = (hi - lo + TM - 1) / TM;
+      if (t < tiles) { e = i; m0 = lo + t * TM; row_hi = hi; found = true; break; }
+      t -= tiles;
+    }
+    if (!found) return;
+  }
 
   const int nquads = a.K / 512;
   const int nq = nquads > wave ? (nquads - wave + 3) / 4 : 0;       // this wavefront's quads
@@ -192,8 +231,8 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   };
 
   const int64_t wpitch = a.K / 2, spitch = a.K / 32;
-  const auto rw = make_rsrc(a.w, (int64_t)a.N * wpitch);
-  const auto rs = make_rsrc(a.s, (int64_t)a.N * spitch);
+  const auto rw = make_rsrc(static_cast<const char*>(a.w) + (int64_t)e * a.N * wpitch, (int64_t)a.N * wpitch);
+  const auto rs = make_rsrc(static_cast<const char*>(a.s) + (int64_t)e * a.N * spitch, (int64_t)a.N * spitch);
   const auto ra = make_rsrc(a.aq, (int64_t)(a.K / 128) * 192 * a.Rp);
   const auto rsa = make_rsrc(a.as, (int64_t)nquads * 32 * a.Rp);
 
@@ -419,9 +458,11 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
     for (int q = 0; q < 4; ++q) {
       const int idx = q * 64 + lane, rl = idx >> 3, pc = idx & 7;
       const int row = m0 + 32 * mt + rl, col = n0 + 64 * nh + pc * 8;
-      if (row < a.R && col < a.N)
-        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + (int64_t)row * a.N + col) =
+      if (row < row_hi && col < a.N) {
+        const int64_t orow = a.out_idx ? (int64_t)a.out_idx[row] : (int64_t)row;
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + col) =
             *reinterpret_cast<const u32x4*>(o16 + rl * 64 + pc * 8);
+      }
     }
   } else {
 #pragma unroll
@@ -429,7 +470,10 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + 32 * mt + 8 * (r >> 2) + 4 * kh + (r & 3), col = n0 + 32 * (2 * nh + h) + li;
-        if (row < a.R && col < a.N) store_out(a.y, (int64_t)row * a.N + col, v[h][r], a.y_dtype);
+        if (row < row_hi && col < a.N) {
+          const int64_t orow = a.out_idx ? (int64_t)a.out_idx[row] : (int64_t)row;
+          store_out(a.y, orow * a.N + col, v[h][r], a.y_dtype);
+        }
       }
   }
 }
@@ -437,7 +481,8 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
 }  // namespace
 
 // Rows of the split-activation workspace (row count rounded up to the tile).
-static int64_t mx_rows(int64_t R) { return ceil_div(R, TM) * TM; }
+// (a tile of a row group may start at any row, so a full tile past the last row is provisioned)
+static int64_t mx_rows(int64_t R) { return ceil_div(R + TM, TM) * TM; }
 
 bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K) {
   if (getenv("QMM_NO_MXFP4_MFMA")) return false;
@@ -456,25 +501,29 @@ void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block) {
   *block = 256;
 }
 
-// x bf16 [R, K]; w uint8 [N, K/2]; s uint8 [N, K/32]; y [R, N]; workspace as sized above.
+// x bf16 [x_rows, K] (rows gathered through lhs_idx when given); w uint8 [E, N, K/2];
+// s uint8 [E, N, K/32]; y [R, N] (rows scattered through out_idx when given);
+// row_offsets [E+1] or null (one weight); workspace as sized above.
 void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, int y_dtype,
-                         int64_t R, int64_t N, int64_t K, void* workspace, hipStream_t st) {
+                         const int32_t* row_offsets, const int32_t* lhs_idx,
+                         const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
+                         int64_t K, void* workspace, hipStream_t st) {
   const int64_t rp = mx_rows(R);
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   void* aq = ws;
   void* as = ws + rp * K * 3 / 2;
   const int64_t threads = rp * (K / 32);
   hipLaunchKernelGGL(mx_split_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t*>(x), static_cast<u32x4*>(aq),
-                     static_cast<uint8_t*>(as), (int)R, (int)K, (int)rp);
+                     static_cast<const uint16_t*>(x), lhs_idx, static_cast<u32x4*>(aq),
+                     static_cast<uint8_t*>(as), (int)R, (int)x_rows, (int)K, (int)rp);
   MxArgs a;
   a.aq = aq; a.as = as; a.w = w; a.s = s; a.y = y;
-  a.R = (int)R; a.N = (int)N; a.K = (int)K; a.Rp = (int)rp;
+  a.row_offsets = row_offsets; a.out_idx = out_idx;
+  a.R = (int)R; a.N = (int)N; a.K = (int)K; a.Rp = (int)rp; a.E = (int)E;
   a.y_dtype = y_dtype;
-  a.m_tiles = (int)ceil_div(R, TM);
+  a.m_tiles = (int)(ceil_div(R, TM) + (row_offsets ? E : 0));
   a.n_tiles = (int)ceil_div(N, TN);
-  int grid, block;
-  mxfp4_geometry(R, N, &grid, &block);
+  const int grid = (int)(ceil_div((int64_t)a.m_tiles * a.n_tiles, 8) * 8), block = 256;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mxfp4_mfma_kernel),

@@ -517,7 +517,9 @@ def test_gather_qmm_many_pairs_skewed_experts(bits, mode):
     y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV),
                              torch.from_numpy(rhs).to(DEV), group_size=gs, bits=bits, mode=mode,
                              out_dtype=torch.float32))
-    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+    # MXFP4 at K % 512 == 0 runs on the block-scaled matrix cores (two FP6 activation terms)
+    tol = TOL_F32_OUT if mode == "mxfp4" else 2e-5
+    assert O.rel_l2(y, want) <= tol, O.rel_l2(y, want)
     # bf16 results, identity lhs (pair p reads row p)
     want2 = O.gather_qmm(x[:, None, :], words, s, b, np.arange(t), rhs[:t], gs, bits, mode,
                          weight_rounding="bf16")[:, 0]
@@ -573,6 +575,37 @@ def test_gather_qmm_with_only_the_sort_workspace_still_runs():
                             _dt(torch.float32), None, _ptr(rd), t, t, e, n, k, 64, 4, 0, _ptr(ws),
                             small - 256, _stream(xd))
     assert rc == 4 and _lib.ERR_NAMES[rc] == "WORKSPACE"
+
+
+@pytest.mark.parametrize("k", [1024, 768])
+def test_grouped_and_gathered_mxfp4_experts(k):
+    """MXFP4 experts (the gpt-oss layout): K % 512 == 0 runs the expert products
+    on the block-scaled matrix cores (tiles never straddle an expert, empty and
+    ragged experts, rows gathered and scattered), other K on the bf16 kernel."""
+    rng = np.random.default_rng(k)
+    e, n = 5, 200
+    _, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+    sizes = np.array([70, 0, 129, 3, 64])
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    x, xd = make_x(rng, r, k)
+    want = O.grouped_qmm(x, words, sb, None, ro, 32, 4, "mxfp4")
+    tol = TOL_F32_OUT if k % 512 == 0 else 2e-5
+    y = out_f32(K.grouped_qmm(xd, wd, sd, None, torch.from_numpy(ro).to(DEV), group_size=32, bits=4,
+                              mode="mxfp4", out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= tol, O.rel_l2(y, want)
+    for a, b in zip(ro[:-1], ro[1:]):                       # every expert's rows on their own
+        if b > a:
+            assert O.rel_l2(y[a:b], want[a:b]) <= tol
+    y16 = out_f32(K.grouped_qmm(xd, wd, sd, None, torch.from_numpy(ro).to(DEV), group_size=32, bits=4,
+                                mode="mxfp4"))
+    assert O.rel_l2(y16, want) <= TOL_BF16_OUT
+    rhs = np.repeat(np.arange(e), sizes).astype(np.int32)
+    perm = rng.permutation(r)
+    yg = out_f32(K.gather_qmm(xd, wd, sd, None, torch.from_numpy(perm.astype(np.int32)).to(DEV),
+                              torch.from_numpy(rhs[perm]).to(DEV), group_size=32, bits=4, mode="mxfp4",
+                              out_dtype=torch.float32))
+    assert O.rel_l2(yg, want[perm]) <= tol, O.rel_l2(yg, want[perm])
 
 
 def test_c5_moe_scaled():
