@@ -4,22 +4,122 @@ execute it on buffers (reference src/metaljax/engine.py:325, :385).
 Only what the quantized-matmul path needs is here: `compile_program` parses
 the module text, `execute` runs the packing prologue and then the program.
 The PJRT plugin, buffer donation/aliasing and the trace cache of the reference
-engine are outside this package.
+engine are outside this package; the entry points a PJRT plugin calls by name
+(`buffer_from_host`, `buffer_to_host`, `buffer_pointer`, `device_kind`,
+`stablehlo_version`; reference src/metaljax/engine.py:133-159, :549-591) are
+kept as a thin surface over host arrays and device tensors.
 """
 
 from __future__ import annotations
 
+import hashlib
+
+import numpy as np
+
 from . import qmm
-from .interpreter import Interpreter, host
+from .interpreter import HostArray, Interpreter, from_numpy, host
+
+# PJRT_Buffer_Type enumerators, in the order of the PJRT C API
+PJRT_TYPES = [
+    "INVALID", "PRED", "S8", "S16", "S32", "S64", "U8", "U16", "U32", "U64",
+    "F16", "F32", "F64", "BF16", "C64", "C128",
+    "F8E5M2", "F8E4M3FN", "F8E4M3B11FNUZ", "F8E5M2FNUZ", "F8E4M3FNUZ",
+    "S4", "U4", "TOKEN", "S2", "U2", "F8E4M3", "F8E3M4", "F8E8M0FNU",
+    "F4E2M1FN", "S1", "U1", "F6E2M3FN", "F6E3M2FN",
+]
+_ENUM = {name: i for i, name in enumerate(PJRT_TYPES)}
+# enumerator -> (StableHLO element type, numpy dtype of the host bytes)
+_ENUM_EL = {
+    _ENUM["PRED"]: ("i1", np.bool_), _ENUM["S8"]: ("i8", np.int8), _ENUM["S16"]: ("i16", np.int16),
+    _ENUM["S32"]: ("i32", np.int32), _ENUM["S64"]: ("i64", np.int64), _ENUM["U8"]: ("ui8", np.uint8),
+    _ENUM["U16"]: ("ui16", np.uint16), _ENUM["U32"]: ("ui32", np.uint32),
+    _ENUM["U64"]: ("ui64", np.uint64), _ENUM["F16"]: ("f16", np.float16),
+    _ENUM["F32"]: ("f32", np.float32), _ENUM["F64"]: ("f64", np.float64),
+    _ENUM["BF16"]: ("bf16", np.uint16),          # host bytes are the 16-bit patterns
+}
+_EL_ENUM = {el: k for k, (el, _) in _ENUM_EL.items()}
+
+
+class Buffer:
+    """A runtime value plus the metadata a PJRT plugin reads: `data` (a host
+    array or a device tensor), `type_enum`, `dims`, `nbytes`."""
+
+    __slots__ = ("data", "type_enum", "dims", "nbytes")
+
+    def __init__(self, data, type_enum: int, dims):
+        self.data = data
+        self.type_enum = int(type_enum)
+        self.dims = [int(d) for d in dims]
+        n = 1
+        for d in self.dims:
+            n *= d
+        self.nbytes = n * np.dtype(_ENUM_EL[self.type_enum][1]).itemsize
+
+
+def buffer_from_host(data, type_enum: int, dims, byte_strides=None, offset: int = 0) -> Buffer:
+    """Host bytes (any buffer-protocol object, or None for zeros) -> Buffer.
+    `byte_strides` / `offset` describe a strided view of `data`, as PJRT's
+    BufferFromHostBuffer hands it over."""
+    dims = [int(d) for d in dims]
+    if type_enum not in _ENUM_EL:
+        name = PJRT_TYPES[type_enum] if 0 <= type_enum < len(PJRT_TYPES) else type_enum
+        raise TypeError(f"Unsupported PJRT buffer type {name}")
+    el, dt = _ENUM_EL[type_enum]
+    if data is None:
+        arr = np.zeros(dims, dt)
+    elif byte_strides is None:
+        arr = np.frombuffer(data, dt).reshape(dims)
+    else:
+        arr = np.ndarray(shape=dims, dtype=dt, buffer=data, offset=offset, strides=list(byte_strides))
+        arr = np.ascontiguousarray(arr).reshape(dims)
+    if el == "bf16":
+        arr = (arr.astype(np.uint32) << 16).view(np.float32)      # held as float32 values
+    return Buffer(from_numpy(arr, el), type_enum, dims)
+
+
+def buffer_to_host(buf) -> bytes:
+    """The bytes of a Buffer (or of any runtime value) in its element type."""
+    h = host(buf.data if isinstance(buf, Buffer) else buf)
+    if h.el == "bf16":
+        from .packing import f32_to_bf16_bits
+        return f32_to_bf16_bits(np.ascontiguousarray(h.a, np.float32)).tobytes()
+    return np.ascontiguousarray(h.a).tobytes()
+
+
+def buffer_pointer(buf) -> int:
+    """Address of the value's storage: the device pointer of a tensor, the
+    host address of a host array (stable while the Buffer is alive)."""
+    v = buf.data if isinstance(buf, Buffer) else buf
+    if isinstance(v, HostArray):
+        return int(v.a.ctypes.data)
+    return int(v.data_ptr())
+
+
+def device_kind() -> str:
+    try:
+        import torch
+        if torch.cuda.is_available():
+            return torch.cuda.get_device_name(0)
+    except Exception:
+        pass
+    return "AMD GPU (none visible)"
+
+
+def stablehlo_version() -> list:
+    """The StableHLO text forms `ir.parse_module` reads are those of the 1.x
+    pretty printer; there is no MLIR library to ask."""
+    return [1, 0, 0]
 
 
 class Executable:
-    def __init__(self, interp, name="main"):
+    def __init__(self, interp, name="main", fingerprint=""):
         self.interp = interp
         self.name = name
+        self.fingerprint = fingerprint
         self.num_params = len(interp.main.body.args)
         self.num_outputs = len(interp.main.result_types)
         self.out_types = [t.el for t in interp.main.result_types]
+        self.out_type_enums = [_EL_ENUM.get(t.el, 0) for t in interp.main.result_types]
         self.out_dims = [list(t.shape) for t in interp.main.result_types]
         self.donated_params = sorted(interp.donated_args)
         self.generation = 0                 # bumped whenever the rewrite set changes
@@ -33,9 +133,8 @@ def compile_program(code, fmt="mlir", options=None) -> Executable:
     """`code`: StableHLO module text (str or UTF-8 bytes)."""
     if fmt not in ("mlir", "stablehlo"):
         raise ValueError(f"Unsupported program format {fmt!r}: module text only")
-    if isinstance(code, (bytes, bytearray)):
-        code = bytes(code).decode("utf-8")
-    return Executable(Interpreter(code))
+    raw = bytes(code) if isinstance(code, (bytes, bytearray)) else code.encode("utf-8")
+    return Executable(Interpreter(raw.decode("utf-8")), fingerprint=hashlib.sha256(raw).hexdigest())
 
 
 def execute(ex: Executable, buffers):
@@ -43,7 +142,7 @@ def execute(ex: Executable, buffers):
     first (a no-op once the same buffers have been seen); if that changed the
     set of rewritten dots, anything cached around the old structure is dropped
     (reference engine.py:395-400)."""
-    args = list(buffers)
+    args = [b.data if isinstance(b, Buffer) else b for b in buffers]
     if qmm.ENABLED:
         if qmm.prologue(ex.interp, args):
             ex.invalidate_traces()

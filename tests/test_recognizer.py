@@ -398,3 +398,41 @@ def test_emit_fails_loudly_without_a_gpu():
     with pytest.raises(Exception) as e:
         engine.execute(ex, args)
     assert not isinstance(e.value, I.UnsupportedOp)
+
+
+# ------------------------------------------------------- engine surface ----
+
+def test_engine_surface_names_a_pjrt_plugin_calls():
+    """compile_program / execute / buffer_from_host / buffer_to_host /
+    buffer_pointer / device_kind / stablehlo_version and the executable's
+    attributes (reference src/metaljax/engine.py:133-175, :549-591)."""
+    import numpy as np
+    from metaljax_amd import engine
+    text = T.float_dot(8, 16, 4, el="f32")          # y = x @ (w * r[:, None]): w [8,16], r [8], x [4,8]
+    ex = engine.compile_program(text.encode(), "mlir", None)
+    assert ex.name == "main" and len(ex.fingerprint) == 64
+    assert ex.num_params == 3 and ex.num_outputs == 1
+    assert ex.out_dims == [[4, 16]] and ex.donated_params == []
+    assert ex.out_type_enums == [engine.PJRT_TYPES.index("F32")]
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal((8, 16)).astype(np.float32)
+    r = rng.standard_normal((8,)).astype(np.float32)
+    x = rng.standard_normal((4, 8)).astype(np.float32)
+    f32 = engine.PJRT_TYPES.index("F32")
+    # a transposed host view arrives with strides
+    wt = np.ascontiguousarray(w.T)
+    bw = engine.buffer_from_host(memoryview(wt), f32, [8, 16], [4, 4 * 8], 0)
+    br = engine.buffer_from_host(memoryview(r), f32, [8], None)
+    bx = engine.buffer_from_host(memoryview(x), f32, [4, 8], None)
+    assert bx.nbytes == x.nbytes and bx.dims == [4, 8] and bx.type_enum == f32
+    assert engine.buffer_pointer(bx) != 0
+    (y,) = engine.execute(ex, [bw, br, bx])
+    got = np.frombuffer(engine.buffer_to_host(y), np.float32).reshape(4, 16)
+    np.testing.assert_allclose(got, x @ (w * r[:, None]), rtol=1e-5, atol=1e-5)
+    # bf16 bytes round-trip as 16-bit patterns
+    bits = np.array([0x3F80, 0xC000, 0x0000], np.uint16)
+    bf = engine.buffer_from_host(memoryview(bits), engine.PJRT_TYPES.index("BF16"), [3], None)
+    assert engine.buffer_to_host(bf) == bits.tobytes()
+    with pytest.raises(TypeError, match="Unsupported"):
+        engine.buffer_from_host(None, engine.PJRT_TYPES.index("C64"), [1], None)
+    assert isinstance(engine.device_kind(), str) and len(engine.stablehlo_version()) == 3
