@@ -161,6 +161,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other named shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--m16-only", action="store_true", help="run the headline decode leg only")
+    ap.add_argument("--shape", choices=["C3", "C4", "C5"], default=None,
+                    help="time one of the other named shapes only (for profiling that kernel)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a 64 MiB read + 64 MiB write elementwise kernel five times, "
                          "for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -181,6 +183,9 @@ def main():
         for _ in range(5):
             torch.bitwise_not(src, out=dst)
         torch.cuda.synchronize()
+    if args.shape:
+        print(json.dumps({args.shape: bench_once(int(args.shape[1]))}))
+        return 0
     wl, ms, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
     us = ms * 1e3 / args.steps
     gbs = wl.algorithmic_bytes / us / 1e3
