@@ -37,9 +37,12 @@
 // Order of issue.  The first byte of a kernel arrives 2-3 us after it starts
 // and the weight stream is what bounds the kernel, so the first weight tile is
 // requested at once, between the activation rounds: x0 x1 t0 x2 (the four
-// slots), then one item per freed slot: x3 t1 t2 t3.  Loads retire in order,
-// so "item i has landed" is a wait on the number of loads issued after it; the
-// schedule and those counts are worked out at compile time (struct Sched).
+// slots), then one item per freed slot: x3 t1 t2 t3, running on into the next
+// pass (K > CW slices) without draining the ring.  Loads retire in order, so
+// "item i has landed" is a wait on the number of loads issued after it; the
+// schedule and those counts are worked out at compile time (struct Sched),
+// the slot of every item is a small piece of scalar bookkeeping that both
+// roles run identically.
 #include <type_traits>
 #include <utility>
 
@@ -98,15 +101,12 @@ struct Sched {
     return -1;
   }
   static constexpr int loads(int item) { return item < XR ? LX : LT; }
-  // the issue at position j >= B happens after barrier j-B+1 and takes the slot of item j-B
-  static constexpr int slot_at(int j) { return j < B ? j : slot_at(pos(j - B)); }
-  static constexpr int slot(int item) { return slot_at(pos(item)); }
-  // loads that may still be outstanding when item k is declared landed
-  static constexpr int allowed(int k) {
-    int issued = B + (k >= 1 ? k - 1 : 0);
-    if (issued > NI) issued = NI;
+  // Loads that may still be outstanding when item k of a pass is declared
+  // landed, `end` issue positions (counted from the start of that pass, running
+  // on into the next pass, whose items repeat the order) having been issued.
+  static constexpr int allowed(int k, int end) {
     int n = 0;
-    for (int j = pos(k) + 1; j < issued; ++j) n += loads(item_at(j));
+    for (int j = pos(k) + 1; j < end; ++j) n += loads(item_at(j % NI));
     return n > 63 ? 63 : n;
   }
 };
@@ -225,10 +225,10 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // wavefronts' partial sums and store the 16 x 16 results, under the next
     // item's arithmetic.  Lane l, component e of an accumulator is output row
     // 4*(l/16) + e, column l % 16 of the tile.
-    auto reduce_tile = [&](int p, auto tc) __attribute__((always_inline)) {
+    auto reduce_tile = [&](int p, auto tc, int slot) __attribute__((always_inline)) {
       constexpr int t = decltype(tc)::value;
       if (p != passes - 1 || t >= ntiles) return;
-      const float* part = reinterpret_cast<const float*>(ring + S::slot(XR + t) * kItem);
+      const float* part = reinterpret_cast<const float*>(ring + slot * kItem);
 #pragma unroll
       for (int e = lw; e < 4; e += NL) {
         float v = 0.f;
@@ -239,22 +239,50 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if (m < a.M && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
       }
     };
+    // Slot of every item of the current pass (by order of use) and of the next
+    // pass's items issued ahead; both roles keep this bookkeeping identically.
+    int sl_cur[NI], sl_nxt[NI], prev_last = 0;
+#pragma unroll
+    for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k] = 0;
+    static_for<S::B>([&](auto jc) __attribute__((always_inline)) {
+      constexpr int j = decltype(jc)::value;
+      sl_cur[S::item_at(j)] = j;
+      issue_item(0, std::integral_constant<int, S::item_at(j)>{}, j);
+    });
     for (int p = 0; p < passes; ++p) {
-      static_for<S::B>([&](auto jc) __attribute__((always_inline)) {
-        constexpr int j = decltype(jc)::value;
-        issue_item(p, std::integral_constant<int, S::item_at(j)>{}, S::slot_at(j));
-      });
+      const bool last = p == passes - 1;
       static_for<NI>([&](auto kc) __attribute__((always_inline)) {
         constexpr int k = decltype(kc)::value;
-        wait_vmcnt<S::allowed(k)>();              // item k has landed
+        constexpr int e = S::B + k - 1;           // issue positions out when item k (not the very first) is awaited
+        // item k has landed:
+        if constexpr (k == 0) {
+          if (p == 0) wait_vmcnt<S::allowed(0, S::B)>();
+          else wait_vmcnt<S::allowed(0, e)>();
+        } else {
+          if (last) wait_vmcnt<S::allowed(k, e < NI ? e : NI)>();
+          else wait_vmcnt<S::allowed(k, e)>();
+        }
         item_barrier();
-        constexpr int j = S::B + k - 1;           // the slot of item k-1 is free now
-        if constexpr (k >= 1 && j < NI)
-          issue_item(p, std::integral_constant<int, S::item_at(j)>{}, S::slot_at(j));
-        if constexpr (k >= XR + 1) reduce_tile(p, std::integral_constant<int, k - 1 - XR>{});
+        // the slot of the item used just before is free now: the next item in issue order takes it
+        const int freed = k >= 1 ? sl_cur[k >= 1 ? k - 1 : 0] : prev_last;
+        if (k >= 1 || p >= 1) {
+          if constexpr (e < NI) {
+            sl_cur[S::item_at(e)] = freed;
+            issue_item(p, std::integral_constant<int, S::item_at(e)>{}, freed);
+          } else if (!last) {
+            sl_nxt[S::item_at(e - NI)] = freed;
+            issue_item(p + 1, std::integral_constant<int, S::item_at(e - NI)>{}, freed);
+          }
+        }
+        if constexpr (k >= XR + 1) reduce_tile(p, std::integral_constant<int, k - 1 - XR>{}, sl_cur[k - 1]);
       });
-      item_barrier();                             // the pass is consumed: its slots may be refilled
-      reduce_tile(p, std::integral_constant<int, TMAX - 1>{});
+      prev_last = sl_cur[NI - 1];
+      if (last) {
+        item_barrier();                           // everything consumed
+        reduce_tile(p, std::integral_constant<int, TMAX - 1>{}, prev_last);
+      }
+#pragma unroll
+      for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k];
     }
   } else {
     // ----------------------------------------------------- compute wavefronts
@@ -265,14 +293,23 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const bf16x8 ones = as_bf16x8(one, one, one, one);
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
     const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
+    int sl_cur[NI], sl_nxt[NI], prev_last = 0;     // the loaders' slot bookkeeping, mirrored
+#pragma unroll
+    for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k] = 0;
+    static_for<S::B>([&](auto jc) __attribute__((always_inline)) {
+      constexpr int j = decltype(jc)::value;
+      sl_cur[S::item_at(j)] = j;
+    });
     for (int p = 0; p < passes; ++p) {
+      const bool last = p == passes - 1;
       const bool active = p * CW + wave < slices;               // uniform
       bf16x8 xa[CPS][2];
       bf16x8 axh, axm, axo;
       auto consume = [&](auto ic) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
         item_barrier();
-        const unsigned char* base = ring + S::slot(i) * kItem + rowb;
+        const int slot = sl_cur[i];
+        const unsigned char* base = ring + slot * kItem + rowb;
         if constexpr (i < XR) {
           // activations of chunks 2i, 2i+1 into operand layout
           if (active) {
@@ -309,7 +346,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         } else {
           constexpr int t = i - XR;
           if (active && t < ntiles) {
-            const unsigned char* tb = tabs + S::slot(i) * kTab + wave * 256 + r * 16;
+            const unsigned char* tb = tabs + slot * kTab + wave * 256 + r * 16;
             u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
             u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
             if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
@@ -359,14 +396,24 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           // slice of the tile was (nobody else reads that region, and a tile's
           // slot is not refilled within a pass); the loaders add the slices up.
           if (p == passes - 1 && t < ntiles) {
-            float* part = reinterpret_cast<float*>(ring + S::slot(i) * kItem + wave * 4096);
+            float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
 #pragma unroll
             for (int e = 0; e < 4; ++e) part[e * kWave + lane] = acc[t][e];
           }
         }
+        // mirror of the loaders' issue after this item's barrier
+        constexpr int e = S::B + i - 1;
+        const int freed = i >= 1 ? sl_cur[i >= 1 ? i - 1 : 0] : prev_last;
+        if (i >= 1 || p >= 1) {
+          if constexpr (e < NI) sl_cur[S::item_at(e)] = freed;
+          else if (!last) sl_nxt[S::item_at(e - NI)] = freed;
+        }
       };
       static_for<NI>(consume);
-      item_barrier();                             // pass consumed
+      prev_last = sl_cur[NI - 1];
+      if (last) item_barrier();                   // everything consumed
+#pragma unroll
+      for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k];
     }
   }
 }
@@ -401,13 +448,14 @@ void launch_g(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st)
 }  // namespace
 
 // The loader-wavefront kernel pays off where a workgroup streams three or
-// four tiles over exactly eight K-slices, i.e. one pass (measured: 3-5 % faster
-// on 4096 x 14336 and 4096 x 28672 four-bit weights; with two passes the ring
-// drains between them and it is 13 % slower, as it is with two tiles).  Eight
-// compute and four loader wavefronts.  Everything else stays on the
-// self-loading kernel.
+// four tiles over eight K-slices at a time (measured 3-5 % faster on 4096 x
+// 14336 and 4096 x 28672 four-bit weights; with two tiles a workgroup the
+// activation items outweigh the tiles and it is 13 % slower).  Eight compute
+// and four loader wavefronts.  Everything else stays on the self-loading
+// kernel.
 bool skinny2_supported(int64_t K, int bits, int waves, int rows_per_wg) {
-  return waves == 8 && K == 8 * (2048 / bits) && rows_per_wg > 32 && rows_per_wg <= 64;
+  (void)K; (void)bits;
+  return waves == 8 && rows_per_wg > 32 && rows_per_wg <= 64;
 }
 
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {

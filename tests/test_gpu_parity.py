@@ -240,6 +240,9 @@ def test_gemv_batched():
     (8, 128, 16, 12000, 2048),   # eight-bit codes, one pass
     (4, 64, 2, 5000, 8192),      # two passes of four-bit slices
     (4, 64, 1, 16384, 6144),     # 12 slices: the second pass is half empty
+    (8, 64, 7, 12000, 4096),     # eight-bit codes, two passes, three tiles a workgroup
+    (4, 128, 16, 9000, 8192),    # two passes, group 128
+    (4, 64, 3, 10000, 12288),    # three passes
 ])
 def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     """Shapes big enough for the decode kernel whose loader wavefronts stream
