@@ -43,6 +43,7 @@
 // schedule and those counts are worked out at compile time (struct Sched),
 // the slot of every item is a small piece of scalar bookkeeping that both
 // roles run identically.
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -90,7 +91,7 @@ struct Sched {
   static constexpr int NI = XR + TMAX;
   static constexpr int B = NI < 4 ? NI : 4;                 // ring slots = items issued up front
   static constexpr int item_at(int j) {                     // the item issued j-th
-    if (j < 2) return j;
+    if (XR == 0 || j < 2) return j;
     if (j == 2) return XR;
     if (j < XR + 1) return j - 1;
     return j;
@@ -121,11 +122,11 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <int BITS, int CW, int NL, int TMAX, int GSHIFT>
+template <int BITS, int CW, int NL, int TMAX, int GSHIFT, int XD>
 __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, int rows_per_wg) {
   constexpr int KS = 2048 / BITS;                 // codes per slice: 512 | 256
   constexpr int CPS = KS / 64;                    // 64-code chunks per slice: 8 | 4
-  constexpr int XR = KS / 128;                    // activation rounds per slice: 4 | 2
+  constexpr int XR = XD ? 0 : KS / 128;           // activation rounds per slice through the ring: 4 | 2, or none
   constexpr int NI = XR + TMAX;                   // items per pass
   constexpr int kItem = CW * 4096;
   constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;   // scale rows | bias rows of one tile
@@ -182,9 +183,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     }
     const int trow = lane & 15, tsl = lane >> 4;  // table loads: lane = (slice within four, row)
 
-    // item `i` (compile-time kind) of pass `p` into ring slot `slot`
-    auto issue_item = [&](int p, auto ic, int slot) __attribute__((always_inline)) {
-      constexpr int i = decltype(ic)::value;
+    // weight tile t of pass `p`, and its table rows, into ring slot `slot`
+    auto issue_tile = [&](int p, int t, int slot) __attribute__((always_inline)) {
       unsigned char* base = ring + slot * kItem;
       static_for<QI>([&](auto qc) __attribute__((always_inline)) {
         constexpr int q = decltype(qc)::value;
@@ -192,32 +192,40 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const int j = lw + q * NL;                // uniform
         const int sloc = j >> 2, rq = j & 3;
         const int sl = p * CW + sloc;
-        const bool ok = sl < slices;              // also false for passes past the last
-        unsigned char* dst = base + sloc * 4096 + rq * 1024;
-        if constexpr (i < XR) {
-          const uint32_t so = ok ? (uint32_t)(sl * KS + i * 128) * 2u : 0u;
-          dma16(rx, dst, ok ? xv[o] : kOutOfRange, so);
-        } else {
-          constexpr int t = i - XR;
-          const bool rok = ok && n_begin + t * 16 + wrow[o] < n_end;
-          const uint32_t so = ok ? (uint32_t)sl * 256u + (uint32_t)(t * 16 * wpr) : 0u;
-          dma16(rw, dst, rok ? wv[o] : kOutOfRange, so);
-        }
+        const bool rok = sl < slices && n_begin + t * 16 + wrow[o] < n_end;   // false for passes past the last
+        const uint32_t so = rok ? (uint32_t)sl * 256u + (uint32_t)(t * 16 * wpr) : 0u;
+        dma16(rw, base + sloc * 4096 + rq * 1024, rok ? wv[o] : kOutOfRange, so);
       });
-      if constexpr (i >= XR) {
-        constexpr int t = i - XR;
-        unsigned char* tb = tabs + slot * kTab;
+      unsigned char* tb = tabs + slot * kTab;
 #pragma unroll
-        for (int q = 0; q < QT; ++q) {
-          const int jt = lw + q * NL;             // uniform
-          const int kind = jt / (NTAB / 2), h = jt % (NTAB / 2);
-          const int sloc = 4 * h + tsl;
+      for (int q = 0; q < QT; ++q) {
+        const int jt = lw + q * NL;               // uniform
+        const int kind = jt / (NTAB / 2), h = jt % (NTAB / 2);
+        const int sloc = 4 * h + tsl;
+        const int sl = p * CW + sloc;
+        const int64_t n = n_begin + t * 16 + trow;
+        const bool ok = sloc < CW && sl < slices && n < n_end;
+        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> GSHIFT) * 2u : kOutOfRange;
+        dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
+      }
+    };
+    // item `i` (compile-time kind) of pass `p` into ring slot `slot`
+    auto issue_item = [&](int p, auto ic, int slot) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i < XR) {
+        unsigned char* base = ring + slot * kItem;
+        static_for<QI>([&](auto qc) __attribute__((always_inline)) {
+          constexpr int q = decltype(qc)::value;
+          constexpr int o = (q * NL) & 3;
+          const int j = lw + q * NL;              // uniform
+          const int sloc = j >> 2, rq = j & 3;
           const int sl = p * CW + sloc;
-          const int64_t n = n_begin + t * 16 + trow;
-          const bool ok = sloc < CW && sl < slices && n < n_end;
-          const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> GSHIFT) * 2u : kOutOfRange;
-          dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
-        }
+          const bool ok = sl < slices;            // also false for passes past the last
+          const uint32_t so = ok ? (uint32_t)(sl * KS + i * 128) * 2u : 0u;
+          dma16(rx, base + sloc * 4096 + rq * 1024, ok ? xv[o] : kOutOfRange, so);
+        });
+      } else {
+        issue_tile(p, i - XR, slot);
       }
     };
     // The K slices of tile t meet here: after the barrier that follows the
@@ -225,8 +233,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // wavefronts' partial sums and store the 16 x 16 results, under the next
     // item's arithmetic.  Lane l, component e of an accumulator is output row
     // 4*(l/16) + e, column l % 16 of the tile.
-    auto reduce_tile = [&](int p, auto tc, int slot) __attribute__((always_inline)) {
-      constexpr int t = decltype(tc)::value;
+    auto reduce_tile = [&](int p, int t, int slot) __attribute__((always_inline)) {
       if (p != passes - 1 || t >= ntiles) return;
       const float* part = reinterpret_cast<const float*>(ring + slot * kItem);
 #pragma unroll
@@ -239,6 +246,31 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if (m < a.M && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
       }
     };
+    if constexpr (XD) {
+      // Every item is a tile: item g = p * TMAX + t lives in slot g % B.  A load
+      // instruction is accepted at the pace at which data comes back (issuing
+      // a tile takes about as long as receiving one), and a wavefront stuck in
+      // issue cannot publish what has already landed: so the loaders keep two
+      // items out -- item g+1 is requested before item g is published, g+2
+      // right after -- and no more (refilling two slots after a publication
+      // measured 0.5 us slower).
+      static_assert(!XD || S::B >= 4, "two items in flight, one being consumed, one being reduced");
+      const int G = passes * TMAX;
+      issue_tile(0, 0, 0);
+      if (G > 1) issue_tile(1 / TMAX, 1 % TMAX, 1 % S::B);
+#pragma nounroll
+      for (int g = 0; g < G; ++g) {
+        // item g has landed: only item g+1 may still be out (a store in
+        // between only tightens the wait)
+        if (g + 1 < G) wait_vmcnt<LT>(); else wait_vmcnt<0>();
+        item_barrier();                           // item g published; item g-1 consumed
+        if (g + 2 < G) issue_tile((g + 2) / TMAX, (g + 2) % TMAX, (g + 2) % S::B);   // that slot's last tile was reduced a step ago
+        if (g >= 1) reduce_tile((g - 1) / TMAX, (g - 1) % TMAX, (g - 1) % S::B);
+      }
+      item_barrier();                             // everything consumed
+      reduce_tile(passes - 1, TMAX - 1, (G - 1) % S::B);
+      return;
+    }
     // Slot of every item of the current pass (by order of use) and of the next
     // pass's items issued ahead; both roles keep this bookkeeping identically.
     int sl_cur[NI], sl_nxt[NI], prev_last = 0;
@@ -251,10 +283,11 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     });
     for (int p = 0; p < passes; ++p) {
       const bool last = p == passes - 1;
-      static_for<NI>([&](auto kc) __attribute__((always_inline)) {
+      // publication of item k: wait until it has landed, barrier, refill the
+      // slot of the item used just before with the next item in issue order
+      auto publish = [&](auto kc) __attribute__((always_inline)) {
         constexpr int k = decltype(kc)::value;
         constexpr int e = S::B + k - 1;           // issue positions out when item k (not the very first) is awaited
-        // item k has landed:
         if constexpr (k == 0) {
           if (p == 0) wait_vmcnt<S::allowed(0, S::B)>();
           else wait_vmcnt<S::allowed(0, e)>();
@@ -263,7 +296,6 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           else wait_vmcnt<S::allowed(k, e)>();
         }
         item_barrier();
-        // the slot of the item used just before is free now: the next item in issue order takes it
         const int freed = k >= 1 ? sl_cur[k >= 1 ? k - 1 : 0] : prev_last;
         if (k >= 1 || p >= 1) {
           if constexpr (e < NI) {
@@ -274,13 +306,34 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
             issue_item(p + 1, std::integral_constant<int, S::item_at(e - NI)>{}, freed);
           }
         }
-        if constexpr (k >= XR + 1) reduce_tile(p, std::integral_constant<int, k - 1 - XR>{}, sl_cur[k - 1]);
-      });
-      prev_last = sl_cur[NI - 1];
-      if (last) {
-        item_barrier();                           // everything consumed
-        reduce_tile(p, std::integral_constant<int, TMAX - 1>{}, prev_last);
+      };
+      static_for<XR + 1>(publish);                // the activation rounds and the first tile
+      // The other tiles, and the barrier that ends the last pass, as a real
+      // loop: after its barrier, step k sums the K-slices of the tile used just
+      // before (item k-1), and that code is then the same, already fetched,
+      // copy for every tile -- a kernel that runs each instruction once pays an
+      // instruction-cache miss for every new block, and at the very end of the
+      // kernel nothing hides it (measured: 1.2 us for the last tile's sum as a
+      // separate copy, 0.3 us for a second run of the same code).
+#pragma nounroll
+      for (int k = XR + 1; k <= NI; ++k) {
+        if (k == NI) {
+          if (!last) break;
+          item_barrier();                         // everything consumed
+        } else {
+          if (k == XR + 1) { if constexpr (TMAX > 1) publish(std::integral_constant<int, XR + 1>{}); }
+          else if (k == XR + 2) { if constexpr (TMAX > 2) publish(std::integral_constant<int, (TMAX > 2 ? XR + 2 : 0)>{}); }
+          else { if constexpr (TMAX > 3) publish(std::integral_constant<int, (TMAX > 3 ? XR + 3 : 0)>{}); }
+        }
+        const int t = k - 1 - XR;
+        int slot = sl_cur[XR];
+        if constexpr (TMAX > 1) slot = t == 1 ? sl_cur[XR + 1] : slot;
+        if constexpr (TMAX > 2) slot = t == 2 ? sl_cur[XR + (TMAX > 2 ? 2 : 0)] : slot;
+        if constexpr (TMAX > 3) slot = t == 3 ? sl_cur[XR + (TMAX > 3 ? 3 : 0)] : slot;
+        reduce_tile(p, t, slot);
       }
+      static_assert(TMAX <= 4, "the tile loop names at most four tiles");
+      prev_last = sl_cur[NI - 1];
 #pragma unroll
       for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k];
     }
@@ -293,6 +346,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const bf16x8 ones = as_bf16x8(one, one, one, one);
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
     const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
+    const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+    const uint32_t xlane = r < a.M ? (uint32_t)((int64_t)r * a.K * 2) + (uint32_t)kg * 32u : kOutOfRange;
     int sl_cur[NI], sl_nxt[NI], prev_last = 0;     // the loaders' slot bookkeeping, mirrored
 #pragma unroll
     for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k] = 0;
@@ -305,10 +360,49 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       const bool active = p * CW + wave < slices;               // uniform
       bf16x8 xa[CPS][2];
       bf16x8 axh, axm, axo;
+      // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
+      // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
+      auto chunk_sums = [&]() __attribute__((always_inline)) {
+        float xh[8], xm[8], xo[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          float xs = 0.f;
+          if (c < CPS) {
+            f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
+            t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
+            xs = kg == 0 ? t4[0] : 0.f;
+          }
+          split3(xs, xh[c], xm[c], xo[c]);
+        }
+        axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
+        axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
+        axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
+      };
+      if constexpr (XD) {
+        // This wavefront's slice of the activations straight from global memory
+        // (L2 after the first workgroup) into operand layout: lane (r, kg) takes
+        // pieces 2*kg and 2*kg + 1 of every chunk of row r.
+        u32x4 raw[CPS][2];
+        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
+#pragma unroll
+        for (int c = 0; c < CPS; ++c)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
+                rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
+#pragma unroll
+        for (int c = 0; c < CPS; ++c)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
+            else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
+          }
+        if (active) chunk_sums();
+      }
       auto consume = [&](auto ic) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
         item_barrier();
-        const int slot = sl_cur[i];
+        const int slot = XD ? (p * TMAX + i) % S::B : sl_cur[i];
         const unsigned char* base = ring + slot * kItem + rowb;
         if constexpr (i < XR) {
           // activations of chunks 2i, 2i+1 into operand layout
@@ -324,24 +418,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
               }
           }
           if constexpr (i == XR - 1) {
-            // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
-            // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
-            if (active) {
-              float xh[8], xm[8], xo[8];
-#pragma unroll
-              for (int c = 0; c < 8; ++c) {
-                float xs = 0.f;
-                if (c < CPS) {
-                  f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
-                  t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
-                  xs = kg == 0 ? t4[0] : 0.f;
-                }
-                split3(xs, xh[c], xm[c], xo[c]);
-              }
-              axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
-              axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
-              axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
-            }
+            if (active) chunk_sums();
           }
         } else {
           constexpr int t = i - XR;
@@ -418,13 +495,13 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   }
 }
 
-template <int BITS, int CW, int NL, int TMAX, int GSHIFT>
+template <int BITS, int CW, int NL, int TMAX, int GSHIFT, int XD>
 void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch);
   constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
-  constexpr int XR = 2048 / BITS / 128;
+  constexpr int XR = XD ? 0 : 2048 / BITS / 128;
   const size_t lds = (size_t)(XR + TMAX < 4 ? XR + TMAX : 4) * (CW * 4096 + 2 * kTabKind);
-  auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT>;
+  auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   static bool configured = false;                 // one flag per instantiation
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -436,8 +513,18 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
 
 template <int BITS, int CW, int NL, int TMAX>
 void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1>(a, batch, rows_per_wg, st);
-  else launch_one<BITS, CW, NL, TMAX, 0>(a, batch, rows_per_wg, st);
+  // One pass (K within CW slices): the compute wavefronts fetch their own
+  // activations and every ring slot starts with a weight tile.
+  static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
+  static const int force = env ? atoi(env) : -1;
+  const bool xd = force >= 0 ? force != 0 : a.K * BITS / 8 / 256 <= CW && a.M <= 8;
+  if (xd) {
+    if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, 1>(a, batch, rows_per_wg, st);
+    else launch_one<BITS, CW, NL, TMAX, 0, 1>(a, batch, rows_per_wg, st);
+  } else {
+    if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, 0>(a, batch, rows_per_wg, st);
+    else launch_one<BITS, CW, NL, TMAX, 0, 0>(a, batch, rows_per_wg, st);
+  }
 }
 
 template <int BITS>
