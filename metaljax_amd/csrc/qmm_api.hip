@@ -13,7 +13,7 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
                    int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st);
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
-bool skinny2_supported(int64_t K, int bits, int waves, int rows_per_wg);
+bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
 void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
@@ -189,12 +189,14 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
   if (M <= kGemvMaxM && mode == QMM_MODE_AFFINE && (group_size == 64 || group_size == 128) &&
       (bits == 4 || bits == 8) && K % (2048 / bits) == 0) {
     // the staged decode kernel (bf16 tables assumed): contiguous row ranges
-    int waves, rows;
+    int waves, rows, rows2;
     skinny_geometry(N, K, bits, &waves, &rows);
+    // eight compute + four loader wavefronts where the loader kernel serves the shape
+    const bool loaders = !getenv("QMM_SKINNY_V1") && skinny2_plan(M, N, K, bits, &rows2);
+    if (loaders) rows = rows2;
     if (kernel) *kernel = QMM_KERNEL_GEMV;
     if (grid) *grid = (int)ceil_div(N, rows);
-    // eight compute + four loader wavefronts where the loader kernel serves the shape
-    if (block) *block = skinny2_supported(K, bits, waves, rows) && !getenv("QMM_SKINNY_V1") ? 64 * 12 : 64 * waves;
+    if (block) *block = loaders ? 64 * 12 : 64 * waves;
     return QMM_OK;
   }
   if (M <= kGemvMaxM) {

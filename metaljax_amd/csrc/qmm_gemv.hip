@@ -376,7 +376,7 @@ bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                       const void* b);
 void skinny_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int tab, hipStream_t st);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
-bool skinny2_supported(int64_t K, int bits, int waves, int rows_per_wg);
+bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st);
 
 // Tile / slice / unroll choice; QMM_GEMV_T, QMM_GEMV_WAVES and QMM_GEMV_U
@@ -414,9 +414,8 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
     // big weights: the kernel with loader wavefronts (QMM_SKINNY_V1 keeps the
     // self-loading one everywhere, for comparison)
     static const int v1 = env_int("QMM_SKINNY_V1");
-    int waves, rows;
-    skinny_geometry(N, K, bits, &waves, &rows);
-    if (!v1 && skinny2_supported(K, bits, waves, rows)) skinny2_dispatch(a, batch, gs, bits, rows, st);
+    int rows;
+    if (!v1 && skinny2_plan(M, N, K, bits, &rows)) skinny2_dispatch(a, batch, gs, bits, rows, st);
     else skinny_dispatch(a, batch, gs, bits, tab, st);
     return;
   }

@@ -12,7 +12,25 @@
 // only afterwards.  Here NL loader wavefronts do nothing but issue
 // direct-to-LDS loads (they are the ones that block), and CW compute
 // wavefronts never touch global memory until the final store: they consume
-// "items" from a three-slot LDS ring as the loaders complete them.
+// "items" from a four-slot LDS ring as the loaders complete them.
+//
+// Two variants (template flag XD):
+//
+// * ring variant (XD = 0; several passes over K, or more than eight rows of
+//   activations): activations and weight tiles both travel through the ring,
+//   as described below;
+// * direct variant (XD = 1; K is exactly one pass and M <= 8): each compute
+//   wavefront fetches its own K-slice of the activations straight into MFMA
+//   operand registers at the start of the kernel, every ring slot holds a
+//   weight tile, and the tile loop is a real loop in both roles, so a
+//   workgroup can take any number of tiles (the host deals up to 128 rows a
+//   workgroup so that a 28672-row weight is still one workgroup per compute
+//   unit).  The loaders keep two tiles requested: tile g+1 before tile g is
+//   published, tile g+2 right after -- issuing a tile takes about as long as
+//   receiving one, and a wavefront stuck in issue cannot publish.  Measured
+//   on 4096 x 14336 four-bit weights: 10.3 us at M = 1 against 11.9 us for the
+//   ring variant; at M = 16 the 128 KB of activations in front of the first
+//   tile cost more than the ring's interleaving (13.3 against 12.8 us).
 //
 // Items of one pass (a pass = CW consecutive K-slices, one per compute
 // wavefront; a slice = 256 packed bytes per row):
@@ -89,7 +107,7 @@ __device__ __forceinline__ uint32_t hi16_pair(float a, float b) {      // (bf16(
 template <int XR, int TMAX, int LX, int LT>
 struct Sched {
   static constexpr int NI = XR + TMAX;
-  static constexpr int B = NI < 4 ? NI : 4;                 // ring slots = items issued up front
+  static constexpr int B = XR == 0 || NI >= 4 ? 4 : NI;     // ring slots (= items issued up front by the ring variant)
   static constexpr int item_at(int j) {                     // the item issued j-th
     if (XR == 0 || j < 2) return j;
     if (j == 2) return XR;
@@ -247,28 +265,29 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       }
     };
     if constexpr (XD) {
-      // Every item is a tile: item g = p * TMAX + t lives in slot g % B.  A load
+      // Every item is a tile: tile g lives in slot g % 4.  A load
       // instruction is accepted at the pace at which data comes back (issuing
       // a tile takes about as long as receiving one), and a wavefront stuck in
       // issue cannot publish what has already landed: so the loaders keep two
       // items out -- item g+1 is requested before item g is published, g+2
       // right after -- and no more (refilling two slots after a publication
       // measured 0.5 us slower).
-      static_assert(!XD || S::B >= 4, "two items in flight, one being consumed, one being reduced");
-      const int G = passes * TMAX;
+      // One pass only (the host sees to it), any number of tiles.
+      static_assert(!XD || S::B == 4, "two items in flight, one being consumed, one being reduced");
+      const int G = ntiles;
       issue_tile(0, 0, 0);
-      if (G > 1) issue_tile(1 / TMAX, 1 % TMAX, 1 % S::B);
+      if (G > 1) issue_tile(0, 1, 1);
 #pragma nounroll
       for (int g = 0; g < G; ++g) {
         // item g has landed: only item g+1 may still be out (a store in
         // between only tightens the wait)
         if (g + 1 < G) wait_vmcnt<LT>(); else wait_vmcnt<0>();
         item_barrier();                           // item g published; item g-1 consumed
-        if (g + 2 < G) issue_tile((g + 2) / TMAX, (g + 2) % TMAX, (g + 2) % S::B);   // that slot's last tile was reduced a step ago
-        if (g >= 1) reduce_tile((g - 1) / TMAX, (g - 1) % TMAX, (g - 1) % S::B);
+        if (g + 2 < G) issue_tile(0, g + 2, (g + 2) & 3);   // that slot's last tile was reduced a step ago
+        if (g >= 1) reduce_tile(0, g - 1, (g - 1) & 3);
       }
       item_barrier();                             // everything consumed
-      reduce_tile(passes - 1, TMAX - 1, (G - 1) % S::B);
+      reduce_tile(0, G - 1, (G - 1) & 3);
       return;
     }
     // Slot of every item of the current pass (by order of use) and of the next
@@ -355,54 +374,117 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       constexpr int j = decltype(jc)::value;
       sl_cur[S::item_at(j)] = j;
     });
+    bf16x8 xa[CPS][2];
+    bf16x8 axh, axm, axo;
+    // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
+    // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
+    auto chunk_sums = [&]() __attribute__((always_inline)) {
+      float xh[8], xm[8], xo[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        float xs = 0.f;
+        if (c < CPS) {
+          f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
+          t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
+          xs = kg == 0 ? t4[0] : 0.f;
+        }
+        split3(xs, xh[c], xm[c], xo[c]);
+      }
+      axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
+      axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
+      axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
+    };
+    // acc + this wavefront's K-slice of one tile: `base` is the lane's row in
+    // the slice's 4 KB of codes, `tb` its table row
+    auto tile_math = [&](const unsigned char* base, const unsigned char* tb, f32x4 acc_in) __attribute__((always_inline)) {
+      u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
+      u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
+      if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
+        svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
+                    byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
+        bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
+                    byte_perm(bvt[1], bvt[1], 0x01000100u), byte_perm(bvt[1], bvt[1], 0x03020302u)};
+      }
+      const bf16x8 bop = __builtin_bit_cast(bf16x8, bvt);
+      f32x4 accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, bop, acc_in, 0, 0, 0);
+      accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, bop, accb, 0, 0, 0);
+      accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, bop, accb, 0, 0, 0);
+      f32x4 accs = zero;
+      if constexpr (BITS == 4) {
+        const bf16x8 sop = __builtin_bit_cast(bf16x8, svt);
+        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, sop, zero, 0, 0, 0);
+        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, sop, accs, 0, 0, 0);
+        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, sop, accs, 0, 0, 0);
+      }
+      f32x4 at = accb;
+#pragma unroll
+      for (int c = 0; c < CPS; ++c) {
+        f32x4 d;
+        if constexpr (BITS == 4) {
+          const uint32_t pc = (uint32_t)(2 * c + (kg >> 1));
+          const u32x2 q = *reinterpret_cast<const u32x2*>(base + ((pc ^ swz) << 4) + (kg & 1) * 8);
+          d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int4(q[0], nib, magic), zero, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int4(q[1], nib, magic), d, 0, 0, 0);
+        } else {
+          const uint32_t pc = (uint32_t)(4 * c + kg);
+          const u32x4 q = *reinterpret_cast<const u32x4*>(base + ((pc ^ swz) << 4));
+          d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int8(q[0], q[1]), zero, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int8(q[2], q[3]), d, 0, 0, 0);
+        }
+        const uint32_t sw = svt[c >> 1];
+        const float sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
+      }
+      if constexpr (BITS == 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) at[e] = fmaf(-128.f, accs[e], at[e]);
+      }
+      return at;
+    };
+    if constexpr (XD) {
+      // One pass.  This wavefront's slice of the activations straight from
+      // global memory (L2 after the first workgroup) into operand layout: lane
+      // (r, kg) takes pieces 2*kg and 2*kg + 1 of every chunk of row r.
+      const bool active = wave < slices;          // uniform
+      u32x4 raw[CPS][2];
+      const uint32_t so = active ? (uint32_t)(wave * KS) * 2u : 0u;
+#pragma unroll
+      for (int c = 0; c < CPS; ++c)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
+              rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
+#pragma unroll
+      for (int c = 0; c < CPS; ++c)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
+          else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
+        }
+      if (active) chunk_sums();
+      // The tiles as a real loop (any number of them): a tile's sums leave for
+      // its slot at once, where the loaders add up the slices.
+#pragma nounroll
+      for (int g = 0; g < ntiles; ++g) {
+        item_barrier();
+        const int slot = g & 3;
+        f32x4 at = zero;
+        if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
+        float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
+      }
+      item_barrier();                             // everything consumed
+      return;
+    }
     for (int p = 0; p < passes; ++p) {
       const bool last = p == passes - 1;
       const bool active = p * CW + wave < slices;               // uniform
-      bf16x8 xa[CPS][2];
-      bf16x8 axh, axm, axo;
-      // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
-      // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
-      auto chunk_sums = [&]() __attribute__((always_inline)) {
-        float xh[8], xm[8], xo[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          float xs = 0.f;
-          if (c < CPS) {
-            f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
-            t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
-            xs = kg == 0 ? t4[0] : 0.f;
-          }
-          split3(xs, xh[c], xm[c], xo[c]);
-        }
-        axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
-        axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
-        axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
-      };
-      if constexpr (XD) {
-        // This wavefront's slice of the activations straight from global memory
-        // (L2 after the first workgroup) into operand layout: lane (r, kg) takes
-        // pieces 2*kg and 2*kg + 1 of every chunk of row r.
-        u32x4 raw[CPS][2];
-        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
-#pragma unroll
-        for (int c = 0; c < CPS; ++c)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
-                rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
-#pragma unroll
-        for (int c = 0; c < CPS; ++c)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
-            else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
-          }
-        if (active) chunk_sums();
-      }
       auto consume = [&](auto ic) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
         item_barrier();
-        const int slot = XD ? (p * TMAX + i) % S::B : sl_cur[i];
+        const int slot = sl_cur[i];
         const unsigned char* base = ring + slot * kItem + rowb;
         if constexpr (i < XR) {
           // activations of chunks 2i, 2i+1 into operand layout
@@ -422,53 +504,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           }
         } else {
           constexpr int t = i - XR;
-          if (active && t < ntiles) {
-            const unsigned char* tb = tabs + slot * kTab + wave * 256 + r * 16;
-            u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
-            u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
-            if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
-              svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
-                          byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
-              bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
-                          byte_perm(bvt[1], bvt[1], 0x01000100u), byte_perm(bvt[1], bvt[1], 0x03020302u)};
-            }
-            const bf16x8 bop = __builtin_bit_cast(bf16x8, bvt);
-            f32x4 accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, bop, acc[t], 0, 0, 0);
-            accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, bop, accb, 0, 0, 0);
-            accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, bop, accb, 0, 0, 0);
-            f32x4 accs = zero;
-            if constexpr (BITS == 4) {
-              const bf16x8 sop = __builtin_bit_cast(bf16x8, svt);
-              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, sop, zero, 0, 0, 0);
-              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, sop, accs, 0, 0, 0);
-              accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, sop, accs, 0, 0, 0);
-            }
-            f32x4 at = accb;
-#pragma unroll
-            for (int c = 0; c < CPS; ++c) {
-              f32x4 d;
-              if constexpr (BITS == 4) {
-                const uint32_t pc = (uint32_t)(2 * c + (kg >> 1));
-                const u32x2 q = *reinterpret_cast<const u32x2*>(base + ((pc ^ swz) << 4) + (kg & 1) * 8);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int4(q[0], nib, magic), zero, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int4(q[1], nib, magic), d, 0, 0, 0);
-              } else {
-                const uint32_t pc = (uint32_t)(4 * c + kg);
-                const u32x4 q = *reinterpret_cast<const u32x4*>(base + ((pc ^ swz) << 4));
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_int8(q[0], q[1]), zero, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int8(q[2], q[3]), d, 0, 0, 0);
-              }
-              const uint32_t sw = svt[c >> 1];
-              const float sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
-#pragma unroll
-              for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
-            }
-            if constexpr (BITS == 4) {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) at[e] = fmaf(-128.f, accs[e], at[e]);
-            }
-            acc[t] = at;
-          }
+          if (active && t < ntiles)
+            acc[t] = tile_math(base, tabs + slot * kTab + wave * 256 + r * 16, acc[t]);
           // Last pass: this wavefront's partial sums of tile t go where its own
           // slice of the tile was (nobody else reads that region, and a tile's
           // slot is not refilled within a pass); the loaders add the slices up.
@@ -500,7 +537,7 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch);
   constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
-  const size_t lds = (size_t)(XR + TMAX < 4 ? XR + TMAX : 4) * (CW * 4096 + 2 * kTabKind);
+  const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
   auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   static bool configured = false;                 // one flag per instantiation
   if (!configured) {
@@ -512,12 +549,7 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
 }
 
 template <int BITS, int CW, int NL, int TMAX>
-void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  // One pass (K within CW slices): the compute wavefronts fetch their own
-  // activations and every ring slot starts with a weight tile.
-  static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
-  static const int force = env ? atoi(env) : -1;
-  const bool xd = force >= 0 ? force != 0 : a.K * BITS / 8 / 256 <= CW && a.M <= 8;
+void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, bool xd, hipStream_t st) {
   if (xd) {
     if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, 1>(a, batch, rows_per_wg, st);
     else launch_one<BITS, CW, NL, TMAX, 0, 1>(a, batch, rows_per_wg, st);
@@ -527,29 +559,62 @@ void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st)
   }
 }
 
-template <int BITS>
-void launch_g(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  launch_k<BITS, 8, 4, 4>(a, batch, rows_per_wg, st);
+int device_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      hipDeviceProp_t p;
+      if (hipGetDeviceProperties(&p, dev) == hipSuccess && p.multiProcessorCount > 0) n = p.multiProcessorCount;
+    }
+    return n;
+  }();
+  return cus;
+}
+
+// One pass (K is exactly the eight slices of the compute wavefronts) and few
+// rows of activations: the variant whose compute wavefronts fetch their own
+// activations.  Its tile loop is a real loop, so a workgroup takes as many
+// rows as make the grid one workgroup per compute unit (or a whole number of
+// such rounds), up to 128.
+bool direct_x(int64_t M, int64_t K, int bits) {
+  static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
+  static const int force = env ? atoi(env) : -1;
+  if (K * bits / 8 / 256 != 8) return false;
+  return force >= 0 ? force != 0 : M <= 8;
 }
 
 }  // namespace
 
-// The loader-wavefront kernel pays off where a workgroup streams three or
-// four tiles over eight K-slices at a time (measured 3-5 % faster on 4096 x
-// 14336 and 4096 x 28672 four-bit weights; with two tiles a workgroup the
-// activation items outweigh the tiles and it is 13 % slower).  Eight compute
-// and four loader wavefronts.  Everything else stays on the self-loading
-// kernel.
-bool skinny2_supported(int64_t K, int bits, int waves, int rows_per_wg) {
-  (void)K; (void)bits;
-  return waves == 8 && rows_per_wg > 32 && rows_per_wg <= 64;
+void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
+
+// Does the loader-wavefront kernel serve this shape, and with how many rows a
+// workgroup?  The ring variant pays off where a workgroup streams three or
+// four tiles over eight K-slices at a time (with two tiles a workgroup its
+// activation items outweigh the tiles and the self-loading kernel is 13 %
+// faster).  Eight compute and four loader wavefronts either way.
+bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg) {
+  int waves, rows;
+  skinny_geometry(N, K, bits, &waves, &rows);
+  if (waves != 8) return false;
+  if (direct_x(M, K, bits)) {
+    const int64_t cus = device_cus();
+    const int64_t per = ceil_div(N, cus);
+    const int64_t rounds = ceil_div(per, 128);
+    int64_t r = ceil_div(N, cus * rounds);
+    if (r < 16) r = 16;
+    *rows_per_wg = (int)r;
+    return true;
+  }
+  *rows_per_wg = rows;
+  return rows > 32 && rows <= 64;
 }
 
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {
   GemvArgs a = a0;
   a.gshift = gs == 128 ? 1 : 0;
-  if (bits == 4) launch_g<4>(a, batch, rows, st);
-  else launch_g<8>(a, batch, rows, st);
+  const bool xd = direct_x(a.M, a.K, bits);
+  if (bits == 4) launch_k<4, 8, 4, 4>(a, batch, rows, xd, st);
+  else launch_k<8, 8, 4, 4>(a, batch, rows, xd, st);
 }
 
 }  // namespace qmm

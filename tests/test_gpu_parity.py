@@ -243,6 +243,13 @@ def test_gemv_batched():
     (8, 64, 7, 12000, 4096),     # eight-bit codes, two passes, three tiles a workgroup
     (4, 128, 16, 9000, 8192),    # two passes, group 128
     (4, 64, 3, 10000, 12288),    # three passes
+    (4, 64, 4, 28672, 4096),     # few rows of activations, one pass: 112 rows = seven tiles a workgroup
+    (4, 64, 1, 28001, 4096),     # the same with N odd: the last tile ragged, the last workgroup short
+    (8, 64, 8, 40000, 2048),     # eight-bit codes in one pass; two rounds of workgroups, five tiles each
+    (4, 128, 8, 20000, 4096),    # group 128, five tiles a workgroup
+    (4, 64, 8, 4100, 4096),      # one pass, small N: one tile a workgroup, 17 rows -> a ragged second tile
+    (4, 64, 3, 2048, 4096),      # fewer workgroups than compute units
+    (8, 128, 5, 6144, 2048),     # eight-bit codes, group 128, two tiles a workgroup
 ])
 def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     """Shapes big enough for the decode kernel whose loader wavefronts stream
