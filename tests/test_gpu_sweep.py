@@ -108,3 +108,32 @@ def test_grouped_and_gathered_random_case(seed):
                       torch.from_numpy(rhs[perm]).to(DEV), group_size=gs, bits=bits,
                       out_dtype=torch.float32).float().cpu().numpy()
     assert O.rel_l2(yg, want[perm]) <= 2e-5, (e, n, k, gs, bits, O.rel_l2(yg, want[perm]))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_one_pass_decode_random_case(seed):
+    """Decode shapes whose K is exactly one pass of eight 256-byte slices (the
+    kernel whose compute wavefronts fetch their own activations when M <= 8):
+    any number of tiles a workgroup, ragged last tiles, several rounds of
+    workgroups, a leading batch axis, both output types."""
+    rng = np.random.default_rng(9100 + seed)
+    bits = int(rng.choice([4, 8]))
+    k = 4096 if bits == 4 else 2048
+    gs = int(rng.choice([64, 128]))
+    m = int(rng.integers(1, 13))                       # above 8 the ring variant takes over
+    n = int(rng.choice([rng.integers(16, 600), rng.integers(600, 9000), rng.integers(9000, 36000)]))
+    batch = int(rng.choice([1, 1, 2])) if n < 9000 else 1
+    lead = (batch,) if batch > 1 else ()
+    codes = rng.integers(0, 1 << bits, size=lead + (n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    s = O.round_bf16(rng.uniform(0.005, 0.02, lead + (n, k // gs)).astype(np.float32))
+    b = O.round_bf16(-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s)
+    x = O.round_bf16(rng.standard_normal(lead + (m, k)).astype(np.float32))
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    y32 = K.quantized_matmul(_bf16_dev(x), wd, _bf16_dev(s), _bf16_dev(b), group_size=gs, bits=bits,
+                             out_dtype=torch.float32).float().cpu().numpy()
+    want = O.qmm(x, words, s, b, gs, bits)
+    err = O.rel_l2(y32, want)
+    assert err <= 2e-5, (m, n, k, gs, bits, batch, err)
+    y16 = K.quantized_matmul(_bf16_dev(x), wd, _bf16_dev(s), _bf16_dev(b), group_size=gs, bits=bits)
+    np.testing.assert_array_equal(y16.float().cpu().numpy(), O.round_bf16(y32))
