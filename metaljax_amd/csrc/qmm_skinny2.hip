@@ -575,12 +575,15 @@ int device_cus() {
 // rows of activations: the variant whose compute wavefronts fetch their own
 // activations.  Its tile loop is a real loop, so a workgroup takes as many
 // rows as make the grid one workgroup per compute unit (or a whole number of
-// such rounds), up to 128.
-bool direct_x(int64_t M, int64_t K, int bits) {
+// such rounds), up to 128.  With more than eight rows of activations their
+// direct fetch costs 2-4 us more than the ring's rounds, which still pays
+// where the ring variant (at most 64 rows a workgroup) would need a second
+// round of workgroups (28672 x 4096 at M = 16: 17 against 22 us).
+bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
   static const int force = env ? atoi(env) : -1;
   if (K * bits / 8 / 256 != 8) return false;
-  return force >= 0 ? force != 0 : M <= 8;
+  return force >= 0 ? force != 0 : M <= 8 || ceil_div(N, (int64_t)device_cus()) > 64;
 }
 
 }  // namespace
@@ -596,7 +599,7 @@ bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg) {
   int waves, rows;
   skinny_geometry(N, K, bits, &waves, &rows);
   if (waves != 8) return false;
-  if (direct_x(M, K, bits)) {
+  if (direct_x(M, N, K, bits)) {
     const int64_t cus = device_cus();
     const int64_t per = ceil_div(N, cus);
     const int64_t rounds = ceil_div(per, 128);
@@ -612,7 +615,7 @@ bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg) {
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {
   GemvArgs a = a0;
   a.gshift = gs == 128 ? 1 : 0;
-  const bool xd = direct_x(a.M, a.K, bits);
+  const bool xd = direct_x(a.M, a.N, a.K, bits);
   if (bits == 4) launch_k<4, 8, 4, 4>(a, batch, rows, xd, st);
   else launch_k<8, 8, 4, 4>(a, batch, rows, xd, st);
 }

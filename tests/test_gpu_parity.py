@@ -250,6 +250,8 @@ def test_gemv_batched():
     (4, 64, 8, 4100, 4096),      # one pass, small N: one tile a workgroup, 17 rows -> a ragged second tile
     (4, 64, 3, 2048, 4096),      # fewer workgroups than compute units
     (8, 128, 5, 6144, 2048),     # eight-bit codes, group 128, two tiles a workgroup
+    (4, 64, 16, 28672, 4096),    # sixteen rows of activations, wide weight: seven tiles a workgroup, activations fetched directly
+    (8, 64, 13, 17000, 2048),    # the same with eight-bit codes and a ragged last tile
 ])
 def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     """Shapes big enough for the decode kernel whose loader wavefronts stream
