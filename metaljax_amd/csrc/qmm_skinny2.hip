@@ -16,21 +16,25 @@
 //
 // Two variants (template flag XD):
 //
-// * ring variant (XD = 0; several passes over K, or more than eight rows of
-//   activations): activations and weight tiles both travel through the ring,
-//   as described below;
-// * direct variant (XD = 1; K is exactly one pass and M <= 8): each compute
-//   wavefront fetches its own K-slice of the activations straight into MFMA
-//   operand registers at the start of the kernel, every ring slot holds a
-//   weight tile, and the tile loop is a real loop in both roles, so a
-//   workgroup can take any number of tiles (the host deals up to 128 rows a
-//   workgroup so that a 28672-row weight is still one workgroup per compute
-//   unit).  The loaders keep two tiles requested: tile g+1 before tile g is
-//   published, tile g+2 right after -- issuing a tile takes about as long as
-//   receiving one, and a wavefront stuck in issue cannot publish.  Measured
-//   on 4096 x 14336 four-bit weights: 10.3 us at M = 1 against 11.9 us for the
-//   ring variant; at M = 16 the 128 KB of activations in front of the first
-//   tile cost more than the ring's interleaving (13.3 against 12.8 us).
+// * ring variant (XD = 0; more than eight rows of activations on a weight of
+//   at most 64 rows per compute unit): activations and weight tiles both
+//   travel through the ring, as described below;
+// * direct variant (M <= 8, or any M where the weight is wide enough for the
+//   ring variant to need a second round of workgroups): each compute wavefront
+//   fetches its own K-slice of the activations straight into MFMA operand
+//   registers when a pass begins, every ring slot holds a weight tile, and the
+//   loaders' tile loop is a real loop.  XD = 1, K exactly one pass: the compute
+//   wavefronts' tile loop is a real loop too, any number of tiles, a tile's
+//   sums leave for LDS at once; XD = 2, several passes: the tiles' sums stay in
+//   registers from pass to pass (at most eight tiles, unrolled).  The host
+//   deals up to 128 rows a workgroup, so that a 28672-row weight is still one
+//   workgroup per compute unit.  The loaders keep two tiles requested: tile
+//   g+1 before tile g is published, tile g+2 right after -- issuing a tile
+//   takes about as long as receiving one, and a wavefront stuck in issue
+//   cannot publish.  Measured on 4096 x 14336 four-bit weights: 10.3 us at
+//   M = 1 against 11.9 us for the ring variant; at M = 16 the 128 KB of
+//   activations in front of the first tile cost more than the ring's
+//   interleaving (13.3 against 12.8 us).
 //
 // Items of one pass (a pass = CW consecutive K-slices, one per compute
 // wavefront; a slice = 256 packed bytes per row):
@@ -272,22 +276,27 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // items out -- item g+1 is requested before item g is published, g+2
       // right after -- and no more (refilling two slots after a publication
       // measured 0.5 us slower).
-      // One pass only (the host sees to it), any number of tiles.
+      // Item g = pass g / ntiles, tile g % ntiles, in slot g % 4; any number of
+      // tiles with one pass, up to TMAX (accumulators in registers) with more.
       static_assert(!XD || S::B == 4, "two items in flight, one being consumed, one being reduced");
-      const int G = ntiles;
-      issue_tile(0, 0, 0);
-      if (G > 1) issue_tile(0, 1, 1);
+      const int G = passes * ntiles;
+      auto issue = [&](int g) __attribute__((always_inline)) {
+        const int p = g / ntiles;
+        issue_tile(p, g - p * ntiles, g & 3);
+      };
+      issue(0);
+      if (G > 1) issue(1);
 #pragma nounroll
       for (int g = 0; g < G; ++g) {
         // item g has landed: only item g+1 may still be out (a store in
         // between only tightens the wait)
         if (g + 1 < G) wait_vmcnt<LT>(); else wait_vmcnt<0>();
         item_barrier();                           // item g published; item g-1 consumed
-        if (g + 2 < G) issue_tile(0, g + 2, (g + 2) & 3);   // that slot's last tile was reduced a step ago
-        if (g >= 1) reduce_tile(0, g - 1, (g - 1) & 3);
+        if (g + 2 < G) issue(g + 2);              // that slot's last tile was consumed (and, in the last pass, reduced) a step ago
+        if (g >= 1 && g - 1 >= G - ntiles) reduce_tile(passes - 1, g - 1 - (G - ntiles), (g - 1) & 3);
       }
       item_barrier();                             // everything consumed
-      reduce_tile(0, G - 1, (G - 1) & 3);
+      reduce_tile(passes - 1, ntiles - 1, (G - 1) & 3);
       return;
     }
     // Slot of every item of the current pass (by order of use) and of the next
@@ -351,7 +360,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if constexpr (TMAX > 3) slot = t == 3 ? sl_cur[XR + (TMAX > 3 ? 3 : 0)] : slot;
         reduce_tile(p, t, slot);
       }
-      static_assert(TMAX <= 4, "the tile loop names at most four tiles");
+      static_assert(XD || TMAX <= 4, "the tile loop names at most four tiles");
       prev_last = sl_cur[NI - 1];
 #pragma unroll
       for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k];
@@ -443,37 +452,64 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       return at;
     };
     if constexpr (XD) {
-      // One pass.  This wavefront's slice of the activations straight from
+      // This wavefront's slice of pass p of the activations straight from
       // global memory (L2 after the first workgroup) into operand layout: lane
       // (r, kg) takes pieces 2*kg and 2*kg + 1 of every chunk of row r.
-      const bool active = wave < slices;          // uniform
-      u32x4 raw[CPS][2];
-      const uint32_t so = active ? (uint32_t)(wave * KS) * 2u : 0u;
+      auto fetch_x = [&](int p, bool active) __attribute__((always_inline)) {
+        u32x4 raw[CPS][2];
+        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
 #pragma unroll
-      for (int c = 0; c < CPS; ++c)
+        for (int c = 0; c < CPS; ++c)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
-              rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
+          for (int j = 0; j < 2; ++j)
+            raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
+                rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
 #pragma unroll
-      for (int c = 0; c < CPS; ++c)
+        for (int c = 0; c < CPS; ++c)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
-          else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
-        }
-      if (active) chunk_sums();
-      // The tiles as a real loop (any number of them): a tile's sums leave for
-      // its slot at once, where the loaders add up the slices.
+          for (int j = 0; j < 2; ++j) {
+            if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
+            else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
+          }
+        if (active) chunk_sums();
+      };
+      if constexpr (XD == 1) {
+        // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
+        // for its slot at once, where the loaders add up the slices.
+        const bool active = wave < slices;        // uniform
+        fetch_x(0, active);
 #pragma nounroll
-      for (int g = 0; g < ntiles; ++g) {
-        item_barrier();
-        const int slot = g & 3;
-        f32x4 at = zero;
-        if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
-        float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
+        for (int g = 0; g < ntiles; ++g) {
+          item_barrier();
+          const int slot = g & 3;
+          f32x4 at = zero;
+          if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
+          float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
+          for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
+        }
+      } else {
+        // Several passes: the tiles' sums stay in registers from pass to pass
+        // (at most TMAX tiles, unrolled); the next pass's activations are
+        // fetched when the pass begins.
+        for (int p = 0; p < passes; ++p) {
+          const bool active = p * CW + wave < slices;   // uniform
+          fetch_x(p, active);
+          static_for<TMAX>([&](auto tc) __attribute__((always_inline)) {
+            constexpr int t = decltype(tc)::value;
+            if (t < ntiles) {
+              item_barrier();
+              const int slot = (p * ntiles + t) & 3;
+              if (active)
+                acc[t] = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, acc[t]);
+              if (p == passes - 1) {
+                float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) part[e * kWave + lane] = acc[t][e];
+              }
+            }
+          });
+        }
       }
       item_barrier();                             // everything consumed
       return;
@@ -548,15 +584,10 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);
 }
 
-template <int BITS, int CW, int NL, int TMAX>
-void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, bool xd, hipStream_t st) {
-  if (xd) {
-    if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, 1>(a, batch, rows_per_wg, st);
-    else launch_one<BITS, CW, NL, TMAX, 0, 1>(a, batch, rows_per_wg, st);
-  } else {
-    if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, 0>(a, batch, rows_per_wg, st);
-    else launch_one<BITS, CW, NL, TMAX, 0, 0>(a, batch, rows_per_wg, st);
-  }
+template <int BITS, int CW, int NL, int TMAX, int XD>
+void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
+  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st);
+  else launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st);
 }
 
 int device_cus() {
@@ -582,8 +613,17 @@ int device_cus() {
 bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
   static const int force = env ? atoi(env) : -1;
-  if (K * bits / 8 / 256 != 8) return false;
-  return force >= 0 ? force != 0 : M <= 8 || ceil_div(N, (int64_t)device_cus()) > 64;
+  if (force >= 0) return force != 0;
+  const int64_t per = ceil_div(N, (int64_t)device_cus());
+  if (M > 8 && per <= 64) return false;
+  // Several passes over K: the next pass's activations are fetched when the
+  // pass begins, which costs about 0.8 us a pass; measured against the other
+  // kernels at M = 4 (us): 28672 x 8192 30.8 / 38.4, 57344 x 8192 61 / 79,
+  // 10240 x 8192 16.1 / 18.3, eight-bit 14336 x 4096 16.7 / 18.6 and 22016 x
+  // 4096 25.2 / 30.8, but 8192 x 8192 14.2 / 12.9 and 4096 x 14336 15.3 / 12.3:
+  // it pays from three tiles a workgroup on.
+  if (K * bits / 8 / 256 != 8) return per > 32;
+  return true;
 }
 
 }  // namespace
@@ -616,8 +656,19 @@ void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int r
   GemvArgs a = a0;
   a.gshift = gs == 128 ? 1 : 0;
   const bool xd = direct_x(a.M, a.N, a.K, bits);
-  if (bits == 4) launch_k<4, 8, 4, 4>(a, batch, rows, xd, st);
-  else launch_k<8, 8, 4, 4>(a, batch, rows, xd, st);
+  if (xd) {                                       // up to eight tiles' sums in registers over several passes
+    const bool one_pass = a.K * bits / 8 / 256 <= 8;
+    if (one_pass) {
+      if (bits == 4) launch_k<4, 8, 4, 4, 1>(a, batch, rows, st);
+      else launch_k<8, 8, 4, 4, 1>(a, batch, rows, st);
+    } else {
+      if (bits == 4) launch_k<4, 8, 4, 8, 2>(a, batch, rows, st);
+      else launch_k<8, 8, 4, 8, 2>(a, batch, rows, st);
+    }
+    return;
+  }
+  if (bits == 4) launch_k<4, 8, 4, 4, 0>(a, batch, rows, st);
+  else launch_k<8, 8, 4, 4, 0>(a, batch, rows, st);
 }
 
 }  // namespace qmm

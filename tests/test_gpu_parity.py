@@ -252,6 +252,10 @@ def test_gemv_batched():
     (8, 128, 5, 6144, 2048),     # eight-bit codes, group 128, two tiles a workgroup
     (4, 64, 16, 28672, 4096),    # sixteen rows of activations, wide weight: seven tiles a workgroup, activations fetched directly
     (8, 64, 13, 17000, 2048),    # the same with eight-bit codes and a ragged last tile
+    (4, 64, 4, 28672, 8192),     # two passes with directly fetched activations, seven tiles' sums in registers
+    (4, 128, 7, 20000, 6144),    # the second pass half empty, five tiles, group 128
+    (8, 64, 2, 22016, 4096),     # eight-bit codes, two passes, six tiles
+    (4, 64, 16, 30000, 12288),   # sixteen rows, wide weight, three passes, eight tiles (the last ragged)
 ])
 def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     """Shapes big enough for the decode kernel whose loader wavefronts stream
