@@ -180,6 +180,13 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   f32x4 acc[TMAX];
 #pragma unroll
   for (int t = 0; t < TMAX; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // Row packing (several passes, direct variant): the operand's sixteen rows
+  // hold the activations of every pass at once -- rows [q*PK, q*PK + M) are
+  // the M rows of x over pass q's K-slices -- so nothing is fetched between
+  // passes.  A tile of pass p then yields meaningful sums only in row block p
+  // (the other blocks multiply another pass's activations with this pass's
+  // weights and are masked off), and the blocks are added up at the end.
+  const int PK = XD != 2 ? 0 : (passes <= 2 && a.M <= 8) ? 8 : (passes <= 4 && a.M <= 4) ? 4 : 0;
 
   if (wave >= CW) {
     // ------------------------------------------------------------ loaders ----
@@ -263,9 +270,16 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         float v = 0.f;
 #pragma unroll
         for (int wv = 0; wv < CW; ++wv) v += part[wv * 1024 + e * kWave + lane];
+        if constexpr (XD == 2) {
+          if (PK != 0) {                            // row blocks of the passes -> rows [0, PK)
+            v += __shfl_xor(v, 32);
+            if (PK == 4) v += __shfl_xor(v, 16);
+          }
+        }
         const int m = 4 * (lane >> 4) + e;
         const int64_t n = n_begin + t * 16 + (lane & 15);
-        if (m < a.M && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+        const bool row_ok = m < a.M && (PK == 0 || m < PK);
+        if (row_ok && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
       }
     };
     if constexpr (XD) {
@@ -455,7 +469,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // This wavefront's slice of pass p of the activations straight from
       // global memory (L2 after the first workgroup) into operand layout: lane
       // (r, kg) takes pieces 2*kg and 2*kg + 1 of every chunk of row r.
-      auto fetch_x = [&](int p, bool active) __attribute__((always_inline)) {
+      auto fetch_x = [&](int p, bool active, uint32_t lane_off) __attribute__((always_inline)) {
         u32x4 raw[CPS][2];
         const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
 #pragma unroll
@@ -463,7 +477,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
           for (int j = 0; j < 2; ++j)
             raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
-                rxc, active ? xlane + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
+                rxc, active ? lane_off + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
 #pragma unroll
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
@@ -477,7 +491,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
         const bool active = wave < slices;        // uniform
-        fetch_x(0, active);
+        fetch_x(0, active, xlane);
 #pragma nounroll
         for (int g = 0; g < ntiles; ++g) {
           item_barrier();
@@ -492,16 +506,31 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // Several passes: the tiles' sums stay in registers from pass to pass
         // (at most TMAX tiles, unrolled); the next pass's activations are
         // fetched when the pass begins.
+        if (PK != 0) {
+          // every pass's activations at once: lane row r = q*PK + m reads row m
+          // over the K-slice of pass q (lanes past M, past the passes or past
+          // the last slice read zeros)
+          const int q = r / PK, m = r - q * PK;
+          const bool ok = m < a.M && q * CW + wave < slices;
+          const uint32_t off = ok ? (uint32_t)((int64_t)m * a.K * 2) + (uint32_t)kg * 32u + (uint32_t)(q * CW * KS) * 2u
+                                  : kOutOfRange;
+          fetch_x(0, wave < slices, off);
+        }
+        const int my_pass = PK == 8 ? kg >> 1 : kg;   // the pass whose sums this lane's accumulator rows hold
         for (int p = 0; p < passes; ++p) {
           const bool active = p * CW + wave < slices;   // uniform
-          fetch_x(p, active);
+          if (PK == 0) fetch_x(p, active, xlane);
           static_for<TMAX>([&](auto tc) __attribute__((always_inline)) {
             constexpr int t = decltype(tc)::value;
             if (t < ntiles) {
               item_barrier();
               const int slot = (p * ntiles + t) & 3;
-              if (active)
-                acc[t] = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, acc[t]);
+              if (active) {
+                const f32x4 d = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
+                const bool mine = PK == 0 || my_pass == p;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[t][e] += mine ? d[e] : 0.f;
+              }
               if (p == passes - 1) {
                 float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
 #pragma unroll
@@ -622,7 +651,14 @@ bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   // 10240 x 8192 16.1 / 18.3, eight-bit 14336 x 4096 16.7 / 18.6 and 22016 x
   // 4096 25.2 / 30.8, but 8192 x 8192 14.2 / 12.9 and 4096 x 14336 15.3 / 12.3:
   // it pays from three tiles a workgroup on.
-  if (K * bits / 8 / 256 != 8) return per > 32;
+  const int64_t slices = K * bits / 8 / 256;
+  if (slices != 8) {
+    // ... unless the kernel can pack every pass's activations into the sixteen
+    // operand rows at once (passes x M <= 16), which takes the fetches away
+    const int64_t passes = ceil_div(slices, (int64_t)8);
+    const bool packs = (passes <= 2 && M <= 8) || (passes <= 4 && M <= 4);
+    return per > 32 || packs;
+  }
   return true;
 }
 

@@ -256,6 +256,12 @@ def test_gemv_batched():
     (4, 128, 7, 20000, 6144),    # the second pass half empty, five tiles, group 128
     (8, 64, 2, 22016, 4096),     # eight-bit codes, two passes, six tiles
     (4, 64, 16, 30000, 12288),   # sixteen rows, wide weight, three passes, eight tiles (the last ragged)
+    (4, 64, 4, 4096, 14336),     # 3.5 passes, four rows: every pass's activations packed into the operand's row blocks of four
+    (4, 64, 3, 4100, 12288),     # three passes packed by four (one block unused), ragged second tile
+    (4, 128, 8, 8192, 8192),     # two passes packed by eight rows, two tiles a workgroup
+    (8, 64, 5, 6144, 4096),      # eight-bit codes, two passes packed by eight
+    (4, 64, 1, 5000, 14336),     # one row, 3.5 passes
+    (4, 64, 5, 4096, 14336),     # five rows do not pack into four passes: the self-loading kernel
 ])
 def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     """Shapes big enough for the decode kernel whose loader wavefronts stream
