@@ -14,6 +14,12 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
+bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
+                               const void* s, const void* b, int64_t E);
+void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
+                              int y_dtype, const int32_t* row_offsets, const int32_t* src_row,
+                              const int32_t* out_row, int64_t P, int64_t T, int64_t E, int64_t N,
+                              int64_t K, int gs, int bits, hipStream_t st);
 void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
@@ -66,6 +72,10 @@ constexpr int64_t kGemvMaxM = 16;
 // Pairs at or below which the gather form runs one decode launch per pair
 // instead of sorting rows by expert.
 constexpr int64_t kGatherGemvMaxPairs = 64;
+// From this many pairs on (and up to kGatherGemvMaxPairs) the pairs are sorted
+// by expert and every expert's weight is streamed once (grouped decode); below
+// it the sort's launch costs more than a shared expert saves.
+constexpr int64_t kGroupedDecodeMinPairs = 4;
 
 int check_quant(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* w,
                 const void* s, const void* b) {
@@ -167,7 +177,8 @@ size_t qmm_workspace_bytes(int64_t, int64_t M, int64_t N, int64_t K, int, int, i
 }
 
 size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K) {
-  if (P <= kGatherGemvMaxPairs) return 0;
+  if (P < kGroupedDecodeMinPairs) return 0;
+  if (P <= kGatherGemvMaxPairs) return route_bytes(P, E);    // the expert sort of the grouped decode
   // the expert sort's arrays, then (when the register-operand kernel serves
   // the shape) the re-laid copy of the gathered activation rows
   size_t relaid = gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0;
@@ -340,6 +351,22 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   if (P > INT32_MAX / 2 || N > INT32_MAX || K > INT32_MAX || E > 65535 || T * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  static const bool no_grouped_decode = getenv("QMM_NO_GROUPED_DECODE") != nullptr;
+  if (P >= kGroupedDecodeMinPairs && P <= kGatherGemvMaxPairs && !no_grouped_decode && workspace &&
+      workspace_bytes >= route_bytes(P, E) &&
+      skinny2_grouped_supported(N, K, group_size, bits, mode, table_dtype, scales, biases, E)) {
+    int32_t* ro = static_cast<int32_t*>(workspace);
+    int32_t* cursor = ro + E + 1;
+    int32_t* src_row = cursor + E;
+    int32_t* out_row = src_row + P;
+    hipLaunchKernelGGL(route_kernel, dim3(1), dim3(1024), 0, st, lhs_idx, rhs_idx, (int)P, (int)E,
+                       ro, cursor, src_row, out_row);
+    rc = check_launch("route launch");
+    if (rc) return rc;
+    skinny2_grouped_dispatch(x, w, scales, biases, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
+                             group_size, bits, st);
+    return check_launch("grouped decode launch");
+  }
   if (P <= kGatherGemvMaxPairs) {
     gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, P, 1, N, K, group_size, bits,
                   mode, lhs_idx, rhs_idx, st);

@@ -57,6 +57,14 @@ struct GemvArgs {
   // gather form: batch entry z multiplies x[lhs_idx[z]] by w[rhs_idx[z]]
   const int32_t* lhs_idx;
   const int32_t* rhs_idx;
+  // grouped decode (loader-wavefront kernel, direct variants): workgroup row
+  // (blockIdx.y = expert e, blockIdx.z = chunk c) multiplies the up to sixteen
+  // rows x[src_row[row_offsets[e] + 16 c + r]] by w[e] and stores row r at
+  // y[out_row[row_offsets[e] + 16 c + r]]; x has x_rows rows
+  const int32_t* row_offsets = nullptr;
+  const int32_t* src_row = nullptr;
+  const int32_t* out_row = nullptr;
+  int x_rows = 0;
 };
 
 // Keeps a loop-invariant constant in a vector register: gfx950's three-operand

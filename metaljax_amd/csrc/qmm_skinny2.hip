@@ -174,8 +174,22 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   const int slices = a.K / KS;
   const int passes = (slices + CW - 1) / CW;
 
-  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
-  const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  // Rows of activations of this workgroup: a.M, or in the grouped form (direct
+  // variants only) what expert blockIdx.y has in chunk blockIdx.z.
+  int M = a.M;
+  const int32_t* src_row = nullptr;
+  const int32_t* out_row = nullptr;
+  if (XD != 0 && a.row_offsets) {
+    const int lo = a.row_offsets[bz] + 16 * (int)blockIdx.z, hi = a.row_offsets[bz + 1];
+    M = hi - lo < 16 ? hi - lo : 16;
+    if (M <= 0) return;                           // uniform: before any barrier
+    src_row = a.src_row + lo;
+    out_row = a.out_row + lo;
+    xz = 0;
+    wz = bz;
+  }
 
   f32x4 acc[TMAX];
 #pragma unroll
@@ -186,7 +200,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   // passes.  A tile of pass p then yields meaningful sums only in row block p
   // (the other blocks multiply another pass's activations with this pass's
   // weights and are masked off), and the blocks are added up at the end.
-  const int PK = XD != 2 ? 0 : (passes <= 2 && a.M <= 8) ? 8 : (passes <= 4 && a.M <= 4) ? 4 : 0;
+  const int PK = XD != 2 ? 0 : (passes <= 2 && M <= 8) ? 8 : (passes <= 4 && M <= 4) ? 4 : 0;
 
   if (wave >= CW) {
     // ------------------------------------------------------------ loaders ----
@@ -278,8 +292,10 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         }
         const int m = 4 * (lane >> 4) + e;
         const int64_t n = n_begin + t * 16 + (lane & 15);
-        const bool row_ok = m < a.M && (PK == 0 || m < PK);
-        if (row_ok && n < n_end) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+        const bool row_ok = m < M && (PK == 0 || m < PK);
+        int64_t yrow = bz * a.M + m;
+        if (out_row) yrow = row_ok ? (int64_t)out_row[m] : -1;
+        if (row_ok && yrow >= 0 && n < n_end) store_out(a.y, yrow * (int64_t)a.N + n, v, a.y_dtype);
       }
     };
     if constexpr (XD) {
@@ -388,8 +404,17 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const bf16x8 ones = as_bf16x8(one, one, one, one);
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
     const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
-    const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
-    const uint32_t xlane = r < a.M ? (uint32_t)((int64_t)r * a.K * 2) + (uint32_t)kg * 32u : kOutOfRange;
+    // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
+    const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
+    const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, xrows * a.K * 2);
+    auto xrow = [&](int m) -> int64_t {
+      if (m >= M) return -1;
+      if (!src_row) return m;
+      const int64_t sr = src_row[m];
+      return sr < xrows ? sr : -1;
+    };
+    const int64_t xr0 = xrow(r);
+    const uint32_t xlane = xr0 >= 0 ? (uint32_t)(xr0 * a.K * 2) + (uint32_t)kg * 32u : kOutOfRange;
     int sl_cur[NI], sl_nxt[NI], prev_last = 0;     // the loaders' slot bookkeeping, mirrored
 #pragma unroll
     for (int k = 0; k < NI; ++k) sl_cur[k] = sl_nxt[k] = 0;
@@ -511,9 +536,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           // over the K-slice of pass q (lanes past M, past the passes or past
           // the last slice read zeros)
           const int q = r / PK, m = r - q * PK;
-          const bool ok = m < a.M && q * CW + wave < slices;
-          const uint32_t off = ok ? (uint32_t)((int64_t)m * a.K * 2) + (uint32_t)kg * 32u + (uint32_t)(q * CW * KS) * 2u
-                                  : kOutOfRange;
+          const int64_t xr = q * CW + wave < slices ? xrow(m) : -1;
+          const uint32_t off = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)kg * 32u + (uint32_t)(q * CW * KS) * 2u
+                                       : kOutOfRange;
           fetch_x(0, wave < slices, off);
         }
         const int my_pass = PK == 8 ? kg >> 1 : kg;   // the pass whose sums this lane's accumulator rows hold
@@ -598,8 +623,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 }
 
 template <int BITS, int CW, int NL, int TMAX, int GSHIFT, int XD>
-void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch);
+void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st, int chunks = 1) {
+  dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
   constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
   const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
@@ -614,9 +639,9 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
 }
 
 template <int BITS, int CW, int NL, int TMAX, int XD>
-void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st) {
-  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st);
-  else launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st);
+void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st, int chunks = 1) {
+  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
+  else launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st, chunks);
 }
 
 int device_cus() {
@@ -705,6 +730,53 @@ void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int r
   }
   if (bits == 4) launch_k<4, 8, 4, 4, 0>(a, batch, rows, st);
   else launch_k<8, 8, 4, 4, 0>(a, batch, rows, st);
+}
+
+bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* s,
+                      const void* b);
+
+// Grouped decode: the pairs of an expert-indexed product, sorted by expert
+// (row_offsets / src_row / out_row as the routing pass writes them), as one
+// decode product per expert and chunk of sixteen rows: every expert's weight
+// is streamed once however many pairs name it.  Grid y = expert, z = chunk;
+// workgroups whose expert has no rows in their chunk leave at once.
+bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
+                               const void* s, const void* b, int64_t E) {
+  if (!skinny_supported(N, K, gs, bits, mode, tab, s, b)) return false;
+  return K * bits / 8 / 256 >= 8 && E <= 65535;
+}
+
+void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
+                              int y_dtype, const int32_t* row_offsets, const int32_t* src_row,
+                              const int32_t* out_row, int64_t P, int64_t T, int64_t E, int64_t N,
+                              int64_t K, int gs, int bits, hipStream_t st) {
+  GemvArgs a;
+  a.x = static_cast<const uint16_t*>(x);
+  a.w = static_cast<const uint32_t*>(w);
+  a.s = s;
+  a.b = b;
+  a.y = y;
+  a.M = 1; a.N = (int)N; a.K = (int)K;
+  a.gshift = gs == 128 ? 1 : 0;
+  a.y_dtype = y_dtype;
+  a.lhs_idx = nullptr;
+  a.rhs_idx = nullptr;
+  a.row_offsets = row_offsets;
+  a.src_row = src_row;
+  a.out_row = out_row;
+  a.x_rows = (int)T;
+  const int64_t cus = device_cus();
+  const int64_t rounds = ceil_div(ceil_div(N, cus), (int64_t)128);
+  int64_t rows = ceil_div(N, cus * rounds);
+  if (rows < 16) rows = 16;
+  const int chunks = (int)ceil_div(P, (int64_t)16);          // all pairs may name one expert
+  if (K * bits / 8 / 256 <= 8) {
+    if (bits == 4) launch_k<4, 8, 4, 4, 1>(a, E, (int)rows, st, chunks);
+    else launch_k<8, 8, 4, 4, 1>(a, E, (int)rows, st, chunks);
+  } else {
+    if (bits == 4) launch_k<4, 8, 4, 8, 2>(a, E, (int)rows, st, chunks);
+    else launch_k<8, 8, 4, 8, 2>(a, E, (int)rows, st, chunks);
+  }
 }
 
 }  // namespace qmm

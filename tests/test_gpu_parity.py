@@ -702,3 +702,63 @@ def test_unsupported_and_bad_shapes_raise_without_launching():
         K.quantized_matmul(x, w, s, None, group_size=64, bits=4)       # affine without biases
     with pytest.raises(K.QmmError):
         K.quantized_matmul(x.cpu(), w, s, s, group_size=64, bits=4)    # no CPU path
+
+
+@pytest.mark.parametrize("bits,gs,t,pairs,e,n,k,skew", [
+    (4, 64, 4, 8, 8, 9000, 4096, False),       # top-2 of eight experts for four tokens
+    (4, 64, 16, 32, 4, 5000, 4096, False),     # eight pairs an expert on average
+    (4, 128, 24, 48, 3, 2100, 4096, True),     # most pairs on one expert: more than sixteen rows = several chunks
+    (8, 64, 6, 12, 5, 3000, 2048, False),      # eight-bit codes
+    (4, 64, 5, 10, 4, 4100, 8192, False),      # two passes over K (rows packed by eight or fetched per pass)
+    (4, 64, 30, 60, 2, 1000, 12288, True),     # three passes, up to sixteen rows an expert chunk
+])
+def test_gather_qmm_few_pairs_grouped_by_expert(bits, gs, t, pairs, e, n, k, skew):
+    """Between 4 and 64 pairs: the pairs are sorted by expert and each expert's
+    weight is streamed once against its (up to sixteen at a time) rows; results
+    come back in pair order."""
+    rng = np.random.default_rng(pairs * 31 + e)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    if skew:
+        rhs[rng.random(pairs) < 0.8] = e - 1
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, gs, bits)[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                             group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+    y16 = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                               group_size=gs, bits=bits))
+    np.testing.assert_array_equal(y16, O.round_bf16(y))
+
+
+def test_gather_qmm_few_pairs_invalid_indices_touch_nothing():
+    """Grouped decode: a pair naming no expert keeps its output row as it was,
+    a pair naming a row outside x multiplies zeros."""
+    rng = np.random.default_rng(77)
+    e, n, k, t = 4, 2048, 4096, 6
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = np.array([0, 5, 2, 9, 1, 3, -1, 4], dtype=np.int32)      # 9 and -1 are outside x
+    rhs = np.array([1, 7, 0, 2, -3, 3, 1, 1], dtype=np.int32)      # 7 and -3 name no expert
+    from metaljax_amd import _lib
+    lib = _lib.load()
+    p = len(lhs)
+    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k))
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    y = torch.full((p, n), 7.0, dtype=torch.float32, device=DEV)
+    ld, rd = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    rc = lib.qmm_gather_qmm(xd.data_ptr(), _lib.BF16, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), _lib.BF16,
+                            y.data_ptr(), _lib.F32, ld.data_ptr(), rd.data_ptr(), p, t, e, n, k, 64, 4, 0,
+                            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc)
+    got = y.cpu().numpy()
+    for i in range(p):
+        if not 0 <= rhs[i] < e:
+            np.testing.assert_array_equal(got[i], np.full(n, 7.0, np.float32))
+        elif not 0 <= lhs[i] < t:
+            np.testing.assert_array_equal(got[i], np.zeros(n, np.float32))
+        else:
+            want = O.qmm(x[lhs[i]][None], words[rhs[i]], s[rhs[i]], b[rhs[i]], 64, 4)[0]
+            assert O.rel_l2(got[i], want) <= 2e-5
