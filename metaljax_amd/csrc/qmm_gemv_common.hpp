@@ -65,6 +65,9 @@ struct GemvArgs {
   const int32_t* src_row = nullptr;
   const int32_t* out_row = nullptr;
   int x_rows = 0;
+  // streamed form (one pass over K): a workgroup walks all experts' chunks
+  // itself instead of one workgroup per (expert, chunk); experts = E
+  int experts = 0;
 };
 
 // Keeps a loop-invariant constant in a vector register: gfx950's three-operand
