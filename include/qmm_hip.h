@@ -72,9 +72,11 @@ size_t qmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int g
                            int bits, int mode, int x_dtype);
 
 /* Scratch bytes qmm_gather_qmm wants for P pairs over E experts of [N, K]
- * weights (0 when the pairs are few enough to run as independent decode
- * products): the expert sort's arrays plus the re-laid activation copy of the
- * fast kernel.  With only the sort's share the call still runs, slower. */
+ * weights (0 below four pairs, which run as independent decode products): the
+ * expert sort's arrays, plus the segment list of the grouped decode (up to
+ * 16 pairs an expert on average: one decode product per expert and sixteen
+ * pairs) or the re-laid activation copy of the prefill kernel (more pairs).
+ * With less the call still runs, on a slower kernel. */
 size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K);
 
 /* The kernel family and launch geometry the dispatcher would choose. */

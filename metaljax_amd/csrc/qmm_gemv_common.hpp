@@ -58,16 +58,14 @@ struct GemvArgs {
   const int32_t* lhs_idx;
   const int32_t* rhs_idx;
   // grouped decode (loader-wavefront kernel, direct variants): workgroup row
-  // (blockIdx.y = expert e, blockIdx.z = chunk c) multiplies the up to sixteen
-  // rows x[src_row[row_offsets[e] + 16 c + r]] by w[e] and stores row r at
-  // y[out_row[row_offsets[e] + 16 c + r]]; x has x_rows rows
-  const int32_t* row_offsets = nullptr;
+  // blockIdx.y takes segment y of `segments` ([0] = count, then (expert, first
+  // sorted position, rows <= 16) triples): it multiplies the rows
+  // x[src_row[first + r]] by w[expert] and stores row r at y[out_row[first + r]];
+  // x has x_rows rows
+  const int32_t* segments = nullptr;
   const int32_t* src_row = nullptr;
   const int32_t* out_row = nullptr;
   int x_rows = 0;
-  // streamed form (one pass over K): a workgroup walks all experts' chunks
-  // itself instead of one workgroup per (expert, chunk); experts = E
-  int experts = 0;
 };
 
 // Keeps a loop-invariant constant in a vector register: gfx950's three-operand

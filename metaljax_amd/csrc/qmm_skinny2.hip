@@ -177,23 +177,18 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
   // Rows of activations of this workgroup: a.M, or in the grouped form (direct
-  // variants only) what expert blockIdx.y has in chunk blockIdx.z.
+  // variants only) those of segment blockIdx.y.
   int M = a.M;
   const int32_t* src_row = nullptr;
   const int32_t* out_row = nullptr;
-  // streamed experts (XD == 3): the (expert, chunk) segments with at least one
-  // row, listed once per workgroup in LDS behind the ring: seg[0] = count, then
-  // (expert, first sorted position, rows) triples
-  constexpr int kSegCap = 512;
-  int* seg = reinterpret_cast<int*>(smem + S::B * (kItem + kTab));
-  if ((XD == 1 || XD == 2) && a.row_offsets) {
-    const int lo = a.row_offsets[bz] + 16 * (int)blockIdx.z, hi = a.row_offsets[bz + 1];
-    M = hi - lo < 16 ? hi - lo : 16;
-    if (M <= 0) return;                           // uniform: before any barrier
+  if (XD != 0 && a.segments) {
+    if (bz >= a.segments[0]) return;              // uniform: before any barrier
+    const int lo = a.segments[2 + 3 * bz];
+    M = a.segments[3 + 3 * bz];
     src_row = a.src_row + lo;
     out_row = a.out_row + lo;
     xz = 0;
-    wz = bz;
+    wz = a.segments[1 + 3 * bz];
   }
 
   f32x4 acc[TMAX];
@@ -211,9 +206,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // ------------------------------------------------------------ loaders ----
     const int lw = wave - CW;
     const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
-    auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
-    auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * 2, a.N * ng * 2);
-    auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * 2, a.N * ng * 2);
+    const auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
+    const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * 2, a.N * ng * 2);
+    const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * 2, a.N * ng * 2);
     const int lrow = lane >> 4, lp = lane & 15;
     // Load q of this wavefront is instruction j = lw + q*NL of the item: slice
     // j / 4, row quad j % 4 = (lw + o) % 4 with o = q*NL % 4 known at compile
@@ -303,75 +298,6 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if (row_ok && yrow >= 0 && n < n_end) store_out(a.y, yrow * (int64_t)a.N + n, v, a.y_dtype);
       }
     };
-    if constexpr (XD == 3) {
-      // Streamed experts: the first loader wavefront lists the segments, then
-      // the same two-items-out loop runs over every segment's tiles; a
-      // segment's expert selects the weight, its rows the output rows.
-      if (wave == CW) {
-        int n = 0;
-        for (int base = 0; base < a.experts; base += kWave) {
-          const int e = base + lane;
-          int lo = 0, cnt = 0;
-          if (e < a.experts) {
-            lo = a.row_offsets[e];
-            cnt = a.row_offsets[e + 1] - lo;
-            if (cnt < 0) cnt = 0;
-          }
-          const int nch = (cnt + 15) >> 4;
-          int pre = nch;                            // inclusive prefix sum over the lanes
-          for (int d = 1; d < kWave; d <<= 1) {
-            const int v = __shfl_up(pre, d);
-            if (lane >= d) pre += v;
-          }
-          const int total = __shfl(pre, kWave - 1);
-          pre -= nch;
-          for (int c = 0; c < nch; ++c) {
-            const int idx = n + pre + c;
-            if (idx < kSegCap) {
-              seg[4 + 3 * idx] = e;
-              seg[5 + 3 * idx] = lo + 16 * c;
-              seg[6 + 3 * idx] = cnt - 16 * c < 16 ? cnt - 16 * c : 16;
-            }
-          }
-          n += total;
-        }
-        if (lane == 0) seg[0] = n < kSegCap ? n : kSegCap;
-      }
-      item_barrier();                             // the list is there
-      const int nseg = seg[0];
-      const int G = nseg * ntiles;
-      if (G == 0) return;                         // uniform over the workgroup
-      int cur_e = -1;
-      auto issue = [&](int g) __attribute__((always_inline)) {
-        const int sg = g / ntiles;
-        const int e = seg[4 + 3 * sg];
-        if (e != cur_e) {
-          cur_e = e;
-          rw = make_rsrc(reinterpret_cast<const char*>(a.w) + (int64_t)e * a.N * wpr, a.N * wpr);
-          rs = make_rsrc(static_cast<const char*>(a.s) + (int64_t)e * a.N * ng * 2, a.N * ng * 2);
-          rb = make_rsrc(static_cast<const char*>(a.b) + (int64_t)e * a.N * ng * 2, a.N * ng * 2);
-        }
-        issue_tile(0, g - sg * ntiles, g & 3);
-      };
-      auto reduce = [&](int g) __attribute__((always_inline)) {
-        const int sg = g / ntiles;
-        out_row = a.out_row + seg[5 + 3 * sg];
-        M = seg[6 + 3 * sg];
-        reduce_tile(0, g - sg * ntiles, g & 3);
-      };
-      issue(0);
-      if (G > 1) issue(1);
-#pragma nounroll
-      for (int g = 0; g < G; ++g) {
-        if (g + 1 < G) wait_vmcnt<LT>(); else wait_vmcnt<0>();
-        item_barrier();                           // item g published; item g-1 consumed
-        if (g + 2 < G) issue(g + 2);
-        if (g >= 1) reduce(g - 1);
-      }
-      item_barrier();                             // everything consumed
-      reduce(G - 1);
-      return;
-    }
     if constexpr (XD) {
       // Every item is a tile: tile g lives in slot g % 4.  A load
       // instruction is accepted at the pace at which data comes back (issuing
@@ -479,7 +405,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
     const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
     // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
-    const int64_t xrows = (src_row || XD == 3) ? (int64_t)a.x_rows : (int64_t)a.M;
+    const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
     const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, xrows * a.K * 2);
     auto xrow = [&](int m) -> int64_t {
       if (m >= M) return -1;
@@ -586,32 +512,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           }
         if (active) chunk_sums();
       };
-      if constexpr (XD == 3) {
-        // Streamed experts, one pass: per segment fetch its rows' activations
-        // (gathered through the sorted row list), then its tiles.
-        item_barrier();                           // the segment list is there
-        const int nseg = seg[0];
-        const bool active = wave < slices;        // uniform
-        int g = 0;
-#pragma nounroll
-        for (int sg = 0; sg < nseg; ++sg) {
-          src_row = a.src_row + seg[5 + 3 * sg];
-          M = seg[6 + 3 * sg];
-          const int64_t xr = xrow(r);
-          fetch_x(0, active, xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)kg * 32u : kOutOfRange);
-#pragma nounroll
-          for (int t = 0; t < ntiles; ++t, ++g) {
-            item_barrier();
-            const int slot = g & 3;
-            f32x4 at = zero;
-            if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
-            float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
-          }
-        }
-        if (nseg * ntiles == 0) return;           // as the loaders do
-      } else if constexpr (XD == 1) {
+      if constexpr (XD == 1) {
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
         const bool active = wave < slices;        // uniform
@@ -726,8 +627,7 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
   constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
-  const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind) +
-                     (XD == 3 ? (4 + 3 * 512) * sizeof(int) : 0);
+  const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
   auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   static bool configured = false;                 // one flag per instantiation
   if (!configured) {
@@ -836,18 +736,22 @@ bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                       const void* b);
 
 // Grouped decode: the pairs of an expert-indexed product, sorted by expert
-// (row_offsets / src_row / out_row as the routing pass writes them), as one
-// decode product per expert and chunk of sixteen rows: every expert's weight
-// is streamed once however many pairs name it.  Grid y = expert, z = chunk;
-// workgroups whose expert has no rows in their chunk leave at once.
+// (segments / src_row / out_row as the routing pass writes them), as one
+// decode product per segment (an expert's rows, sixteen at a time): every
+// expert's weight is streamed once per sixteen pairs that name it.  Grid y =
+// segment, provisioned for the most there can be (workgroups past the count
+// leave at once; an empty workgroup still costs about a microsecond of a
+// compute unit, which is why the grid is not expert x chunk).
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E) {
   if (!skinny_supported(N, K, gs, bits, mode, tab, s, b)) return false;
-  return K * bits / 8 / 256 >= 8 && E <= 65535;
+  return K * bits / 8 / 256 >= 8;
 }
 
+int64_t skinny2_max_segments(int64_t P, int64_t E) { return (E < P ? E : P) + P / 16; }
+
 void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
-                              int y_dtype, const int32_t* row_offsets, const int32_t* src_row,
+                              int y_dtype, const int32_t* segments, const int32_t* src_row,
                               const int32_t* out_row, int64_t P, int64_t T, int64_t E, int64_t N,
                               int64_t K, int gs, int bits, hipStream_t st) {
   GemvArgs a;
@@ -861,7 +765,7 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   a.y_dtype = y_dtype;
   a.lhs_idx = nullptr;
   a.rhs_idx = nullptr;
-  a.row_offsets = row_offsets;
+  a.segments = segments;
   a.src_row = src_row;
   a.out_row = out_row;
   a.x_rows = (int)T;
@@ -869,19 +773,13 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   const int64_t rounds = ceil_div(ceil_div(N, cus), (int64_t)128);
   int64_t rows = ceil_div(N, cus * rounds);
   if (rows < 16) rows = 16;
-  const int chunks = (int)ceil_div(P, (int64_t)16);          // all pairs may name one expert
-  static const bool no_stream = getenv("QMM_NO_STREAMED_EXPERTS") != nullptr;
-  if (K * bits / 8 / 256 <= 8 && !no_stream && P + chunks <= 512) {
-    // one pass over K: a workgroup streams every expert's tiles itself
-    a.experts = (int)E;
-    if (bits == 4) launch_k<4, 8, 4, 4, 3>(a, 1, (int)rows, st);
-    else launch_k<8, 8, 4, 4, 3>(a, 1, (int)rows, st);
-  } else if (K * bits / 8 / 256 <= 8) {
-    if (bits == 4) launch_k<4, 8, 4, 4, 1>(a, E, (int)rows, st, chunks);
-    else launch_k<8, 8, 4, 4, 1>(a, E, (int)rows, st, chunks);
+  const int64_t segs = skinny2_max_segments(P, E);
+  if (K * bits / 8 / 256 <= 8) {
+    if (bits == 4) launch_k<4, 8, 4, 4, 1>(a, segs, (int)rows, st);
+    else launch_k<8, 8, 4, 4, 1>(a, segs, (int)rows, st);
   } else {
-    if (bits == 4) launch_k<4, 8, 4, 8, 2>(a, E, (int)rows, st, chunks);
-    else launch_k<8, 8, 4, 8, 2>(a, E, (int)rows, st, chunks);
+    if (bits == 4) launch_k<4, 8, 4, 8, 2>(a, segs, (int)rows, st);
+    else launch_k<8, 8, 4, 8, 2>(a, segs, (int)rows, st);
   }
 }
 
