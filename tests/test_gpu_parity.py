@@ -711,9 +711,11 @@ def test_unsupported_and_bad_shapes_raise_without_launching():
     (8, 64, 6, 12, 5, 3000, 2048, False),      # eight-bit codes
     (4, 64, 5, 10, 4, 4100, 8192, False),      # two passes over K (rows packed by eight or fetched per pass)
     (4, 64, 30, 60, 2, 1000, 12288, True),     # three passes, up to sixteen rows an expert chunk
+    (4, 64, 50, 100, 8, 3000, 4096, False),    # more than 64 pairs, still at most 16 an expert on average
+    (4, 64, 40, 120, 8, 2100, 4096, True),     # most of 120 pairs on one expert: seven of its chunks, a few others
 ])
 def test_gather_qmm_few_pairs_grouped_by_expert(bits, gs, t, pairs, e, n, k, skew):
-    """Between 4 and 64 pairs: the pairs are sorted by expert and each expert's
+    """Between 4 and 16 x E pairs: the pairs are sorted by expert and each expert's
     weight is streamed once against its (up to sixteen at a time) rows; results
     come back in pair order."""
     rng = np.random.default_rng(pairs * 31 + e)
