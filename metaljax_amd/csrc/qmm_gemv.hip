@@ -378,6 +378,8 @@ void skinny_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int ta
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st);
+bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
+void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st);
 
 // Tile / slice / unroll choice; QMM_GEMV_T, QMM_GEMV_WAVES and QMM_GEMV_U
 // override it for experiments (read once).
@@ -424,6 +426,8 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
   g.u = env_u ? env_u : 8;
   if (mode == QMM_MODE_MXFP4) {
     a.gshift = 0;
+    // big weights: the loader-wavefront kernel (activations fetched directly)
+    if (!no_skinny && skinny2_mx_supported(N, K, s)) return skinny2_mx_dispatch(a, batch, st);
     if (!env_u) g.u = 4;
     launch_mxfp4(a, batch, g, st);
     return;

@@ -36,6 +36,11 @@
 //   activations in front of the first tile cost more than the ring's
 //   interleaving (13.3 against 12.8 us).
 //
+// The direct variants also serve MXFP4 weights (template value GSHIFT = 2): the
+// hardware converter widens two E2M1 codes at a time with the 32-block's
+// power-of-two scale applied (exact in bf16), the chunks chain through the
+// MFMA accumulator, and a row's table share of a slice is its 16 scale bytes.
+//
 // Items of one pass (a pass = CW consecutive K-slices, one per compute
 // wavefront; a slice = 256 packed bytes per row):
 //   XR activation rounds  [CW slices][16 rows m][256 bytes = 128 codes of x]
@@ -170,7 +175,12 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   const int64_t n_end = n_begin + rows_per_wg < a.N ? n_begin + rows_per_wg : a.N;
   const int ntiles = (int)((n_end - n_begin + 15) / 16);        // uniform, <= TMAX
   const int64_t wpr = (int64_t)a.K * BITS / 8;                  // bytes per weight row
-  const int64_t ng = (int64_t)(a.K / 64) >> GSHIFT;             // table entries per row
+  // GSHIFT: 0 = affine, group 64; 1 = affine, group 128; 2 = MXFP4 (E2M1 codes,
+  // one E8M0 scale byte per 32 codes: a row's table share of a slice is 16 bytes
+  // in every case)
+  constexpr bool MX = GSHIFT == 2;
+  static_assert(!MX || (BITS == 4 && XD != 0), "MXFP4: four-bit codes, direct variants");
+  const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GSHIFT;   // table row = ng * 2 bytes (MXFP4: K/32 bytes)
   const int slices = a.K / KS;
   const int passes = (slices + CW - 1) / CW;
 
@@ -248,8 +258,12 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const int sl = p * CW + sloc;
         const int64_t n = n_begin + t * 16 + trow;
         const bool ok = sloc < CW && sl < slices && n < n_end;
-        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> GSHIFT) * 2u : kOutOfRange;
-        dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
+        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> (MX ? 0 : GSHIFT)) * 2u : kOutOfRange;
+        // (MXFP4 has no second table: the load still goes out, fetching nothing,
+        // so that every loader wavefront issues the same number per tile -- the
+        // waits count loads)
+        if constexpr (MX) dma16(rs, tb + kind * kTabKind + h * 1024, kind == 0 ? vo : kOutOfRange, 0u);
+        else dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
       }
     };
     // item `i` (compile-time kind) of pass `p` into ring slot `slot`
@@ -445,9 +459,26 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // acc + this wavefront's K-slice of one tile: `base` is the lane's row in
     // the slice's 4 KB of codes, `tb` its table row
     auto tile_math = [&](const unsigned char* base, const unsigned char* tb, f32x4 acc_in) __attribute__((always_inline)) {
+      if constexpr (MX) {
+        // E2M1 codes: the converter widens two codes at a time and multiplies
+        // by the 32-block's power-of-two scale (exact in bf16), so the chunks
+        // chain straight through the MFMA accumulator.  Lane kg holds codes
+        // [16 kg, 16 kg + 16) of the chunk: block 2c + kg/2 of the slice.
+        const u32x4 sv = *reinterpret_cast<const u32x4*>(tb);
+        f32x4 at = acc_in;
+#pragma unroll
+        for (int c = 0; c < CPS; ++c) {
+          const uint32_t pc = (uint32_t)(2 * c + (kg >> 1));
+          const u32x2 q = *reinterpret_cast<const u32x2*>(base + ((pc ^ swz) << 4) + (kg & 1) * 8);
+          const float sc = e8m0_to_f32((sv[c >> 1] >> (16 * (c & 1) + 8 * (kg >> 1))) & 255u);
+          at = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_e2m1(q[0], sc), at, 0, 0, 0);
+          at = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_e2m1(q[1], sc), at, 0, 0, 0);
+        }
+        return at;
+      }
       u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
       u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
-      if constexpr (GSHIFT != 0) {   // group 128: one entry serves two chunks -> duplicate each bf16
+      if constexpr (GSHIFT == 1) {   // group 128: one entry serves two chunks -> duplicate each bf16
         svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
                     byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
         bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
@@ -507,10 +538,12 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            if constexpr (BITS == 4) xa[c][j] = pair_stride4(raw[c][j]);
+            if constexpr (BITS == 4 && !MX) xa[c][j] = pair_stride4(raw[c][j]);
             else xa[c][j] = __builtin_bit_cast(bf16x8, raw[c][j]);
           }
-        if (active) chunk_sums();
+        if constexpr (!MX) {
+          if (active) chunk_sums();
+        }
       };
       if constexpr (XD == 1) {
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
@@ -640,6 +673,9 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
 
 template <int BITS, int CW, int NL, int TMAX, int XD>
 void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st, int chunks = 1) {
+  if constexpr (BITS == 4 && XD != 0) {
+    if (a.gshift == 2) return launch_one<BITS, CW, NL, TMAX, 2, XD>(a, batch, rows_per_wg, st, chunks);
+  }
   if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
   else launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st, chunks);
 }
@@ -781,6 +817,26 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
     if (bits == 4) launch_k<4, 8, 4, 8, 2>(a, segs, (int)rows, st);
     else launch_k<8, 8, 4, 8, 2>(a, segs, (int)rows, st);
   }
+}
+
+// MXFP4 decode on the direct variants: K a multiple of 512 with at least eight
+// slices, scale rows dword-aligned (they are fetched as 16-byte runs).
+bool skinny2_mx_supported(int64_t N, int64_t K, const void* s) {
+  static const bool off = getenv("QMM_NO_SKINNY_MX") != nullptr;
+  if (off || K % 512 || K / 512 < 8) return false;
+  if (reinterpret_cast<uintptr_t>(s) & 3u) return false;
+  return N * (K / 2) < 0x7FFFFFFFll;                          // 32-bit lane offsets
+}
+
+void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st) {
+  GemvArgs a = a0;
+  a.gshift = 2;
+  const int64_t cus = device_cus();
+  const int64_t rounds = ceil_div(ceil_div((int64_t)a.N, cus), (int64_t)128);
+  int64_t rows = ceil_div((int64_t)a.N, cus * rounds);
+  if (rows < 16) rows = 16;
+  if (a.K / 512 <= 8) launch_k<4, 8, 4, 4, 1>(a, batch, (int)rows, st);
+  else launch_k<4, 8, 4, 8, 2>(a, batch, (int)rows, st);
 }
 
 }  // namespace qmm

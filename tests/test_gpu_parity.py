@@ -222,6 +222,43 @@ def test_gemv_mxfp4(m):
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (1, 8192, 8192),      # two passes, one row: activations of both passes packed into the operand rows
+    (4, 5000, 4096),      # one pass, ragged last tile
+    (16, 3000, 4096),     # sixteen rows
+    (7, 20000, 4096),     # five tiles a workgroup
+    (3, 4100, 12288),     # three passes packed by four rows
+    (12, 2048, 8192),     # two passes, activations fetched per pass
+    (2, 640, 16384),      # four passes packed by four, fewer workgroups than compute units
+])
+def test_decode_mxfp4_big_weights_on_the_loader_wavefront_kernel(m, n, k):
+    """MXFP4 decode with K a multiple of 512 and at least eight 256-byte slices:
+    the loader-wavefront kernel widens the E2M1 codes with the 32-block's
+    power-of-two scale applied in the conversion (exact in bf16)."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4"))
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
+def test_decode_mxfp4_big_weights_batched_with_extreme_scales():
+    rng = np.random.default_rng(404)
+    e, n, k, m = 2, 1500, 4096, 3
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(e,), lo=100, hi=150)
+    x = O.round_bf16(rng.standard_normal((e, m, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    y = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                   out_dtype=torch.float32))
+    for z in range(e):
+        want = O.qmm(x[z], words[z], sb[z], None, 32, 4, "mxfp4")
+        assert O.rel_l2(y[z], want) <= 2e-5
+
+
 def test_gemv_batched():
     rng = np.random.default_rng(5)
     bsz, n, k = 3, 48, 256
