@@ -801,3 +801,18 @@ def test_gather_qmm_few_pairs_invalid_indices_touch_nothing():
         else:
             want = O.qmm(x[lhs[i]][None], words[rhs[i]], s[rhs[i]], b[rhs[i]], 64, 4)[0]
             assert O.rel_l2(got[i], want) <= 2e-5
+
+
+@pytest.mark.parametrize("k,pairs,e", [(4096, 20, 6), (8192, 40, 3)])
+def test_gather_qmm_few_pairs_grouped_by_expert_mxfp4(k, pairs, e):
+    """MXFP4 experts, few pairs: grouped decode on the loader-wavefront kernel."""
+    rng = np.random.default_rng(k + pairs)
+    n, t = 1200, 10
+    _, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    want = O.gather_qmm(x[:, None, :], words, sb, None, lhs, rhs, 32, 4, "mxfp4")[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, None, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                             group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
