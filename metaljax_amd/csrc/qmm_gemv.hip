@@ -377,7 +377,9 @@ bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
 void skinny_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int tab, hipStream_t st);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
-void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st);
+void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st,
+                      int tab, bool force_direct);
+int skinny2_direct_rows(int64_t N);
 bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
 void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st);
 
@@ -417,8 +419,19 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
     // self-loading one everywhere, for comparison)
     static const int v1 = env_int("QMM_SKINNY_V1");
     int rows;
-    if (!v1 && skinny2_plan(M, N, K, bits, &rows)) skinny2_dispatch(a, batch, gs, bits, rows, st);
+    if (!v1 && skinny2_plan(M, N, K, bits, &rows)) skinny2_dispatch(a, batch, gs, bits, rows, st, tab, false);
     else skinny_dispatch(a, batch, gs, bits, tab, st);
+    return;
+  }
+  // float16 tables (what MLX writes for float16 models): the loader-wavefront
+  // kernel reads them, the self-loading one does not
+  static const int no_f16 = env_int("QMM_NO_SKINNY_F16");
+  if (!no_skinny && !no_f16 && tab == QMM_F16 && K * bits / 8 / 256 >= 8 &&
+      skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b)) {
+    int rows;
+    const bool planned = skinny2_plan(M, N, K, bits, &rows);
+    if (!planned) rows = skinny2_direct_rows(N);
+    skinny2_dispatch(a, batch, gs, bits, rows, st, tab, !planned);
     return;
   }
   Geometry g;

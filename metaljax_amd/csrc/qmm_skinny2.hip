@@ -178,9 +178,13 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   // GSHIFT: 0 = affine, group 64; 1 = affine, group 128; 2 = MXFP4 (E2M1 codes,
   // one E8M0 scale byte per 32 codes: a row's table share of a slice is 16 bytes
   // in every case)
+  // 3 and 4 = groups of 64 and 128 with float16 tables (an entry is split into
+  // two bf16 terms, exactly, where it has to be a matrix operand).
   constexpr bool MX = GSHIFT == 2;
+  constexpr bool F16T = GSHIFT >= 3;
+  constexpr int GLOG = (GSHIFT == 1 || GSHIFT == 4) ? 1 : 0;   // log2(group / 64)
   static_assert(!MX || (BITS == 4 && XD != 0), "MXFP4: four-bit codes, direct variants");
-  const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GSHIFT;   // table row = ng * 2 bytes (MXFP4: K/32 bytes)
+  const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GLOG;   // table row = ng * 2 bytes (MXFP4: K/32 bytes)
   const int slices = a.K / KS;
   const int passes = (slices + CW - 1) / CW;
 
@@ -258,7 +262,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const int sl = p * CW + sloc;
         const int64_t n = n_begin + t * 16 + trow;
         const bool ok = sloc < CW && sl < slices && n < n_end;
-        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> (MX ? 0 : GSHIFT)) * 2u : kOutOfRange;
+        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> (MX ? 0 : GLOG)) * 2u : kOutOfRange;
         // (MXFP4 has no second table: the load still goes out, fetching nothing,
         // so that every loader wavefront issues the same number per tile -- the
         // waits count loads)
@@ -478,23 +482,47 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       }
       u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
       u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
-      if constexpr (GSHIFT == 1) {   // group 128: one entry serves two chunks -> duplicate each bf16
+      if constexpr (GLOG == 1) {     // group 128: one entry serves two chunks -> duplicate each 16-bit entry
         svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
                     byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
         bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
                     byte_perm(bvt[1], bvt[1], 0x01000100u), byte_perm(bvt[1], bvt[1], 0x03020302u)};
       }
-      const bf16x8 bop = __builtin_bit_cast(bf16x8, bvt);
-      f32x4 accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, bop, acc_in, 0, 0, 0);
-      accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, bop, accb, 0, 0, 0);
-      accb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, bop, accb, 0, 0, 0);
+      // eight table entries as matrix operands over the chunk index: one bf16
+      // operand, or for float16 tables two (hi + lo, exact: 11 significant bits)
+      auto split_f16 = [&](const u32x4& t, bf16x8& hi, bf16x8& lo) __attribute__((always_inline)) {
+        uint32_t h[4], l[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float f0 = f16_bits_to_f32(t[i] & 0xFFFFu), f1 = f16_bits_to_f32(t[i] >> 16);
+          const float h0 = __uint_as_float(__float_as_uint(f0) & 0xFFFF0000u);
+          const float h1 = __uint_as_float(__float_as_uint(f1) & 0xFFFF0000u);
+          h[i] = hi16_pair(h0, h1);
+          l[i] = hi16_pair(f0 - h0, f1 - h1);     // at most three significant bits: exact in bf16
+        }
+        hi = as_bf16x8(h[0], h[1], h[2], h[3]);
+        lo = as_bf16x8(l[0], l[1], l[2], l[3]);
+      };
+      auto xs_times = [&](const u32x4& t, f32x4 in) __attribute__((always_inline)) {
+        if constexpr (F16T) {
+          bf16x8 hi, lo;
+          split_f16(t, hi, lo);
+          f32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, hi, in, 0, 0, 0);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, hi, r, 0, 0, 0);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, hi, r, 0, 0, 0);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, lo, r, 0, 0, 0);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, lo, r, 0, 0, 0);
+          return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, lo, r, 0, 0, 0);
+        } else {
+          const bf16x8 op = __builtin_bit_cast(bf16x8, t);
+          f32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, op, in, 0, 0, 0);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, op, r, 0, 0, 0);
+          return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, op, r, 0, 0, 0);
+        }
+      };
+      const f32x4 accb = xs_times(bvt, acc_in);
       f32x4 accs = zero;
-      if constexpr (BITS == 4) {
-        const bf16x8 sop = __builtin_bit_cast(bf16x8, svt);
-        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, sop, zero, 0, 0, 0);
-        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, sop, accs, 0, 0, 0);
-        accs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, sop, accs, 0, 0, 0);
-      }
+      if constexpr (BITS == 4) accs = xs_times(svt, zero);
       f32x4 at = accb;
 #pragma unroll
       for (int c = 0; c < CPS; ++c) {
@@ -511,7 +539,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_int8(q[2], q[3]), d, 0, 0, 0);
         }
         const uint32_t sw = svt[c >> 1];
-        const float sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
+        float sc;
+        if constexpr (F16T) sc = f16_bits_to_f32((c & 1) ? sw >> 16 : sw & 0xFFFFu);
+        else sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
 #pragma unroll
         for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
       }
@@ -676,8 +706,12 @@ void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st,
   if constexpr (BITS == 4 && XD != 0) {
     if (a.gshift == 2) return launch_one<BITS, CW, NL, TMAX, 2, XD>(a, batch, rows_per_wg, st, chunks);
   }
-  if (a.gshift) launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
-  else launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st, chunks);
+  switch (a.gshift) {
+    case 1: return launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
+    case 3: return launch_one<BITS, CW, NL, TMAX, 3, XD>(a, batch, rows_per_wg, st, chunks);
+    case 4: return launch_one<BITS, CW, NL, TMAX, 4, XD>(a, batch, rows_per_wg, st, chunks);
+    default: return launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st, chunks);
+  }
 }
 
 int device_cus() {
@@ -749,10 +783,22 @@ bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg) {
   return rows > 32 && rows <= 64;
 }
 
-void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st) {
+// Rows a workgroup for the direct variants whatever the shape (float16 tables:
+// the self-loading kernel does not read them).
+int skinny2_direct_rows(int64_t N) {
+  const int64_t cus = device_cus();
+  const int64_t rounds = ceil_div(ceil_div(N, cus), (int64_t)128);
+  const int64_t r = ceil_div(N, cus * rounds);
+  return (int)(r < 16 ? 16 : r);
+}
+
+// tab: QMM_BF16 or QMM_F16 tables; force_direct: a direct variant even where
+// the ring variant or the self-loading kernel would be chosen
+void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st,
+                      int tab, bool force_direct) {
   GemvArgs a = a0;
-  a.gshift = gs == 128 ? 1 : 0;
-  const bool xd = direct_x(a.M, a.N, a.K, bits);
+  a.gshift = (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : 0);
+  const bool xd = force_direct || direct_x(a.M, a.N, a.K, bits);
   if (xd) {                                       // up to eight tiles' sums in registers over several passes
     const bool one_pass = a.K * bits / 8 / 256 <= 8;
     if (one_pass) {

@@ -314,6 +314,28 @@ def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     np.testing.assert_array_equal(y16, O.round_bf16(y32))
 
 
+@pytest.mark.parametrize("bits,gs,m,n,k", [
+    (4, 64, 4, 9000, 4096),      # one pass, activations fetched directly
+    (4, 128, 1, 4096, 4096),     # group 128, one tile a workgroup
+    (8, 64, 16, 5000, 2048),     # eight-bit codes, sixteen rows
+    (4, 64, 16, 14336, 4096),    # sixteen rows, 56 rows a workgroup: activations through the ring
+    (4, 64, 3, 3000, 8192),      # two passes, rows packed
+    (4, 128, 12, 2048, 12288),   # three passes, one tile a workgroup, activations fetched per pass
+])
+def test_decode_big_weights_float16_tables(bits, gs, m, n, k):
+    """float16 scales and biases (what float16 models carry): the loader-wavefront
+    kernel splits an entry into two bf16 terms where it is a matrix operand, so
+    the result is as exact as with bf16 tables."""
+    rng = np.random.default_rng(bits * 100 + gs + m + n + k)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab="f16")
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits))
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
 def test_decode_big_weights_batched_and_gathered():
     rng = np.random.default_rng(99)
     e, n, k = 3, 9000, 4096
