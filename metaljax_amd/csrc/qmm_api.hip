@@ -19,7 +19,7 @@ bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode,
 void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
                               int y_dtype, const int32_t* segments, const int32_t* src_row,
                               const int32_t* out_row, int64_t P, int64_t T, int64_t E, int64_t N,
-                              int64_t K, int gs, int bits, int mode, hipStream_t st);
+                              int64_t K, int gs, int bits, int mode, int tab, hipStream_t st);
 int64_t skinny2_max_segments(int64_t P, int64_t E);
 void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, const int32_t* row_offsets, const int32_t* lhs_idx,
@@ -399,7 +399,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
     rc = check_launch("route launch");
     if (rc) return rc;
     skinny2_grouped_dispatch(x, w, scales, biases, y, y_dtype, segments, src_row, out_row, P, T, E, N, K,
-                             group_size, bits, mode, st);
+                             group_size, bits, mode, table_dtype, st);
     return check_launch("grouped decode launch");
   }
   if (P <= kGatherGemvMaxPairs) {

@@ -829,7 +829,7 @@ bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E) {
   if (mode == QMM_MODE_MXFP4) return skinny2_mx_supported(N, K, s);
-  if (!skinny_supported(N, K, gs, bits, mode, tab, s, b)) return false;
+  if (!skinny_supported(N, K, gs, bits, mode, tab == QMM_F16 ? QMM_BF16 : tab, s, b)) return false;
   return K * bits / 8 / 256 >= 8;
 }
 
@@ -838,7 +838,7 @@ int64_t skinny2_max_segments(int64_t P, int64_t E) { return (E < P ? E : P) + P 
 void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
                               int y_dtype, const int32_t* segments, const int32_t* src_row,
                               const int32_t* out_row, int64_t P, int64_t T, int64_t E, int64_t N,
-                              int64_t K, int gs, int bits, int mode, hipStream_t st) {
+                              int64_t K, int gs, int bits, int mode, int tab, hipStream_t st) {
   GemvArgs a;
   a.x = static_cast<const uint16_t*>(x);
   a.w = static_cast<const uint32_t*>(w);
@@ -846,7 +846,7 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   a.b = b;
   a.y = y;
   a.M = 1; a.N = (int)N; a.K = (int)K;
-  a.gshift = mode == QMM_MODE_MXFP4 ? 2 : gs == 128 ? 1 : 0;
+  a.gshift = mode == QMM_MODE_MXFP4 ? 2 : (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : 0);
   a.y_dtype = y_dtype;
   a.lhs_idx = nullptr;
   a.rhs_idx = nullptr;

@@ -793,6 +793,19 @@ def test_gather_qmm_few_pairs_grouped_by_expert(bits, gs, t, pairs, e, n, k, ske
     np.testing.assert_array_equal(y16, O.round_bf16(y))
 
 
+def test_gather_qmm_few_pairs_grouped_by_expert_float16_tables():
+    rng = np.random.default_rng(1616)
+    e, n, k, t, pairs = 4, 2500, 4096, 9, 24
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, tab="f16", lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, 64, 4)[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                             group_size=64, bits=4, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
 def test_gather_qmm_few_pairs_invalid_indices_touch_nothing():
     """Grouped decode: a pair naming no expert keeps its output row as it was,
     a pair naming a row outside x multiplies zeros."""
