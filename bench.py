@@ -89,6 +89,36 @@ def bench_decode(cfg, M, steps, warmup):
     return wl, ms, n_sets, ys[0]
 
 
+def bench_decode_random(m, n, k, bits=4, mode="affine", tables="bf16", steps=200, warmup=20):
+    """Per-launch time of a decode shape outside the named configurations, on
+    random codes (timing only): graph replay over rotating weight sets."""
+    import torch
+    from metaljax_amd import kernels as K
+    g = torch.Generator(device="cuda").manual_seed(n + k)
+    words = k * bits // 32
+    x = torch.randn((m, k), device="cuda", generator=g).bfloat16()
+    if mode == "mxfp4":
+        s = torch.randint(118, 132, (n, k // 32), dtype=torch.uint8, device="cuda", generator=g)
+        b = None
+        gs = 32
+    else:
+        dt = torch.float16 if tables == "f16" else torch.bfloat16
+        s = (torch.rand((n, k // 64), device="cuda", generator=g) * 0.01 + 0.005).to(dt)
+        b = (-8 * s.float()).to(dt)
+        gs = 64
+    per_set = n * words * 4
+    n_sets = max(2, (2 * LLC_BYTES) // per_set + 1)
+    ws = [torch.randint(-2**31, 2**31 - 1, (n, words), dtype=torch.int32, device="cuda", generator=g)
+          for _ in range(n_sets)]
+    ys = [torch.empty((m, n), dtype=torch.bfloat16, device="cuda") for _ in range(n_sets)]
+    ms = run_rotating(lambda i: K.BoundQmm(x, ws[i], s, b, ys[i], group_size=gs, bits=bits, mode=mode),
+                      n_sets, steps, warmup)
+    us = ms * 1e3 / steps
+    nbytes = n * words * 4 + s.numel() * s.element_size() * (1 if b is None else 2) + (m * k + m * n) * 2
+    return {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+            "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
 def bench_once(cfg, steps=20, warmup=3):
     """A short timing of one of the other named shapes (weights are reused, so
     they may sit in the last-level cache; these shapes are compute-bound)."""
@@ -223,6 +253,14 @@ def main():
                                       "GB/s": round(wlc1.algorithmic_bytes / usc1 / 1e3, 1),
                                       "frac_of_hbm_peak": round(wlc1.algorithmic_bytes / usc1 / 1e3 / HBM_PEAK_GBS, 4)}}
         out["other_shapes"].update({f"C{c}": bench_once(c) for c in (3, 4, 5)})
+        # decode shapes outside the named configurations (random codes, timing only)
+        out["other_decode_shapes"] = {
+            "int4 g64 [28672,4096] M=4": bench_decode_random(4, 28672, 4096),
+            "int4 g64 [4096,14336] M=4": bench_decode_random(4, 4096, 14336),
+            "int4 g64 f16 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f16"),
+            "int8 g64 [14336,4096] M=4": bench_decode_random(4, 14336, 4096, bits=8),
+            "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
+        }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
