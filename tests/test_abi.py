@@ -66,6 +66,32 @@ def test_plan_picks_the_regime(lib):
     assert k.value == _lib.KERNEL_GEMM and g.value >= 256
 
 
+def test_plan_of_the_decode_variants(lib):
+    """The decode plan follows the kernel choice: 768-thread workgroups (eight
+    compute + four loader wavefronts) where the loader-wavefront kernel serves
+    the shape, one workgroup per compute unit (256 assumed without a device)
+    with up to 128 rows each when the activations are fetched directly."""
+    k, g, b = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.qmm_plan(4, 28672, 4096, 64, 4, 0, k, g, b) == 0
+    assert (k.value, b.value) == (_lib.KERNEL_GEMV, 768)
+    rows = -(-28672 // g.value)
+    assert 16 <= rows <= 128 and g.value * rows >= 28672
+    assert lib.qmm_plan(16, 14336, 4096, 64, 4, 0, k, g, b) == 0        # ring variant: at most 64 rows
+    assert b.value == 768 and -(-14336 // g.value) <= 64
+    assert lib.qmm_plan(4, 4096, 1024, 64, 4, 0, k, g, b) == 0          # two slices: the self-loading kernel
+    assert k.value == _lib.KERNEL_GEMV and b.value < 768
+
+
+def test_gather_workspace_covers_the_grouped_decode(lib):
+    """From four pairs up to sixteen an expert the workspace holds the expert
+    sort and the segment list; below four pairs nothing is needed."""
+    assert lib.qmm_gather_workspace_bytes(2, 8, 14336, 4096) == 0
+    few = lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096)
+    sort_only = ((2 * 8 + 1 + 2 * 16) * 4 + 255) // 256 * 256
+    assert few >= sort_only and few % 256 == 0
+    assert lib.qmm_gather_workspace_bytes(128, 8, 14336, 4096) >= lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096)
+
+
 def test_workspace_queries_need_no_device(lib):
     assert lib.qmm_workspace_bytes(1, 16, 14336, 4096, 64, 4, 0, _lib.BF16) == 0
     need = lib.qmm_gather_workspace_bytes(1024, 8, 14336, 4096)
