@@ -137,3 +137,87 @@ def test_one_pass_decode_random_case(seed):
     assert err <= 2e-5, (m, n, k, gs, bits, batch, err)
     y16 = K.quantized_matmul(_bf16_dev(x), wd, _bf16_dev(s), _bf16_dev(b), group_size=gs, bits=bits)
     np.testing.assert_array_equal(y16.float().cpu().numpy(), O.round_bf16(y32))
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_big_decode_random_case(seed):
+    """Decode shapes with at least eight 256-byte K-slices, drawn at random over
+    everything the loader-wavefront kernel distinguishes: passes over K (one to
+    four, the last possibly part full), rows of activations (row packing or a
+    fetch per pass), tiles a workgroup, code width, group size, bf16 / float16
+    tables, MXFP4, a batch axis."""
+    rng = np.random.default_rng(12000 + seed)
+    kind = str(rng.choice(["int4", "int4", "int8", "mxfp4"]))
+    bits = 8 if kind == "int8" else 4
+    slice_k = 2048 // bits                                   # codes in a 256-byte slice
+    slices = int(rng.integers(8, 33))
+    k = slices * slice_k
+    if kind == "mxfp4":
+        k = max(4096, k // 512 * 512)
+    m = int(rng.integers(1, 17))
+    n = int(rng.choice([rng.integers(16, 400), rng.integers(400, 6000), rng.integers(6000, 30000)]))
+    if n * k > 120_000_000:                                  # keep the oracle's float64 product quick
+        n = 120_000_000 // k
+    batch = 2 if (n * k < 8_000_000 and rng.random() < 0.3) else 1
+    lead = (batch,) if batch > 1 else ()
+    x = O.round_bf16(rng.standard_normal(lead + (m, k)).astype(np.float32))
+    codes = rng.integers(0, 1 << bits, size=lead + (n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    if kind == "mxfp4":
+        sb = rng.integers(110, 140, size=lead + (n, k // 32)).astype(np.uint8)
+        y = K.quantized_matmul(_bf16_dev(x), wd, torch.from_numpy(sb).to(DEV), None, group_size=32, bits=4,
+                               mode="mxfp4", out_dtype=torch.float32).float().cpu().numpy()
+        want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+        info = (kind, m, n, k, batch)
+    else:
+        gs = int(rng.choice([64, 128]))
+        tab = str(rng.choice(["bf16", "bf16", "f16"]))
+        s = rng.uniform(0.005, 0.02, lead + (n, k // gs)).astype(np.float32)
+        b = -(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s
+        if tab == "bf16":
+            s, b = O.round_bf16(s), O.round_bf16(b)
+        else:
+            s, b = s.astype(np.float16).astype(np.float32), b.astype(np.float16).astype(np.float32)
+        y = K.quantized_matmul(_bf16_dev(x), wd, _tab_dev(s, tab), _tab_dev(b, tab), group_size=gs, bits=bits,
+                               out_dtype=torch.float32).float().cpu().numpy()
+        want = O.qmm(x, words, s, b, gs, bits)
+        info = (kind, gs, tab, m, n, k, batch)
+    err = O.rel_l2(y, want)
+    assert err <= 2e-5, (info, err)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_decode_random_case(seed):
+    """Expert-indexed products with few pairs (4 <= P <= 16 E): random routing,
+    skewed or not, with indices that name no expert or no row now and then."""
+    rng = np.random.default_rng(13000 + seed)
+    kind = str(rng.choice(["int4", "int8", "mxfp4"]))
+    bits = 8 if kind == "int8" else 4
+    k = int(rng.choice([1, 2, 3])) * (4096 if bits == 4 else 2048)
+    e = int(rng.integers(1, 9))
+    n = int(rng.integers(16, 3000))
+    t = int(rng.integers(1, 40))
+    pairs = int(rng.integers(4, 16 * e + 1))
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    if rng.random() < 0.5:
+        rhs[rng.random(pairs) < 0.7] = int(rng.integers(0, e))
+    x = O.round_bf16(rng.standard_normal((t, k)).astype(np.float32))
+    codes = rng.integers(0, 1 << bits, size=(e, n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    ld, rd = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    if kind == "mxfp4":
+        sb = rng.integers(110, 140, size=(e, n, k // 32)).astype(np.uint8)
+        y = K.gather_qmm(_bf16_dev(x), wd, torch.from_numpy(sb).to(DEV), None, ld, rd, group_size=32, bits=4,
+                         mode="mxfp4", out_dtype=torch.float32).float().cpu().numpy()
+        want = O.gather_qmm(x[:, None, :], words, sb, None, lhs, rhs, 32, 4, "mxfp4")[:, 0]
+    else:
+        s = O.round_bf16(rng.uniform(0.005, 0.02, (e, n, k // 64)).astype(np.float32))
+        b = O.round_bf16(-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s)
+        y = K.gather_qmm(_bf16_dev(x), wd, _bf16_dev(s), _bf16_dev(b), ld, rd, group_size=64, bits=bits,
+                         out_dtype=torch.float32).float().cpu().numpy()
+        want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, 64, bits)[:, 0]
+    err = O.rel_l2(y, want)
+    assert err <= 2e-5, (kind, k, e, n, t, pairs, err)
