@@ -102,7 +102,7 @@ def bench_decode_random(m, n, k, bits=4, mode="affine", tables="bf16", steps=200
         b = None
         gs = 32
     else:
-        dt = torch.float16 if tables == "f16" else torch.bfloat16
+        dt = {"f16": torch.float16, "f32": torch.float32}.get(tables, torch.bfloat16)
         s = (torch.rand((n, k // 64), device="cuda", generator=g) * 0.01 + 0.005).to(dt)
         b = (-8 * s.float()).to(dt)
         gs = 64
@@ -258,6 +258,7 @@ def main():
             "int4 g64 [28672,4096] M=4": bench_decode_random(4, 28672, 4096),
             "int4 g64 [4096,14336] M=4": bench_decode_random(4, 4096, 14336),
             "int4 g64 f16 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f16"),
+            "int4 g64 f32 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f32"),
             "int8 g64 [14336,4096] M=4": bench_decode_random(4, 14336, 4096, bits=8),
             "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
         }

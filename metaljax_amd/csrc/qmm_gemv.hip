@@ -423,10 +423,11 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
     else skinny_dispatch(a, batch, gs, bits, tab, st);
     return;
   }
-  // float16 tables (what MLX writes for float16 models): the loader-wavefront
-  // kernel reads them, the self-loading one does not
+  // float16 tables (what float16 models carry) and float32 tables (biases that
+  // do not fit 16 bits): the loader-wavefront kernel reads them, the
+  // self-loading one does not
   static const int no_f16 = env_int("QMM_NO_SKINNY_F16");
-  if (!no_skinny && !no_f16 && tab == QMM_F16 && K * bits / 8 / 256 >= 8 &&
+  if (!no_skinny && !no_f16 && (tab == QMM_F16 || tab == QMM_F32) && K * bits / 8 / 256 >= 8 &&
       skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b)) {
     int rows;
     const bool planned = skinny2_plan(M, N, K, bits, &rows);

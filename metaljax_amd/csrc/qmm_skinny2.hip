@@ -156,9 +156,14 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   constexpr int XR = XD ? 0 : KS / 128;           // activation rounds per slice through the ring: 4 | 2, or none
   constexpr int NI = XR + TMAX;                   // items per pass
   constexpr int kItem = CW * 4096;
-  constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;   // scale rows | bias rows of one tile
+  // Table kind (GSHIFT): 0 / 1 = bf16 tables, groups of 64 / 128; 2 = MXFP4
+  // (E2M1 codes, one E8M0 byte per 32 codes); 3 / 4 = float16 tables; 5 / 6 =
+  // float32 tables.  A row's table share of a slice is 16 bytes, except for
+  // float32 tables with groups of 64 (eight 4-byte entries: 32 bytes, WIDE).
+  constexpr bool WIDE = GSHIFT == 5;
+  constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (WIDE ? 2 : 1);   // scale rows | bias rows of one tile
   constexpr int kTab = 2 * kTabKind;
-  constexpr int NTAB = 2 * (CW >= 4 ? CW / 4 : 1);      // table load instructions per tile
+  constexpr int NTAB = 2 * (CW >= 4 ? CW / 4 : 1) * (WIDE ? 2 : 1);        // table load instructions per tile
   static_assert((CW * 4) % NL == 0 && NTAB % NL == 0, "loader shares must be whole");
   constexpr int QI = CW * 4 / NL;                 // code / activation loads per loader wavefront per item
   constexpr int QT = NTAB / NL;                   // table loads per loader wavefront per tile
@@ -175,16 +180,15 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   const int64_t n_end = n_begin + rows_per_wg < a.N ? n_begin + rows_per_wg : a.N;
   const int ntiles = (int)((n_end - n_begin + 15) / 16);        // uniform, <= TMAX
   const int64_t wpr = (int64_t)a.K * BITS / 8;                  // bytes per weight row
-  // GSHIFT: 0 = affine, group 64; 1 = affine, group 128; 2 = MXFP4 (E2M1 codes,
-  // one E8M0 scale byte per 32 codes: a row's table share of a slice is 16 bytes
-  // in every case)
-  // 3 and 4 = groups of 64 and 128 with float16 tables (an entry is split into
-  // two bf16 terms, exactly, where it has to be a matrix operand).
+  // float16 / float32 entries are split into two / three bf16 terms, exactly,
+  // where they have to be matrix operands.
   constexpr bool MX = GSHIFT == 2;
-  constexpr bool F16T = GSHIFT >= 3;
-  constexpr int GLOG = (GSHIFT == 1 || GSHIFT == 4) ? 1 : 0;   // log2(group / 64)
+  constexpr bool F16T = GSHIFT == 3 || GSHIFT == 4;
+  constexpr bool F32T = GSHIFT >= 5;
+  constexpr int ES = F32T ? 4 : 2;                             // bytes per table entry
+  constexpr int GLOG = (GSHIFT == 1 || GSHIFT == 4 || GSHIFT == 6) ? 1 : 0;   // log2(group / 64)
   static_assert(!MX || (BITS == 4 && XD != 0), "MXFP4: four-bit codes, direct variants");
-  const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GLOG;   // table row = ng * 2 bytes (MXFP4: K/32 bytes)
+  const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GLOG;   // table row = ng * ES bytes (MXFP4: K/32 bytes)
   const int slices = a.K / KS;
   const int passes = (slices + CW - 1) / CW;
 
@@ -221,8 +225,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const int lw = wave - CW;
     const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
     const auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
-    const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * 2, a.N * ng * 2);
-    const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * 2, a.N * ng * 2);
+    const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * ES, a.N * ng * ES);
+    const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * ES, a.N * ng * ES);
     const int lrow = lane >> 4, lp = lane & 15;
     // Load q of this wavefront is instruction j = lw + q*NL of the item: slice
     // j / 4, row quad j % 4 = (lw + o) % 4 with o = q*NL % 4 known at compile
@@ -257,17 +261,20 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
       for (int q = 0; q < QT; ++q) {
         const int jt = lw + q * NL;               // uniform
-        const int kind = jt / (NTAB / 2), h = jt % (NTAB / 2);
+        const int kind = jt / (NTAB / 2), rem = jt % (NTAB / 2);
+        const int h = WIDE ? rem >> 1 : rem, h2 = WIDE ? rem & 1 : 0;   // four-slice group; 16-byte half of a wide row
         const int sloc = 4 * h + tsl;
         const int sl = p * CW + sloc;
         const int64_t n = n_begin + t * 16 + trow;
         const bool ok = sloc < CW && sl < slices && n < n_end;
-        const uint32_t vo = ok ? (uint32_t)(n * ng * 2) + (uint32_t)((sl * CPS) >> (MX ? 0 : GLOG)) * 2u : kOutOfRange;
+        const uint32_t vo = ok ? (uint32_t)(n * ng * ES) + (uint32_t)((sl * CPS) >> (MX ? 0 : GLOG)) * (uint32_t)ES + (uint32_t)h2 * 16u
+                               : kOutOfRange;
+        unsigned char* tdst = tb + kind * kTabKind + (WIDE ? h * 2048 + h2 * 1024 : h * 1024);
         // (MXFP4 has no second table: the load still goes out, fetching nothing,
         // so that every loader wavefront issues the same number per tile -- the
         // waits count loads)
-        if constexpr (MX) dma16(rs, tb + kind * kTabKind + h * 1024, kind == 0 ? vo : kOutOfRange, 0u);
-        else dma16(kind ? rb : rs, tb + kind * kTabKind + h * 1024, vo, 0u);
+        if constexpr (MX) dma16(rs, tdst, kind == 0 ? vo : kOutOfRange, 0u);
+        else dma16(kind ? rb : rs, tdst, vo, 0u);
       }
     };
     // item `i` (compile-time kind) of pass `p` into ring slot `slot`
@@ -423,6 +430,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
     const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
     // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
+    const int tab_row = (wave >> 2) * (WIDE ? 2048 : 1024) + (wave & 3) * 256 + r * 16;   // this lane's table row inside a kind
     const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
     const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, xrows * a.K * 2);
     auto xrow = [&](int m) -> int64_t {
@@ -482,7 +490,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       }
       u32x4 svt = *reinterpret_cast<const u32x4*>(tb);
       u32x4 bvt = *reinterpret_cast<const u32x4*>(tb + kTabKind);
-      if constexpr (GLOG == 1) {     // group 128: one entry serves two chunks -> duplicate each 16-bit entry
+      if constexpr (GLOG == 1 && !F32T) {   // group 128: one entry serves two chunks -> duplicate each 16-bit entry
         svt = u32x4{byte_perm(svt[0], svt[0], 0x01000100u), byte_perm(svt[0], svt[0], 0x03020302u),
                     byte_perm(svt[1], svt[1], 0x01000100u), byte_perm(svt[1], svt[1], 0x03020302u)};
         bvt = u32x4{byte_perm(bvt[0], bvt[0], 0x01000100u), byte_perm(bvt[0], bvt[0], 0x03020302u),
@@ -520,9 +528,52 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, op, r, 0, 0, 0);
         }
       };
-      const f32x4 accb = xs_times(bvt, acc_in);
-      f32x4 accs = zero;
-      if constexpr (BITS == 4) accs = xs_times(svt, zero);
+      // float32 tables: the entries of the eight chunks as floats (group 128: one
+      // entry serves two chunks), and as matrix operands three bf16 terms each
+      float sf[8], bfv[8];
+      if constexpr (F32T) {
+        if constexpr (WIDE) {
+          const u32x4 s1 = *reinterpret_cast<const u32x4*>(tb + 1024);
+          const u32x4 b1 = *reinterpret_cast<const u32x4*>(tb + kTabKind + 1024);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            sf[i] = __uint_as_float(svt[i]); sf[4 + i] = __uint_as_float(s1[i]);
+            bfv[i] = __uint_as_float(bvt[i]); bfv[4 + i] = __uint_as_float(b1[i]);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            sf[2 * i] = sf[2 * i + 1] = __uint_as_float(svt[i]);
+            bfv[2 * i] = bfv[2 * i + 1] = __uint_as_float(bvt[i]);
+          }
+        }
+      }
+      auto xs_times_f32 = [&](const float (&v)[8], f32x4 in) __attribute__((always_inline)) {
+        float h[8], m[8], l[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) split3(v[i], h[i], m[i], l[i]);
+        const bf16x8 oh = as_bf16x8(hi16_pair(h[0], h[1]), hi16_pair(h[2], h[3]), hi16_pair(h[4], h[5]), hi16_pair(h[6], h[7]));
+        const bf16x8 om = as_bf16x8(hi16_pair(m[0], m[1]), hi16_pair(m[2], m[3]), hi16_pair(m[4], m[5]), hi16_pair(m[6], m[7]));
+        const bf16x8 ol = as_bf16x8(hi16_pair(l[0], l[1]), hi16_pair(l[2], l[3]), hi16_pair(l[4], l[5]), hi16_pair(l[6], l[7]));
+        f32x4 r = in;
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, oh, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, oh, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, oh, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, om, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, om, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, om, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, ol, r, 0, 0, 0);
+        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, ol, r, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, ol, r, 0, 0, 0);
+      };
+      f32x4 accb, accs = zero;
+      if constexpr (F32T) {
+        accb = xs_times_f32(bfv, acc_in);
+        if constexpr (BITS == 4) accs = xs_times_f32(sf, zero);
+      } else {
+        accb = xs_times(bvt, acc_in);
+        if constexpr (BITS == 4) accs = xs_times(svt, zero);
+      }
       f32x4 at = accb;
 #pragma unroll
       for (int c = 0; c < CPS; ++c) {
@@ -540,7 +591,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         }
         const uint32_t sw = svt[c >> 1];
         float sc;
-        if constexpr (F16T) sc = f16_bits_to_f32((c & 1) ? sw >> 16 : sw & 0xFFFFu);
+        if constexpr (F32T) sc = sf[c];
+        else if constexpr (F16T) sc = f16_bits_to_f32((c & 1) ? sw >> 16 : sw & 0xFFFFu);
         else sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
 #pragma unroll
         for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
@@ -585,7 +637,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           item_barrier();
           const int slot = g & 3;
           f32x4 at = zero;
-          if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
+          if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + tab_row, zero);
           float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
 #pragma unroll
           for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
@@ -614,7 +666,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
               item_barrier();
               const int slot = (p * ntiles + t) & 3;
               if (active) {
-                const f32x4 d = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + wave * 256 + r * 16, zero);
+                const f32x4 d = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + tab_row, zero);
                 const bool mine = PK == 0 || my_pass == p;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[t][e] += mine ? d[e] : 0.f;
@@ -658,7 +710,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         } else {
           constexpr int t = i - XR;
           if (active && t < ntiles)
-            acc[t] = tile_math(base, tabs + slot * kTab + wave * 256 + r * 16, acc[t]);
+            acc[t] = tile_math(base, tabs + slot * kTab + tab_row, acc[t]);
           // Last pass: this wavefront's partial sums of tile t go where its own
           // slice of the tile was (nobody else reads that region, and a tile's
           // slot is not refilled within a pass); the loaders add the slices up.
@@ -688,7 +740,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 template <int BITS, int CW, int NL, int TMAX, int GSHIFT, int XD>
 void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st, int chunks = 1) {
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
-  constexpr int kTabKind = CW >= 4 ? CW * 256 : 1024;
+  constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (GSHIFT == 5 ? 2 : 1);
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
   const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
   auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
@@ -710,6 +762,8 @@ void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st,
     case 1: return launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
     case 3: return launch_one<BITS, CW, NL, TMAX, 3, XD>(a, batch, rows_per_wg, st, chunks);
     case 4: return launch_one<BITS, CW, NL, TMAX, 4, XD>(a, batch, rows_per_wg, st, chunks);
+    case 5: return launch_one<BITS, CW, NL, TMAX, 5, XD>(a, batch, rows_per_wg, st, chunks);
+    case 6: return launch_one<BITS, CW, NL, TMAX, 6, XD>(a, batch, rows_per_wg, st, chunks);
     default: return launch_one<BITS, CW, NL, TMAX, 0, XD>(a, batch, rows_per_wg, st, chunks);
   }
 }
@@ -797,7 +851,7 @@ int skinny2_direct_rows(int64_t N) {
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st,
                       int tab, bool force_direct) {
   GemvArgs a = a0;
-  a.gshift = (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : 0);
+  a.gshift = (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : tab == QMM_F32 ? 5 : 0);
   const bool xd = force_direct || direct_x(a.M, a.N, a.K, bits);
   if (xd) {                                       // up to eight tiles' sums in registers over several passes
     const bool one_pass = a.K * bits / 8 / 256 <= 8;
@@ -829,7 +883,7 @@ bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E) {
   if (mode == QMM_MODE_MXFP4) return skinny2_mx_supported(N, K, s);
-  if (!skinny_supported(N, K, gs, bits, mode, tab == QMM_F16 ? QMM_BF16 : tab, s, b)) return false;
+  if (!skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b)) return false;   // bf16, float16 and float32 tables alike
   return K * bits / 8 / 256 >= 8;
 }
 
@@ -846,7 +900,7 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   a.b = b;
   a.y = y;
   a.M = 1; a.N = (int)N; a.K = (int)K;
-  a.gshift = mode == QMM_MODE_MXFP4 ? 2 : (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : 0);
+  a.gshift = mode == QMM_MODE_MXFP4 ? 2 : (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : tab == QMM_F32 ? 5 : 0);
   a.y_dtype = y_dtype;
   a.lhs_idx = nullptr;
   a.rhs_idx = nullptr;

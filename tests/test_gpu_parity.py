@@ -336,6 +336,30 @@ def test_decode_big_weights_float16_tables(bits, gs, m, n, k):
     np.testing.assert_array_equal(y16, O.round_bf16(y32))
 
 
+@pytest.mark.parametrize("bits,gs,m,n,k", [
+    (4, 64, 4, 9000, 4096),      # groups of 64: eight 4-byte entries a row and slice (two table loads)
+    (4, 128, 1, 4096, 4096),     # group 128, one tile a workgroup
+    (8, 64, 16, 5000, 2048),     # eight-bit codes, sixteen rows
+    (8, 128, 3, 6144, 4096),     # eight-bit codes, group 128, two passes
+    (4, 64, 16, 14336, 4096),    # sixteen rows, 56 rows a workgroup: activations through the ring
+    (4, 64, 3, 3000, 8192),      # two passes, rows packed
+    (4, 128, 12, 2048, 12288),   # three passes, one tile a workgroup, activations fetched per pass
+    (4, 64, 2, 28001, 4096),     # seven tiles a workgroup, the last ragged
+])
+def test_decode_big_weights_float32_tables(bits, gs, m, n, k):
+    """float32 scales and biases (biases that do not fit 16 bits): an entry is
+    split into three bf16 terms where it is a matrix operand, so the bias term
+    keeps its 24 bits."""
+    rng = np.random.default_rng(bits * 100 + gs + m + n + k + 32)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab="f32")
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, s, b, gs, bits)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits))
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
 def test_decode_big_weights_batched_and_gathered():
     rng = np.random.default_rng(99)
     e, n, k = 3, 9000, 4096
@@ -803,6 +827,20 @@ def test_gather_qmm_few_pairs_grouped_by_expert_float16_tables():
     want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, 64, 4)[:, 0]
     y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
                              group_size=64, bits=4, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+@pytest.mark.parametrize("gs", [64, 128])
+def test_gather_qmm_few_pairs_grouped_by_expert_float32_tables(gs):
+    rng = np.random.default_rng(3232 + gs)
+    e, n, k, t, pairs = 4, 2500, 4096, 9, 24
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, gs, tab="f32", lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    want = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, gs, 4)[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                             group_size=gs, bits=4, out_dtype=torch.float32))
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
 
 
