@@ -199,7 +199,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU; --gpus {args.gpus} is not supported "
-              "(the path shards by weight rows, see DESIGN.md)", file=sys.stderr)
+              "(rows of the weight are independent: more GPUs would each take a share of N)", file=sys.stderr)
         return 2
     import torch
     if not torch.cuda.is_available():
