@@ -38,7 +38,7 @@ namespace {
 constexpr int BN = 128, BK = 64;
 constexpr int kRowBytes = BK * 2;                 // bf16 tile row
 constexpr int kStage = BN * kRowBytes;            // 16 KB
-constexpr int kStages = 3;
+constexpr int kStages = 4;                        // stage of K-tile t = t & 3: a compile-time LDS offset
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
   const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)bytes;
@@ -118,7 +118,11 @@ __device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float 
     }
   } else {
     const uint32_t w = q[pc];
-    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;     // even / odd codes as bytes
+    uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;           // even / odd codes as bytes
+    // kept opaque, so that each code is one byte-to-float conversion of lo / hi
+    // (merged with the masks above they become a bit-field extract plus a conversion)
+    asm("" : "+v"(lo));
+    asm("" : "+v"(hi));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f[2 * j] = fmaf(sc, (float)((lo >> (8 * j)) & 255u), bi);
@@ -229,13 +233,21 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // reads ax[(kt*8 + ks*2 + kh) * Rp + m0 + (wm*RB0 + i*RBI)*32 + li]
   const auto ra = make_rsrc(a.ax, (int64_t)(a.K / 8) * a.Rp * 16);
   const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * (RB0 * 32) + li) * 16);
+  // Ragged tiles by the rows they hold (uniform over the workgroup): at most
+  // WMW row blocks -> every wavefront multiplies one block; one block more ->
+  // that fifth block is split by columns, wavefront w taking its column block
+  // w (five MFMAs a k-step for everyone instead of eight for wavefront 0 and a
+  // barrier wait for the others); beyond that the full tile.
+  const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;
+  const bool five_tile = RAG && MT == 2 && !half_tile && m0 + (WMW + 1) * 32 >= row_hi;
+  const uint32_t avo1 = five_tile ? avo + (uint32_t)((WMW - wm) * 512) : avo + RBI * 512;   // second fragment's rows
   typedef u32x4 AFrag[4][MT];
   auto load_a_part = [&](int kt, AFrag& dst, int ks, auto ac) __attribute__((always_inline)) {   // the fragments of one k-step
     constexpr int ACT = decltype(ac)::value;
     const uint32_t so = (uint32_t)((kt * 8 + ks * 2) * 16) * (uint32_t)a.Rp;
 #pragma unroll
     for (int i = 0; i < ACT; ++i)
-      dst[ks][i] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo + i * (RBI * 512), so, 0);
+      dst[ks][i] = __builtin_amdgcn_raw_buffer_load_b128(ra, i == 0 ? avo : avo1, so, 0);
   };
   auto load_a = [&](int kt, AFrag& dst, auto ac) __attribute__((always_inline)) {
 #pragma unroll
@@ -344,7 +356,6 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // of tiles 1..3 in flight
   TabWin tw_cur, tw_nxt;
   if constexpr (TF != 0) load_win(0, tw_cur);
-  const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;   // uniform over the workgroup
   // Issue order matters: a wait counts the loads issued after the one it needs,
   // and the waits inside the loop must also hold on its first pass.  The words
   // that the loop dequantizes first (tiles 1, 2, 3) therefore go out before the
@@ -374,7 +385,12 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     for (int j = 0; j < NT; ++j)
       fb[set][j] = *reinterpret_cast<const bf16x8*>(pbase + swz(wn * (NT * 32) + j * 32 + li, ks * 2 + kh));
   };
+  bf16x8 fbx[2];                                  // fifth-block tiles: column block wm of the weight tile
+  auto read_bx = [&](const unsigned char* pbase, int ks, int set) {
+    fbx[set] = *reinterpret_cast<const bf16x8*>(pbase + swz(wm * 32 + li, ks * 2 + kh));
+  };
   read_b(smem, 0, 0);
+  if constexpr (RAG && MT == 2) read_bx(smem, 0, 0);
 
   // One K-tile.  A single wavefront per SIMD has to keep its matrix core busy
   // by itself, and both a vector-memory instruction (about 64 clocks to issue
@@ -386,17 +402,24 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // two k-steps ahead was measured too: no faster, more registers.)
   auto step = [&](int kt, auto tc, auto ac) __attribute__((always_inline)) {
     constexpr int t = decltype(tc)::value;         // kt & 3
-    constexpr int ACT = decltype(ac)::value;       // row blocks this wavefront multiplies
-    const unsigned char* pb = smem + (kt % kStages) * kStage;
-    const int nstage = (kt + 1) % kStages;
+    constexpr int ACV = decltype(ac)::value;       // row blocks this wavefront multiplies; 3 = one and a quarter
+    constexpr bool FIVE = ACV == 3;
+    constexpr int ACT = FIVE ? 1 : ACV;
+    constexpr int NM = FIVE ? NT + 1 : ACT * NT;   // MFMAs a k-step
+    const std::integral_constant<int, FIVE ? 2 : ACT> na;   // fragments loaded a k-step
+    const unsigned char* pb = smem + t * kStage;
+    constexpr int nstage = (t + 1) % kStages;
     const bool has_next = kt + 1 < KT;             // uniform
     const int kt2 = clampk(kt + 2), kt4 = clampk(kt + 4);
     float sc, bi;                                  // of tile kt+1 (the first tile of the next quad at t == 3)
     entry(clampk(kt + 1), t == 3 ? tw_nxt : tw_cur, sc, bi);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1);
-      load_a_part(kt2, af[(t + 2) & 3], ks, ac);
+      if (ks < 3) {
+        read_b(pb, ks + 1, (ks + 1) & 1);
+        if constexpr (FIVE) read_bx(pb, ks + 1, (ks + 1) & 1);
+      }
+      load_a_part(kt2, af[(t + 2) & 3], ks, na);
       if (ks == 0) load_w(kt4, wr[t & 3]);          // three K-tiles ahead of its dequantization
       if (TF != 0 && ks == 1 && t == 0) {          // next quad's table window (clamped at the end)
         const int q = (kt >> 2) + 1;
@@ -409,22 +432,28 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
         for (int j = 0; j < NT; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[i][j], 0, 0, 0);
       }
+      if constexpr (FIVE)
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[t][ks][1]),
+                                                             fbx[ks & 1], acc[1][0], 0, 0, 0);
       // (after the last tile this writes a stage nobody reads: cheaper than a branch,
       // which would split the scheduling region)
       if (PPT == 4 || (ks & 1) == 0) store_piece(nstage, wr[(t + 1) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
       // order inside the k-step: fragment reads first, then MFMA / ALU / load slots
-      __builtin_amdgcn_sched_group_barrier(0x100, NT, 0);      // ds reads
+      __builtin_amdgcn_sched_group_barrier(0x100, FIVE ? NT + 1 : NT, 0);      // ds reads
 #pragma unroll
-      for (int m = 0; m < ACT * NT; ++m) {
+      for (int m = 0; m < NM; ++m) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 32 / (ACT * NT), 0);   // a few vector ALU instructions
+        __builtin_amdgcn_sched_group_barrier(0x002, (32 + NM - 1) / NM, 0);   // a few vector ALU instructions
         if (m < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one vector-memory load
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (t == 3) tw_cur = tw_nxt;
     lds_barrier();
-    if (has_next) read_b(smem + nstage * kStage, 0, 0);
+    if (has_next) {
+      read_b(smem + nstage * kStage, 0, 0);
+      if constexpr (FIVE) read_bx(smem + nstage * kStage, 0, 0);
+    }
   };
   auto run = [&](auto ac) __attribute__((always_inline)) {
     int kt = 0;
@@ -440,6 +469,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   };
   if constexpr (RAG && MT == 2) {
     if (half_tile) run(std::integral_constant<int, 1>{});
+    else if (five_tile) run(std::integral_constant<int, 3>{});
     else run(std::integral_constant<int, MT>{});
   } else {
     run(std::integral_constant<int, MT>{});
@@ -456,6 +486,8 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     uint16_t* o16 = reinterpret_cast<uint16_t*>(smem) + wave * (32 * WC);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
+      // a fifth-block tile's second block: rows of block WMW, the 32 columns of block wm
+      const bool fifth = i == 1 && five_tile;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -471,7 +503,9 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
 #pragma unroll
       for (int q = 0; q < WC / 16; ++q) {          // 32 rows x WC/8 pieces over 64 lanes
         const int idx = q * 64 + lane, rl = idx / (WC / 8), pc = idx % (WC / 8);
-        const int m = m0 + (wm * RB0 + i * RBI) * 32 + rl, n = n0 + wn * WC + pc * 8;
+        const int m = m0 + (fifth ? WMW : wm * RB0 + i * RBI) * 32 + rl;
+        const int n = n0 + wn * WC + pc * 8 + (fifth ? wm * 32 : 0);
+        if (fifth && pc >= 4) continue;            // only column block 0 of the staging area holds results
         if (m < row_hi && n < a.N) {
           const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
           *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + n) =
@@ -487,10 +521,12 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     for (int i = 0; i < MT; ++i)
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        const int n = n0 + wn * (NT * 32) + j * 32 + li;
+        const bool fifth = i == 1 && five_tile;
+        if (fifth && j > 0) continue;
+        const int n = n0 + wn * (NT * 32) + j * 32 + li + (fifth ? wm * 32 : 0);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + (wm * RB0 + i * RBI) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          const int m = m0 + (fifth ? WMW : wm * RB0 + i * RBI) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
           if (m < row_hi && n < a.N) {
             const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
             store_out(a.y, orow * a.N + n, acc[i][j][r], a.y_dtype);

@@ -584,6 +584,31 @@ def test_grouped_qmm_with_empty_and_ragged_experts():
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
 
 
+@pytest.mark.parametrize("bits,tab", [(4, "bf16"), (8, "bf16"), (4, "f32")])
+def test_grouped_qmm_experts_around_one_row_block_past_half_a_tile(bits, tab):
+    """256-row tiles: experts of up to 128 rows run one row block a wavefront,
+    129..160 rows a fifth block split by columns, more the full tile.  Sizes on
+    both sides of each border, both epilogues (float32 and 16-byte bf16 stores),
+    a last column tile of 8 columns."""
+    rng = np.random.default_rng(77 + bits)
+    sizes = np.array([128, 129, 160, 161, 145, 97, 256])
+    e, n, k = len(sizes), 264, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, 64, tab, lead=(e,))
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    x, xd = make_x(rng, int(ro[-1]), k)
+    want = O.grouped_qmm(x, words, s, b, ro, 64, bits, weight_rounding="bf16")
+    ro_d = torch.from_numpy(ro).to(DEV)
+    y32 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=64, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=64, bits=bits))
+    for i in range(e):                       # every expert's rows by themselves
+        lo, hi = ro[i], ro[i + 1]
+        assert O.rel_l2(y32[lo:hi], want[lo:hi]) <= 2e-5, (i, O.rel_l2(y32[lo:hi], want[lo:hi]))
+        assert O.rel_l2(y16[lo:hi], want[lo:hi]) <= TOL_BF16_OUT, i
+    # the 16-bit result is the float32 one rounded once
+    assert np.array_equal(y16, out_f32(torch.from_numpy(y32).to(DEV).to(torch.bfloat16)))
+
+
 @pytest.mark.parametrize("pairs", [8, 300])
 def test_gather_qmm_unsorted_pairs(pairs):
     """Token-major, unsorted (token, expert) pairs as mx.gather_qmm takes them."""
