@@ -239,7 +239,8 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // w (five MFMAs a k-step for everyone instead of eight for wavefront 0 and a
   // barrier wait for the others); beyond that the full tile.
   const bool half_tile = RAG && MT == 2 && m0 + WMW * 32 >= row_hi;
-  const bool five_tile = RAG && MT == 2 && !half_tile && m0 + (WMW + 1) * 32 >= row_hi;
+  constexpr bool kFifth = RAG && MT == 2 && WNW == 1 && WMW * 32 == BN;   // one column block a wavefront
+  const bool five_tile = kFifth && !half_tile && m0 + (WMW + 1) * 32 >= row_hi;
   const uint32_t avo1 = five_tile ? avo + (uint32_t)((WMW - wm) * 512) : avo + RBI * 512;   // second fragment's rows
   typedef u32x4 AFrag[4][MT];
   auto load_a_part = [&](int kt, AFrag& dst, int ks, auto ac) __attribute__((always_inline)) {   // the fragments of one k-step
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     fbx[set] = *reinterpret_cast<const bf16x8*>(pbase + swz(wm * 32 + li, ks * 2 + kh));
   };
   read_b(smem, 0, 0);
-  if constexpr (RAG && MT == 2) read_bx(smem, 0, 0);
+  if constexpr (kFifth) read_bx(smem, 0, 0);
 
   // One K-tile.  A single wavefront per SIMD has to keep its matrix core busy
   // by itself, and both a vector-memory instruction (about 64 clocks to issue
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   };
   if constexpr (RAG && MT == 2) {
     if (half_tile) run(std::integral_constant<int, 1>{});
-    else if (five_tile) run(std::integral_constant<int, 3>{});
+    else if (kFifth && five_tile) run(std::integral_constant<int, kFifth ? 3 : MT>{});
     else run(std::integral_constant<int, MT>{});
   } else {
     run(std::integral_constant<int, MT>{});
