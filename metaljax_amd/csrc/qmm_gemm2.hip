@@ -154,8 +154,12 @@ __device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float 
 // in it (a branch would end the region the MFMAs are interleaved in).
 // 0: any layout, one load per entry, types read at run time (unaligned or
 // short tables).
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF>
+//
+// G64 (bf16 tables, groups of 64): a K-tile is one group, so the entry of
+// K-tile t' of a window is its t'-th, the same for every thread: no selects.
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF, bool G64>
 __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
+  static_assert(!G64 || (TF == 1 && MODE == 0), "the one-group-a-K-tile form reads bf16 windows");
   constexpr int WNW = NWAVES / WMW;
   static_assert(WNW * NT * 32 == BN, "the wavefronts must span the weight tile");
   constexpr int WM = MT * 32;                      // rows per wavefront
@@ -319,11 +323,17 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     if constexpr (TF == 3) return f16_bits_to_f32(v & 0xFFFFu);
     return __uint_as_float(v << 16);
   };
-  // (scale, bias) of K-tile kt for this thread
-  auto entry = [&](int kt, const TabWin& tw, float& sc, float& bi) {
-    if constexpr (TF != 0) {
-      sc = pick(tw.s, eidx[kt & 3]);
-      bi = MODE == 1 ? 0.f : pick(tw.b, eidx[kt & 3]);
+  // (scale, bias) of K-tile kt for this thread; tq = kt & 3 at compile time
+  // (a clamped kt past the last tile only feeds a stage that nobody reads)
+  auto entry = [&](int kt, auto tqc, const TabWin& tw, float& sc, float& bi) {
+    constexpr int tq = decltype(tqc)::value;
+    if constexpr (G64) {
+      const uint32_t vs = tw.s[0][tq >> 1], vb = tw.b[0][tq >> 1];
+      sc = __uint_as_float((tq & 1) ? (vs & 0xFFFF0000u) : (vs << 16));
+      bi = __uint_as_float((tq & 1) ? (vb & 0xFFFF0000u) : (vb << 16));
+    } else if constexpr (TF != 0) {
+      sc = pick(tw.s, eidx[tq]);
+      bi = MODE == 1 ? 0.f : pick(tw.b, eidx[tq]);
     } else {
       const int64_t ti = trow + ((kt * BK + whalf * CPT) >> gshift);
       if constexpr (MODE == 1) {
@@ -374,7 +384,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   }
   {
     float sc, bi;
-    entry(0, tw_cur, sc, bi);
+    entry(0, std::integral_constant<int, 0>{}, tw_cur, sc, bi);
 #pragma unroll
     for (int pc = 0; pc < PPT; ++pc) store_piece(0, wr[0], pc, sc, bi);
   }
@@ -413,7 +423,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     const bool has_next = kt + 1 < KT;             // uniform
     const int kt2 = clampk(kt + 2), kt4 = clampk(kt + 4);
     float sc, bi;                                  // of tile kt+1 (the first tile of the next quad at t == 3)
-    entry(clampk(kt + 1), t == 3 ? tw_nxt : tw_cur, sc, bi);
+    entry(clampk(kt + 1), std::integral_constant<int, (t + 1) & 3>{}, t == 3 ? tw_nxt : tw_cur, sc, bi);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       if (ks < 3) {
@@ -537,7 +547,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   }
 }
 
-template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF>
+template <int MODE, int BITS, int MT, int NT, int WMW, int NWAVES, bool RAG, int TF, bool G64 = false>
 void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   constexpr int BM = WMW * MT * 32;
   Gemm2Args a = a0;
@@ -549,7 +559,7 @@ void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   // three weight stages; the epilogue transposes 32 x NT*32 sixteen-bit results per wavefront there
   const size_t epi = (size_t)NWAVES * 32 * NT * 32 * 2;
   const size_t lds = epi > (size_t)(kStages * kStage) ? epi : (size_t)(kStages * kStage);
-  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG, TF>;
+  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG, TF, G64>;
   static bool configured = false;
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -565,7 +575,8 @@ void launch2_tf(const Gemm2Args& a, hipStream_t st) {
   if constexpr (MODE == 1) {
     launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1>(a, st);
   } else {
-    if (a.tab == QMM_BF16) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1>(a, st);
+    if (a.tab == QMM_BF16 && a.gs == 64) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1, true>(a, st);
+    else if (a.tab == QMM_BF16) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 1>(a, st);
     else if (a.tab == QMM_F32) launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 2>(a, st);
     else launch2_k<MODE, BITS, MT, NT, WMW, NWAVES, RAG, 3>(a, st);
   }
