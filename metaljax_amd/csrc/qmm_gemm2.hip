@@ -436,16 +436,19 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
         const int q = (kt >> 2) + 1;
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
       }
+      // The fragment read last is used first: LDS reads return in order, so
+      // one wait covers the k-step instead of one before every MFMA (a single
+      // wavefront a SIMD issues one instruction per four clocks, waits included).
+      if constexpr (FIVE)
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[t][ks][1]),
+                                                             fbx[ks & 1], acc[1][0], 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < ACT; ++i) {
         const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][i]);
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
+        for (int j = NT - 1; j >= 0; --j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[i][j], 0, 0, 0);
       }
-      if constexpr (FIVE)
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[t][ks][1]),
-                                                             fbx[ks & 1], acc[1][0], 0, 0, 0);
       // (after the last tile this writes a stage nobody reads: cheaper than a branch,
       // which would split the scheduling region)
       if (PPT == 4 || (ks & 1) == 0) store_piece(nstage, wr[(t + 1) & 3], PPT == 4 ? ks : ks / 2, sc, bi);
