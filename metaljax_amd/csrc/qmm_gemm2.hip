@@ -29,27 +29,19 @@
 // of tile t; three LDS stages, one LDS-only barrier per K-tile.
 #include <type_traits>
 
-#include "qmm_common.hpp"
+#include "qmm_gemm2_common.hpp"
 
 namespace qmm {
 
+// the grouped kernel for short row groups (qmm_gemm2s.hip)
+bool gemm2s_wanted(const g2::Gemm2Args& a, int mode, int bits);
+void gemm2s_launch(const g2::Gemm2Args& a, int mode, int bits, hipStream_t st);
+
 namespace {
 
-constexpr int BN = 128, BK = 64;
-constexpr int kRowBytes = BK * 2;                 // bf16 tile row
-constexpr int kStage = BN * kRowBytes;            // 16 KB
+using namespace g2;
+
 constexpr int kStages = 4;                        // stage of K-tile t = t & 3: a compile-time LDS offset
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
-  const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
-}
-
-__device__ __forceinline__ void lds_barrier() {   // orders LDS traffic only; global loads stay in flight
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-__device__ __forceinline__ int swz(int row, int piece) { return row * kRowBytes + ((piece ^ (row & 7)) << 4); }
 
 // ---------------------------------------------------------------------------
 // x [x_rows, K] bf16 (rows optionally gathered through lhs_idx) -> ax[K/8][Rp]
@@ -73,64 +65,6 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* __restri
   u32x4 v = {0u, 0u, 0u, 0u};
   if (ok) v = reinterpret_cast<const u32x4*>(x + src * K)[piece];
   ax[(int64_t)piece * Rp + row] = v;
-}
-
-// ---------------------------------------------------------------------------
-struct Gemm2Args {
-  const void* ax;        // re-laid activations
-  const uint32_t* w;     // [E, N, K*bits/32]
-  const void* s;         // [E, N, K/gs]
-  const void* b;
-  void* y;               // [R, N]
-  const int32_t* row_offsets;   // [E+1] or null
-  const int32_t* out_idx;       // optional row scatter for y
-  int R, N, K, E, Rp;
-  int gs, tab, y_dtype;
-  int m_tiles;
-  int tabfast;           // table rows are dword-aligned: fetch them as 16-byte windows
-};
-
-// Rows [lo, hi) of expert i, forced into [0, R] and hi >= lo whatever the offsets hold.
-__device__ __forceinline__ void group_rows(const Gemm2Args& a, int i, int& lo, int& hi) {
-  lo = a.row_offsets[i];
-  hi = a.row_offsets[i + 1];
-  lo = lo < 0 ? 0 : (lo > a.R ? a.R : lo);
-  hi = hi < lo ? lo : (hi > a.R ? a.R : hi);
-}
-
-// 32 codes (one row, one 32-group) -> four 16-byte pieces of bf16 weights
-template <int MODE, int BITS>
-__device__ __forceinline__ u32x4 dequant_piece(const uint32_t* q, int pc, float sc, float bi) {
-  float f[8];
-  if constexpr (MODE == 1) {
-    // exact: the converter widens the two codes of a byte and applies the power-of-two scale
-    const uint32_t w = q[pc];
-    return u32x4{__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 0)),
-                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 1)),
-                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 2)),
-                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 3))};
-  } else if constexpr (BITS == 8) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const uint32_t w = q[2 * pc + h];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) f[4 * h + j] = fmaf(sc, (float)((w >> (8 * j)) & 255u), bi);
-    }
-  } else {
-    const uint32_t w = q[pc];
-    uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;           // even / odd codes as bytes
-    // kept opaque, so that each code is one byte-to-float conversion of lo / hi
-    // (merged with the masks above they become a bit-field extract plus a conversion)
-    asm("" : "+v"(lo));
-    asm("" : "+v"(hi));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f[2 * j] = fmaf(sc, (float)((lo >> (8 * j)) & 255u), bi);
-      f[2 * j + 1] = fmaf(sc, (float)((hi >> (8 * j)) & 255u), bi);
-    }
-  }
-  return u32x4{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-               pack_bf16x2(f[6], f[7])};
 }
 
 // MT x NT MFMA tiles (32 x 32) per wavefront; WMW wavefronts stacked in M and
@@ -638,6 +572,7 @@ void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, 
                          (mode == QMM_MODE_MXFP4 || (reinterpret_cast<uintptr_t>(b) & 3u) == 0);
     a.tabfast = aligned && K % 256 == 0 && N * (K / g) * esz < (1ll << 31) && !getenv("QMM_G2_NOTABFAST");
   }
+  if (gemm2s_wanted(a, mode, bits)) return gemm2s_launch(a, mode, bits, st);
   const int mt = row_tile >= 256 ? 2 : 1;
   if (mode == QMM_MODE_MXFP4) launch2_mt<1, 4>(a, mt, st);
   else if (bits == 4) launch2_mt<0, 4>(a, mt, st);

@@ -1,0 +1,373 @@
+// Grouped (per-expert) prefill-regime quantized matmul for short row groups on
+// gfx950: experts of up to about 160 rows, the MoE prefill case.
+//
+// Why a second kernel.  With row groups this short a 128-column weight tile is
+// dequantized for very little matrix work: in the general kernel, where every
+// wavefront both dequantizes and multiplies, a K-tile of a 128-row tile takes
+// 0.78 us of which the MFMAs are a third; the dequantization (about 100 vector
+// ALU instructions per thread, the LDS writes, the loads that feed them) is
+// the largest part, and a single wavefront a SIMD cannot run it beside its own
+// MFMAs: it issues one instruction per four clocks, of any kind.
+//
+// So the roles are split, as in the decode kernel.  A workgroup is eight
+// wavefronts, two a SIMD:
+//   * producers (wavefronts 4-7) load the packed words and the scale / bias
+//     windows, dequantize K-tile t+1 (float32 fma, one round-to-nearest-even
+//     to bf16: the reference's tile, bit for bit) and write it to LDS;
+//   * consumers (wavefronts 0-3) load their activation fragments (the re-laid
+//     ax[k/8][row] form of the general kernel), read the weight fragments of
+//     K-tile t from LDS and issue the MFMAs.
+// The vector ALU and the matrix core of a SIMD are then driven by different
+// wavefronts and overlap; one workgroup barrier per K-tile publishes tile t+1
+// and frees the stage of tile t-1 (three stages).
+//
+// Tile: up to 160 rows x 128 columns.  Consumer w multiplies row block w
+// (32 rows) with the whole weight tile; rows 128..159, when the tile has them,
+// are a fifth block split by columns: consumer w multiplies it with column
+// block w.  Longer experts take several tiles.
+#include <type_traits>
+
+#include "qmm_gemm2_common.hpp"
+
+namespace qmm {
+
+namespace {
+
+using namespace g2;
+
+constexpr int kS = 3;                 // LDS stages: K-tile t lives in stage t % 3
+constexpr int kTileRows = 160;        // four row blocks + the fifth
+constexpr int kAR = 3;                // activation fragments: K-tile t lives in ring slot t % 3
+
+template <int MODE, int BITS, bool G64>
+__global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
+  static_assert(!G64 || MODE == 0, "one group a K-tile is an affine layout");
+  constexpr int WBITS = (MODE == 1) ? 4 : BITS;
+  constexpr int WPT = 32 * WBITS / 32;             // packed words per producer thread and K-tile: 4 | 8
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- which tile?  XCD x gets a band of column tiles of every expert,
+  // expert after expert; the grid is provisioned for the worst raggedness and
+  // only the row tiles that exist are dealt.
+  const int n_tiles = (a.N + BN - 1) / BN;
+  int m_tiles = 0;
+  for (int i = 0; i < a.E; ++i) {
+    int lo, hi;
+    group_rows(a, i, lo, hi);
+    m_tiles += (hi - lo + kTileRows - 1) / kTileRows;
+  }
+  const int band = (n_tiles + 7) / 8;
+  const int l = blockIdx.x >> 3;
+  const int tile_m = l / band;
+  const int tile_n = (blockIdx.x & 7) * band + l % band;
+  if (tile_m >= m_tiles || tile_n >= n_tiles) return;
+  int e = 0, row_lo = 0, row_hi = 0, mt_idx = 0;
+  {
+    int t = tile_m;
+    bool found = false;
+    for (int i = 0; i < a.E; ++i) {
+      int lo, hi;
+      group_rows(a, i, lo, hi);
+      const int tiles = (hi - lo + kTileRows - 1) / kTileRows;
+      if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
+      t -= tiles;
+    }
+    if (!found) return;
+  }
+  const int m0 = row_lo + mt_idx * kTileRows;
+  if (m0 >= row_hi) return;
+  const int m_end = row_hi < m0 + kTileRows ? row_hi : m0 + kTileRows;
+  const int n0 = tile_n * BN;
+  const int KT = a.K / BK;
+  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
+
+  if (wave >= 4) {
+    // ======================= producers: the weight tile ====================
+    const int ptid = tid - 256;
+    const int wrow = ptid >> 1, whalf = ptid & 1;  // weight row of the tile, 32-code half of its K-tile
+    const int64_t wpr = (int64_t)a.K * WBITS / 32;
+    const int gs = (MODE == 1) ? 32 : a.gs;
+    const int64_t ng = a.K / gs;
+    constexpr int tabsz = (MODE == 1) ? 1 : 2;     // E8M0 bytes | bf16
+    const uint32_t* wb = a.w + (int64_t)e * a.N * wpr;
+    const char* sb = static_cast<const char*>(a.s) + (int64_t)e * a.N * ng * tabsz;
+    const char* bb = (MODE == 1) ? sb : static_cast<const char*>(a.b) + (int64_t)e * a.N * ng * tabsz;
+    int64_t wn_row = n0 + wrow;
+    if (wn_row >= a.N) wn_row = a.N - 1;           // rows past N are computed and never stored
+    const auto rw = make_rsrc(wb, (int64_t)a.N * wpr * 4);
+    const uint32_t wvo = (uint32_t)((wn_row * wpr + whalf * WPT) * 4);
+    struct WRegs { uint32_t q[WPT]; };
+    auto load_w = [&](int kt, WRegs& r) {
+      const uint32_t so = (uint32_t)kt * (BK * WBITS / 8);
+#pragma unroll
+      for (int j = 0; j < WPT; j += 4) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rw, wvo + j * 4, so, 0);
+        r.q[j] = v[0]; r.q[j + 1] = v[1]; r.q[j + 2] = v[2]; r.q[j + 3] = v[3];
+      }
+    };
+    // scale / bias window: the entries of four K-tiles of this thread's row
+    // (at most 16 bytes a table), fetched once per four K-tiles
+    struct TabWin { u32x4 s, b; };
+    const auto rs = make_rsrc(sb, (int64_t)a.N * ng * tabsz);
+    const auto rb = make_rsrc(bb, (int64_t)a.N * ng * tabsz);
+    const uint32_t tvo = (uint32_t)(wn_row * ng * tabsz);
+    const int gshift = gs == 32 ? 5 : (gs == 64 ? 6 : 7);
+    auto load_win = [&](int quad, TabWin& tw) {
+      const uint32_t so = (uint32_t)(((quad * 4 * BK) >> gshift) * tabsz);
+      tw.s = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo, so, 0);
+      if constexpr (MODE == 0) tw.b = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo, so, 0);
+    };
+    uint32_t eidx[4];                              // entry of K-tile t' inside its window, for this thread's half
+#pragma unroll
+    for (int t = 0; t < 4; ++t) eidx[t] = (uint32_t)((t * BK + whalf * 32) >> gshift);
+    auto pick = [&](const u32x4& w, uint32_t ei) -> float {
+      const uint32_t byte = ei * (uint32_t)tabsz;
+      const uint32_t d = byte >> 2;
+      uint32_t v = w[0];
+      v = d == 1 ? w[1] : v;
+      v = d == 2 ? w[2] : v;
+      v = d == 3 ? w[3] : v;
+      v >>= (byte & 3u) * 8u;
+      if constexpr (MODE == 1) return e8m0_to_f32(v & 255u);
+      return __uint_as_float(v << 16);
+    };
+    auto entry = [&](auto tqc, const TabWin& tw, float& sc, float& bi) {
+      constexpr int tq = decltype(tqc)::value;
+      if constexpr (G64) {                          // one group a K-tile: entry tq for every thread
+        const uint32_t vs = tw.s[tq >> 1], vb = tw.b[tq >> 1];
+        sc = __uint_as_float((tq & 1) ? (vs & 0xFFFF0000u) : (vs << 16));
+        bi = __uint_as_float((tq & 1) ? (vb & 0xFFFF0000u) : (vb << 16));
+      } else {
+        sc = pick(tw.s, eidx[tq]);
+        bi = MODE == 1 ? 0.f : pick(tw.b, eidx[tq]);
+      }
+    };
+    auto store_tile = [&](int stage, const WRegs& r, float sc, float bi) {
+#pragma unroll
+      for (int pc = 0; pc < 4; ++pc)
+        *reinterpret_cast<u32x4*>(smem + stage * kStage + swz(wrow, whalf * 4 + pc)) =
+            dequant_piece<MODE, BITS>(r.q, pc, sc, bi);
+    };
+
+    TabWin tw_cur, tw_nxt;
+    WRegs wr[4];                                    // words of K-tile t live in wr[t & 3]
+    load_win(0, tw_cur);
+    load_w(0, wr[0]);
+    load_w(clampk(1), wr[1]);
+    load_w(clampk(2), wr[2]);
+    load_w(clampk(3), wr[3]);
+    tw_nxt = tw_cur;
+    {
+      float sc, bi;
+      entry(std::integral_constant<int, 0>{}, tw_cur, sc, bi);
+      store_tile(0, wr[0], sc, bi);
+    }
+    lds_barrier();                                  // tile 0 is published
+    // step kt runs beside the consumers' K-tile kt and publishes tile kt + 1
+    // (past the last tile it fills a stage that nobody reads)
+    auto pstep = [&](int kt, auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;        // kt & 3
+      float sc, bi;
+      entry(std::integral_constant<int, (t + 1) & 3>{}, t == 3 ? tw_nxt : tw_cur, sc, bi);
+      load_w(clampk(kt + 4), wr[t]);                // tile kt's words were used a step ago
+      if (t == 0) {                                 // next quad's windows (clamped at the end)
+        const int q = (kt >> 2) + 1;
+        load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
+      }
+      store_tile((kt + 1) % kS, wr[(t + 1) & 3], sc, bi);
+      if (t == 3) tw_cur = tw_nxt;
+      lds_barrier();
+      // every step does its own tile's arithmetic: work moved across the
+      // barrier would make the consumers wait for a long step and the
+      // producers idle in the short ones
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    int kt = 0;
+    for (; kt + 4 <= KT; kt += 4) {
+      pstep(kt, std::integral_constant<int, 0>{});
+      pstep(kt + 1, std::integral_constant<int, 1>{});
+      pstep(kt + 2, std::integral_constant<int, 2>{});
+      pstep(kt + 3, std::integral_constant<int, 3>{});
+    }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 0>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 1>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 2>{}); ++kt; }
+    return;
+  }
+
+  // ========================= consumers: the MFMAs ==========================
+  const int wm = wave;                             // row block, and column block of the fifth
+  const int li = lane & 31, kh = lane >> 5;
+  const bool five = m0 + 128 < m_end;              // uniform over the workgroup
+  // lane (row li, k-half kh) of k-step ks reads ax[(kt*8 + ks*2 + kh) * Rp + row]
+  const auto ra = make_rsrc(a.ax, (int64_t)(a.K / 8) * a.Rp * 16);
+  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * 32 + li) * 16);
+  const uint32_t avo1 = avo + (uint32_t)((4 - wm) * 512);       // the fifth block's rows
+  typedef u32x4 AFrag[4][2];
+  auto load_a_part = [&](int kt, AFrag& dst, int ks, auto nac) __attribute__((always_inline)) {
+    const uint32_t so = (uint32_t)((kt * 8 + ks * 2) * 16) * (uint32_t)a.Rp;
+    dst[ks][0] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo, so, 0);
+    if constexpr (decltype(nac)::value == 2) dst[ks][1] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo1, so, 0);
+  };
+
+  f32x16 acc[4], accx;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
+    accx[r] = 0.f;
+  }
+  AFrag af[kAR];
+  bf16x8 fb[2][4], fbx[2];                          // B fragments: k-step ks in set ks & 1
+  auto read_b = [&](const unsigned char* pbase, int ks, int set, auto fc) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      fb[set][j] = *reinterpret_cast<const bf16x8*>(pbase + swz(j * 32 + li, ks * 2 + kh));
+    if constexpr (decltype(fc)::value)
+      fbx[set] = *reinterpret_cast<const bf16x8*>(pbase + swz(wm * 32 + li, ks * 2 + kh));
+  };
+
+  auto run = [&](auto fc) __attribute__((always_inline)) {
+    constexpr bool FIVE = decltype(fc)::value;
+    const std::integral_constant<int, FIVE ? 2 : 1> nac;
+    // tiles 0 and 1 of the activations in flight before the first barrier
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) load_a_part(0, af[0], ks, nac);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) load_a_part(clampk(1), af[1], ks, nac);
+    lds_barrier();                                  // tile 0 is published
+    read_b(smem, 0, 0, fc);
+    auto cstep = [&](int kt, auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;        // kt % 3
+      const unsigned char* pb = smem + t * kStage;
+      constexpr int nstage = (t + 1) % kS;
+      const int kt2 = clampk(kt + 2);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1, fc);
+        load_a_part(kt2, af[(t + 2) % kAR], ks, nac);
+        // the fragment read last feeds the first MFMA: one LDS wait a k-step
+        if constexpr (FIVE)
+          accx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[t][ks][1]),
+                                                         fbx[ks & 1], accx, 0, 0, 0);
+        const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][0]);
+#pragma unroll
+        for (int j = 3; j >= 0; --j)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[j], 0, 0, 0);
+        // order inside the k-step: the next k-step's fragment reads first (their
+        // latency hides under this k-step's MFMAs), the loads spread between the MFMAs
+        if (ks < 3) __builtin_amdgcn_sched_group_barrier(0x100, FIVE ? 5 : 4, 0);
+#pragma unroll
+        for (int m = 0; m < (FIVE ? 5 : 4); ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (m < (FIVE ? 2 : 1)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      lds_barrier();                                // tile kt + 1 is published, tile kt's stage is free
+      if (kt + 1 < KT) read_b(smem + nstage * kStage, 0, 0, fc);
+    };
+    int kt = 0;
+    for (; kt + 3 <= KT; kt += 3) {
+      cstep(kt, std::integral_constant<int, 0>{});
+      cstep(kt + 1, std::integral_constant<int, 1>{});
+      cstep(kt + 2, std::integral_constant<int, 2>{});
+    }
+    if (kt < KT) { cstep(kt, std::integral_constant<int, 0>{}); ++kt; }
+    if (kt < KT) { cstep(kt, std::integral_constant<int, 1>{}); ++kt; }
+  };
+  if (five) run(std::true_type{});
+  else run(std::false_type{});
+
+  // ---- epilogue.  D of a 32x32 tile: lane holds column lane % 32 and rows
+  // (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5), r = 0..15.
+  const bool wide = a.y_dtype != QMM_F32 && (a.N & 7) == 0 &&
+                    (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;
+  if (wide) {
+    // 16-bit outputs: transpose each 32-row block through this wavefront's
+    // share of LDS (free after the last barrier), store 16 bytes a lane
+    uint16_t* o16 = reinterpret_cast<uint16_t*>(smem) + wave * (32 * BN);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {                   // 0: row block wm, all columns; 1: the fifth block, column block wm
+      if (i == 1 && !five) break;
+      const int ncb = i == 0 ? 4 : 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j >= ncb) break;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rl = (r & 3) + 8 * (r >> 2) + 4 * kh;
+          const float v = i == 0 ? acc[j][r] : accx[r];
+          o16[rl * BN + j * 32 + li] =
+              (uint16_t)(a.y_dtype == QMM_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int ppr = ncb * 4;                      // 16-byte pieces per row
+      for (int q = 0; q < (32 * ppr) / 64; ++q) {
+        const int idx = q * 64 + lane, rl = idx / ppr, pc = idx % ppr;
+        const int m = m0 + (i == 0 ? wm : 4) * 32 + rl;
+        const int n = n0 + (i == 0 ? 0 : wm * 32) + pc * 8;
+        if (m < m_end && n < a.N) {
+          const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
+          *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + n) =
+              *reinterpret_cast<const u32x4*>(o16 + rl * BN + pc * 8);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {                   // 4: the fifth block
+      if (j == 4 && !five) break;
+      const int n = n0 + (j < 4 ? j : wm) * 32 + li;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + (j < 4 ? wm : 4) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        if (m < m_end && n < a.N) {
+          const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
+          store_out(a.y, orow * a.N + n, j < 4 ? acc[j][r] : accx[r], a.y_dtype);
+        }
+      }
+    }
+  }
+}
+
+template <int MODE, int BITS, bool G64>
+void launch_s(const Gemm2Args& a, hipStream_t st) {
+  const int64_t m_tiles = ceil_div(a.R, kTileRows) + a.E;      // provisioned: a tile never straddles an expert
+  const int64_t total = ceil_div(ceil_div(a.N, BN), 8) * 8 * m_tiles;
+  const size_t epi = (size_t)4 * 32 * BN * 2;
+  const size_t lds = epi > (size_t)(kS * kStage) ? epi : (size_t)(kS * kStage);
+  hipLaunchKernelGGL((gemm2s_kernel<MODE, BITS, G64>), dim3((unsigned)total), dim3(512), lds, st, a);
+}
+
+}  // namespace
+
+// Short row groups (a mean of at most 144 rows an expert) with 16-byte table
+// windows of bf16 (E8M0 for MXFP4) entries; everything else stays on the
+// general kernel.
+bool gemm2s_wanted(const g2::Gemm2Args& a, int mode, int bits) {
+  static const char* env = getenv("QMM_GEMM2S");   // "0": never, "1": whenever it can run
+  if (env && env[0] == '0') return false;
+  const bool can = a.row_offsets && a.E > 0 && a.tabfast && a.K % 256 == 0 &&
+                   (mode == QMM_MODE_MXFP4 || (a.tab == QMM_BF16 && (bits == 4 || bits == 8)));
+  if (!can) return false;
+  if (env && env[0] == '1') return true;
+  return a.R / a.E <= 144;
+}
+
+void gemm2s_launch(const g2::Gemm2Args& a, int mode, int bits, hipStream_t st) {
+  if (mode == QMM_MODE_MXFP4) launch_s<1, 4, false>(a, st);
+  else if (bits == 4) { if (a.gs == 64) launch_s<0, 4, true>(a, st); else launch_s<0, 4, false>(a, st); }
+  else { if (a.gs == 64) launch_s<0, 8, true>(a, st); else launch_s<0, 8, false>(a, st); }
+}
+
+}  // namespace qmm

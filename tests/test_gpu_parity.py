@@ -609,6 +609,41 @@ def test_grouped_qmm_experts_around_one_row_block_past_half_a_tile(bits, tab):
     assert np.array_equal(y16, out_f32(torch.from_numpy(y32).to(DEV).to(torch.bfloat16)))
 
 
+@pytest.mark.parametrize("bits,gs,k", [(4, 64, 512), (4, 32, 768), (4, 128, 256), (8, 64, 1024)])
+def test_grouped_qmm_short_experts_on_the_split_role_kernel(bits, gs, k):
+    """A mean of at most 144 rows an expert with bf16 tables and K % 256 == 0
+    runs the kernel whose wavefronts are split into dequantizing producers and
+    multiplying consumers: tiles of up to 160 rows (a fifth row block split by
+    columns), longer experts in several tiles, an empty expert, a last column
+    tile of 8 columns, both epilogues, and the gathered form's row scatter."""
+    rng = np.random.default_rng(91 + bits + gs)
+    sizes = np.array([128, 129, 160, 161, 145, 97, 33, 0, 320, 1])
+    e, n = len(sizes), 264
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, lead=(e,))
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    assert r // e <= 144
+    x, xd = make_x(rng, r, k)
+    want = O.grouped_qmm(x, words, s, b, ro, gs, bits, weight_rounding="bf16")
+    ro_d = torch.from_numpy(ro).to(DEV)
+    y32 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=gs, bits=bits, out_dtype=torch.float32))
+    y16 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=gs, bits=bits))
+    for i in range(e):                       # every expert's rows by themselves
+        lo, hi = ro[i], ro[i + 1]
+        if hi > lo:
+            assert O.rel_l2(y32[lo:hi], want[lo:hi]) <= 2e-5, (i, O.rel_l2(y32[lo:hi], want[lo:hi]))
+            assert O.rel_l2(y16[lo:hi], want[lo:hi]) <= TOL_BF16_OUT, i
+    # the 16-bit result is the float32 one rounded once
+    assert np.array_equal(y16, out_f32(torch.from_numpy(y32).to(DEV).to(torch.bfloat16)))
+    # the same products as unsorted (token, expert) pairs
+    rhs = np.repeat(np.arange(e), sizes).astype(np.int32)
+    perm = rng.permutation(r)
+    yg = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(perm.astype(np.int32)).to(DEV),
+                              torch.from_numpy(rhs[perm]).to(DEV), group_size=gs, bits=bits,
+                              out_dtype=torch.float32))
+    assert O.rel_l2(yg, want[perm]) <= 2e-5, O.rel_l2(yg, want[perm])
+
+
 @pytest.mark.parametrize("pairs", [8, 300])
 def test_gather_qmm_unsorted_pairs(pairs):
     """Token-major, unsorted (token, expert) pairs as mx.gather_qmm takes them."""
