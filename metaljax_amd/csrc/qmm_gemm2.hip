@@ -20,7 +20,7 @@
 //     tid%2), dequantizes them with the row's scale/bias of that 32-group
 //     (float32 fma, one round-to-nearest-even to bf16: the reference's tile
 //     semantics, bit for bit) and writes four 16-byte pieces of the bf16 tile
-//     to LDS (piece p of row r at p ^ (r & 7));
+//     to LDS (piece p of row r at p ^ ((r >> 1) & 7): every 16-lane pass covers all banks);
 //   * every wavefront reads the whole weight tile back as B fragments and
 //     multiplies it with its own activation fragments (registers).
 // Schedule: the packed words of tile t+4 (they come from HBM and are consumed

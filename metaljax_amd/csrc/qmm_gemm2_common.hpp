@@ -21,7 +21,15 @@ __device__ __forceinline__ void lds_barrier() {   // orders LDS traffic only; gl
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-__device__ __forceinline__ int swz(int row, int piece) { return row * kRowBytes + ((piece ^ (row & 7)) << 4); }
+// A bf16 tile row is 128 bytes = half of the 64 banks, so the parity of the
+// row picks the half and 16-byte piece p of row r sits at p ^ ((r >> 1) & 7):
+// the 16 lanes of one pass of a ds_read_b128 / ds_write_b128 (16 consecutive
+// rows of one piece, or 8 rows x 2 halves of 4 pieces) then touch every bank
+// once.  (With p ^ (r & 7) rows r and r + 8 shared their banks: every fragment
+// read took two passes.)
+__device__ __forceinline__ int swz(int row, int piece) {
+  return row * kRowBytes + ((piece ^ ((row >> 1) & 7)) << 4);
+}
 
 // ---------------------------------------------------------------------------
 struct Gemm2Args {
