@@ -12,8 +12,9 @@
 // So the roles are split, as in the decode kernel.  A workgroup is eight
 // wavefronts, two a SIMD:
 //   * producers (wavefronts 4-7) load the packed words and the scale / bias
-//     windows, dequantize K-tile t+1 (float32 fma, one round-to-nearest-even
-//     to bf16: the reference's tile, bit for bit) and write it to LDS;
+//     windows, dequantize a K-tile (float32 fma, one round-to-nearest-even
+//     to bf16: the reference's tile, bit for bit) two K-tiles ahead of its use
+//     and write it to LDS one K-tile ahead;
 //   * consumers (wavefronts 0-3) load their activation fragments (the re-laid
 //     ax[k/8][row] form of the general kernel), read the weight fragments of
 //     K-tile t from LDS and issue the MFMAs.
@@ -145,39 +146,51 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
         bi = MODE == 1 ? 0.f : pick(tw.b, eidx[tq]);
       }
     };
-    auto store_tile = [&](int stage, const WRegs& r, float sc, float bi) {
+    // Pipeline of a weight tile: its words are requested six K-tiles before it
+    // is published, it is dequantized into registers two K-tiles before, and
+    // written to LDS at the start of the step before (the write then has the
+    // whole step to finish before the barrier that publishes it).
+    auto dequant_tile = [&](u32x4 (&dst)[4], const WRegs& r, float sc, float bi) {
+#pragma unroll
+      for (int pc = 0; pc < 4; ++pc) dst[pc] = dequant_piece<MODE, BITS>(r.q, pc, sc, bi);
+    };
+    auto write_tile = [&](int stage, const u32x4 (&src)[4]) {
 #pragma unroll
       for (int pc = 0; pc < 4; ++pc)
-        *reinterpret_cast<u32x4*>(smem + stage * kStage + swz(wrow, whalf * 4 + pc)) =
-            dequant_piece<MODE, BITS>(r.q, pc, sc, bi);
+        *reinterpret_cast<u32x4*>(smem + stage * kStage + swz(wrow, whalf * 4 + pc)) = src[pc];
     };
-
     TabWin tw_cur, tw_nxt;
-    WRegs wr[4];                                    // words of K-tile t live in wr[t & 3]
+    WRegs wr[8];                                    // words of K-tile t live in wr[t & 7]
+    u32x4 pend[4];                                  // the dequantized tile that the next step writes
     load_win(0, tw_cur);
-    load_w(0, wr[0]);
-    load_w(clampk(1), wr[1]);
-    load_w(clampk(2), wr[2]);
-    load_w(clampk(3), wr[3]);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) load_w(clampk(i), wr[i]);
     tw_nxt = tw_cur;
     {
       float sc, bi;
       entry(std::integral_constant<int, 0>{}, tw_cur, sc, bi);
-      store_tile(0, wr[0], sc, bi);
+      dequant_tile(pend, wr[0], sc, bi);
+      write_tile(0, pend);
+      entry(std::integral_constant<int, 1>{}, tw_cur, sc, bi);
+      dequant_tile(pend, wr[1], sc, bi);
     }
     lds_barrier();                                  // tile 0 is published
-    // step kt runs beside the consumers' K-tile kt and publishes tile kt + 1
-    // (past the last tile it fills a stage that nobody reads)
+    __builtin_amdgcn_sched_barrier(0);
+    // step kt runs beside the consumers' K-tile kt: it publishes tile kt + 1 and
+    // dequantizes tile kt + 2 (past the last tile: clamped repeats into stages
+    // that nobody reads)
     auto pstep = [&](int kt, auto tc) __attribute__((always_inline)) {
-      constexpr int t = decltype(tc)::value;        // kt & 3
-      float sc, bi;
-      entry(std::integral_constant<int, (t + 1) & 3>{}, t == 3 ? tw_nxt : tw_cur, sc, bi);
-      load_w(clampk(kt + 4), wr[t]);                // tile kt's words were used a step ago
+      constexpr int t8 = decltype(tc)::value;       // kt & 7
+      constexpr int t = t8 & 3;
+      write_tile((kt + 1) % kS, pend);
+      load_w(clampk(kt + 6), wr[(t8 + 6) & 7]);     // that slot's tile was dequantized four steps ago
       if (t == 0) {                                 // next quad's windows (clamped at the end)
         const int q = (kt >> 2) + 1;
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
       }
-      store_tile((kt + 1) % kS, wr[(t + 1) & 3], sc, bi);
+      float sc, bi;
+      entry(std::integral_constant<int, (t + 2) & 3>{}, t >= 2 ? tw_nxt : tw_cur, sc, bi);
+      dequant_tile(pend, wr[(t8 + 2) & 7], sc, bi);
       if (t == 3) tw_cur = tw_nxt;
       lds_barrier();
       // every step does its own tile's arithmetic: work moved across the
@@ -186,15 +199,23 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
-    for (; kt + 4 <= KT; kt += 4) {
+    for (; kt + 8 <= KT; kt += 8) {
       pstep(kt, std::integral_constant<int, 0>{});
       pstep(kt + 1, std::integral_constant<int, 1>{});
       pstep(kt + 2, std::integral_constant<int, 2>{});
       pstep(kt + 3, std::integral_constant<int, 3>{});
+      pstep(kt + 4, std::integral_constant<int, 4>{});
+      pstep(kt + 5, std::integral_constant<int, 5>{});
+      pstep(kt + 6, std::integral_constant<int, 6>{});
+      pstep(kt + 7, std::integral_constant<int, 7>{});
     }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 0>{}); ++kt; }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 1>{}); ++kt; }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 2>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 3>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 4>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 5>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 6>{}); ++kt; }
     return;
   }
 
