@@ -110,6 +110,44 @@ def test_grouped_and_gathered_random_case(seed):
     assert O.rel_l2(yg, want[perm]) <= 2e-5, (e, n, k, gs, bits, O.rel_l2(yg, want[perm]))
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_grouped_short_experts_random_case(seed):
+    """Grouped products that run on the split-role kernel (a mean of at most
+    144 rows an expert, bf16 tables, K % 256 == 0): many experts, empty ones,
+    experts past one 160-row tile, any N (also below one column tile and not a
+    multiple of 8), every output type."""
+    rng = np.random.default_rng(12000 + seed)
+    e = int(rng.integers(1, 13))
+    n = int(rng.choice([rng.integers(1, 128), rng.integers(128, 400)]))
+    gs = int(rng.choice([32, 64, 128]))
+    k = 256 * int(rng.integers(1, 5))
+    bits = int(rng.choice([4, 8]))
+    sizes = rng.integers(0, 150, size=e)
+    sizes[rng.integers(0, e)] += int(rng.choice([20, 120, 200]))
+    if sizes.sum() // e > 144:
+        sizes = sizes // 2 + 1
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    codes = rng.integers(0, 1 << bits, size=(e, n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, bits)
+    s = O.round_bf16(rng.uniform(0.005, 0.02, (e, n, k // gs)).astype(np.float32))
+    b = O.round_bf16(-(rng.integers(0, 1 << bits, s.shape).astype(np.float32)) * s)
+    x = O.round_bf16(rng.standard_normal((r, k)).astype(np.float32))
+    wd = torch.from_numpy(np.ascontiguousarray(words).view(np.int32)).to(DEV)
+    sd, bd, xd = _bf16_dev(s), _bf16_dev(b), _bf16_dev(x)
+    want = O.grouped_qmm(x, words, s, b, ro, gs, bits, weight_rounding="bf16")
+    out_dtype = [torch.float32, torch.bfloat16, torch.float16][seed % 3]
+    tol = 2e-5 if out_dtype == torch.float32 else (1e-2 if out_dtype == torch.bfloat16 else 2e-3)
+    y = K.grouped_qmm(xd, wd, sd, bd, torch.from_numpy(ro).to(DEV), group_size=gs, bits=bits,
+                      out_dtype=out_dtype).float().cpu().numpy()
+    assert y.shape == want.shape
+    if r:
+        assert O.rel_l2(y, want) <= tol, (e, n, k, gs, bits, sizes, O.rel_l2(y, want))
+        for lo, hi in zip(ro[:-1], ro[1:]):
+            if hi > lo:
+                assert O.rel_l2(y[lo:hi], want[lo:hi]) <= tol, (lo, hi)
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_one_pass_decode_random_case(seed):
     """Decode shapes whose K is exactly one pass of eight 256-byte slices (the
