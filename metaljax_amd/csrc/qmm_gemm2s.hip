@@ -146,10 +146,11 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
         bi = MODE == 1 ? 0.f : pick(tw.b, eidx[tq]);
       }
     };
-    // Pipeline of a weight tile: its words are requested six K-tiles before it
-    // is published, it is dequantized into registers two K-tiles before, and
-    // written to LDS at the start of the step before (the write then has the
-    // whole step to finish before the barrier that publishes it).
+    // Pipeline of a weight tile: its words are requested a quad at a time,
+    // seven to ten K-tiles before it is published, it is dequantized into
+    // registers two K-tiles before, and written to LDS at the start of the
+    // step before (the write then has the whole step to finish before the
+    // barrier that publishes it).
     auto dequant_tile = [&](u32x4 (&dst)[4], const WRegs& r, float sc, float bi) {
 #pragma unroll
       for (int pc = 0; pc < 4; ++pc) dst[pc] = dequant_piece<MODE, BITS>(r.q, pc, sc, bi);
@@ -160,11 +161,22 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
         *reinterpret_cast<u32x4*>(smem + stage * kStage + swz(wrow, whalf * 4 + pc)) = src[pc];
     };
     TabWin tw_cur, tw_nxt;
-    WRegs wr[8];                                    // words of K-tile t live in wr[t & 7]
+    // Words of K-tile t live in wr[t % 12].  They are requested a quad (four
+    // K-tiles) at a time: the four 16-byte pieces that a thread needs for a
+    // quad lie in one 128-byte line of its row (four-bit codes; two lines with
+    // eight-bit codes), and asked for one K-tile at a time the line came in
+    // four times, each time evicted again by the 36 KB a K-tile moves through
+    // the 32 KB L1.
+    WRegs wr[12];
     u32x4 pend[4];                                  // the dequantized tile that the next step writes
-    load_win(0, tw_cur);
+    auto load_quad = [&](int kt0, auto sc0) __attribute__((always_inline)) {
+      constexpr int s0 = decltype(sc0)::value;      // ring slot of tile kt0
 #pragma unroll
-    for (int i = 0; i < 6; ++i) load_w(clampk(i), wr[i]);
+      for (int i = 0; i < 4; ++i) load_w(clampk(kt0 + i), wr[(s0 + i) % 12]);
+    };
+    load_win(0, tw_cur);
+    load_quad(0, std::integral_constant<int, 0>{});
+    load_quad(4, std::integral_constant<int, 4>{});
     tw_nxt = tw_cur;
     {
       float sc, bi;
@@ -180,17 +192,19 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     // dequantizes tile kt + 2 (past the last tile: clamped repeats into stages
     // that nobody reads)
     auto pstep = [&](int kt, auto tc) __attribute__((always_inline)) {
-      constexpr int t8 = decltype(tc)::value;       // kt & 7
-      constexpr int t = t8 & 3;
+      constexpr int t12 = decltype(tc)::value;      // kt % 12
+      constexpr int t = t12 & 3;
       write_tile((kt + 1) % kS, pend);
-      load_w(clampk(kt + 6), wr[(t8 + 6) & 7]);     // that slot's tile was dequantized four steps ago
-      if (t == 0) {                                 // next quad's windows (clamped at the end)
-        const int q = (kt >> 2) + 1;
+      if constexpr (t == 0) {
+        // the quad two ahead, into the slots of the quad before this one
+        // (its last tile was dequantized three steps ago)
+        load_quad(kt + 8, std::integral_constant<int, (t12 + 8) % 12>{});
+        const int q = (kt >> 2) + 1;                // next quad's windows (clamped at the end)
         load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
       }
       float sc, bi;
       entry(std::integral_constant<int, (t + 2) & 3>{}, t >= 2 ? tw_nxt : tw_cur, sc, bi);
-      dequant_tile(pend, wr[(t8 + 2) & 7], sc, bi);
+      dequant_tile(pend, wr[(t12 + 2) % 12], sc, bi);
       if (t == 3) tw_cur = tw_nxt;
       lds_barrier();
       // every step does its own tile's arithmetic: work moved across the
@@ -199,7 +213,7 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
-    for (; kt + 8 <= KT; kt += 8) {
+    for (; kt + 12 <= KT; kt += 12) {
       pstep(kt, std::integral_constant<int, 0>{});
       pstep(kt + 1, std::integral_constant<int, 1>{});
       pstep(kt + 2, std::integral_constant<int, 2>{});
@@ -208,6 +222,10 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       pstep(kt + 5, std::integral_constant<int, 5>{});
       pstep(kt + 6, std::integral_constant<int, 6>{});
       pstep(kt + 7, std::integral_constant<int, 7>{});
+      pstep(kt + 8, std::integral_constant<int, 8>{});
+      pstep(kt + 9, std::integral_constant<int, 9>{});
+      pstep(kt + 10, std::integral_constant<int, 10>{});
+      pstep(kt + 11, std::integral_constant<int, 11>{});
     }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 0>{}); ++kt; }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 1>{}); ++kt; }
@@ -216,6 +234,10 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     if (kt < KT) { pstep(kt, std::integral_constant<int, 4>{}); ++kt; }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 5>{}); ++kt; }
     if (kt < KT) { pstep(kt, std::integral_constant<int, 6>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 7>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 8>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 9>{}); ++kt; }
+    if (kt < KT) { pstep(kt, std::integral_constant<int, 10>{}); ++kt; }
     return;
   }
 
