@@ -46,10 +46,13 @@
 //   XR activation rounds  [CW slices][16 rows m][256 bytes = 128 codes of x]
 //   TMAX weight tiles     [CW slices][16 rows n][256 packed bytes] + table rows
 // Every item is CW * 4 KB.  Inside a slice's 4 KB, row r holds its 16-byte
-// piece p at position p ^ (r & 7): the loader lane that fills position
-// (r, lp) fetches global piece lp ^ (r & 7), so the global access stays inside
-// the same 128-byte segments (coalesced) and the operand-order readback
-// (lane = row l % 16) is spread over the banks without padding.
+// piece p at position p ^ (r & 15): the loader lane that fills position
+// (r, lp) fetches global piece lp ^ (r & 15), so the global access stays inside
+// the row's 256 bytes (coalesced) and the operand-order readback (lane = row
+// l % 16: sixteen rows of one piece in a pass) touches sixteen different
+// positions, i.e. every bank once, without padding.  (With p ^ (r & 7) rows r
+// and r + 8 shared their banks: SQ_LDS_BANK_CONFLICT was 36 % of
+// SQ_LDS_IDX_ACTIVE.)
 //
 // Synchronisation is one workgroup barrier per item: a loader wavefront
 // arrives after its share of item i has landed, a compute wavefront after it
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     for (int o = 0; o < 4; ++o) {
       const int rq = (lw + o) & 3;
       const int row = 4 * rq + lrow;
-      const uint32_t gp = (uint32_t)(lp ^ (row & 7));
+      const uint32_t gp = (uint32_t)(lp ^ (row & 15));
       wrow[o] = row;
       wv[o] = (uint32_t)((n_begin + row) * wpr) + gp * 16;
       xv[o] = row < a.M ? (uint32_t)((int64_t)row * a.K * 2) + gp * 16 : kOutOfRange;
@@ -423,7 +426,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   } else {
     // ----------------------------------------------------- compute wavefronts
     const int r = lane & 15, kg = lane >> 4;
-    const uint32_t swz = (uint32_t)(r & 7);
+    const uint32_t swz = (uint32_t)(r & 15);
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const uint32_t one = pin_vgpr(kOnesBf16x2);
     const bf16x8 ones = as_bf16x8(one, one, one, one);
