@@ -94,16 +94,25 @@ def quantized_matmul(x, w, scales, biases=None, transpose=True, group_size=64, b
 
 
 def grouped_qmm(x, w, scales, biases, row_offsets, group_size=64, bits=4, mode="affine",
-                out_dtype=None):
+                out_dtype=None, out=None):
     """Rows of x [R,K] sorted by expert; rows [row_offsets[e], row_offsets[e+1])
     multiply expert e's weight w[e] ([E,N,...]).  row_offsets int32 [E+1] on the
-    device.  Returns [R,N]."""
+    device.  Returns [R,N]: a new tensor whose rows outside the offsets are
+    zero, or `out` (contiguous [R,N] of the output type), whose rows outside the
+    offsets are left as they are."""
     _need_cuda(x, w, scales, biases, row_offsets)
     lib = _lib.load()
     (e,), n, k = _weight_dims(w, bits, mode)
     r = x.shape[0]
-    out_dtype = out_dtype or x.dtype
-    y = torch.zeros((r, n), dtype=out_dtype, device=x.device)
+    if out is not None:
+        _need_cuda(out)
+        out_dtype = out_dtype or out.dtype
+        if tuple(out.shape) != (r, n) or out.dtype != out_dtype or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous [{r},{n}] tensor of {out_dtype}")
+        y = out
+    else:
+        out_dtype = out_dtype or x.dtype
+        y = torch.zeros((r, n), dtype=out_dtype, device=x.device)
     x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
     biases = None if biases is None else biases.contiguous()
     ro = row_offsets.to(torch.int32).contiguous()

@@ -644,6 +644,29 @@ def test_grouped_qmm_short_experts_on_the_split_role_kernel(bits, gs, k):
     assert O.rel_l2(yg, want[perm]) <= 2e-5, O.rel_l2(yg, want[perm])
 
 
+def test_grouped_qmm_into_a_given_output_leaves_uncovered_rows_alone():
+    """out=: rows inside the offsets are written, the others keep what they
+    held (a fresh output has zeros there)."""
+    rng = np.random.default_rng(33)
+    e, n, k = 2, 72, 256
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    ro = np.array([2, 40, 61], dtype=np.int32)          # rows 0-1 and 61-63 belong to no expert
+    x, xd = make_x(rng, 64, k)
+    want = O.grouped_qmm(x, words, s, b, ro, 64, 4, weight_rounding="bf16")
+    ro_d = torch.from_numpy(ro).to(DEV)
+    fresh = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=64, bits=4, out_dtype=torch.float32))
+    assert not fresh[:2].any() and not fresh[61:].any()
+    given = torch.full((64, n), 7.0, dtype=torch.float32, device=DEV)
+    ret = K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=64, bits=4, out=given)
+    assert ret is given
+    got = out_f32(given)
+    assert np.array_equal(got[2:61], fresh[2:61])
+    assert (got[:2] == 7.0).all() and (got[61:] == 7.0).all()
+    assert O.rel_l2(got[2:61], want[2:61]) <= 2e-5
+    with pytest.raises(ValueError):
+        K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=64, bits=4, out=given[:, :8])
+
+
 @pytest.mark.parametrize("pairs", [8, 300])
 def test_gather_qmm_unsorted_pairs(pairs):
     """Token-major, unsorted (token, expert) pairs as mx.gather_qmm takes them."""
