@@ -1,5 +1,8 @@
 // Grouped (per-expert) prefill-regime quantized matmul for short row groups on
-// gfx950: experts of up to about 160 rows, the MoE prefill case.
+// gfx950: experts of up to about 160 rows, the MoE prefill case.  It serves the
+// expert-indexed product that the reference hands to mx.gather_qmm
+// (src/metaljax/moe.py:1283-1340) with the dequantization semantics of
+// src/metaljax/qmm.py:71-79 (w = scale * q + bias as one fma).
 //
 // Why a second kernel.  With row groups this short a 128-column weight tile is
 // dequantized for very little matrix work: in the general kernel, where every
