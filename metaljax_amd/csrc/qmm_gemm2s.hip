@@ -42,8 +42,15 @@ using namespace g2;
 constexpr int kS = 3;                 // LDS stages: K-tile t lives in stage t % 3
 constexpr int kTileRows = 160;        // four row blocks + the fifth
 constexpr int kAR = 3;                // activation fragments: K-tile t lives in ring slot t % 3
+// Table rows staged in LDS (a row's scales / biases of the whole K when they
+// fit 128 bytes): 128 + 16 bytes a row, so that eight rows fall on different banks.
+constexpr int kTabRow = 144;
+constexpr int kTabKind = BN * kTabRow;
 
-template <int MODE, int BITS, bool G64>
+// TLDS: a tile's table rows are fetched once, into LDS (each row's line comes
+// in once instead of once per four K-tiles); otherwise 16-byte windows per
+// four K-tiles in registers.
+template <int MODE, int BITS, bool G64, bool TLDS>
 __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
   static_assert(!G64 || MODE == 0, "one group a K-tile is an affine layout");
   constexpr int WBITS = (MODE == 1) ? 4 : BITS;
@@ -138,9 +145,19 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       if constexpr (MODE == 1) return e8m0_to_f32(v & 255u);
       return __uint_as_float(v << 16);
     };
-    auto entry = [&](auto tqc, const TabWin& tw, float& sc, float& bi) {
+    unsigned char* tabs = smem + kS * kStage + wrow * kTabRow;
+    auto entry = [&](int kt, auto tqc, const TabWin& tw, float& sc, float& bi) {
       constexpr int tq = decltype(tqc)::value;
-      if constexpr (G64) {                          // one group a K-tile: entry tq for every thread
+      if constexpr (TLDS) {
+        const int ei = (kt * BK + whalf * 32) >> gshift;
+        if constexpr (MODE == 1) {
+          sc = e8m0_to_f32(tabs[ei]);
+          bi = 0.f;
+        } else {
+          sc = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(tabs)[ei]);
+          bi = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(tabs + kTabKind)[ei]);
+        }
+      } else if constexpr (G64) {                          // one group a K-tile: entry tq for every thread
         const uint32_t vs = tw.s[tq >> 1], vb = tw.b[tq >> 1];
         sc = __uint_as_float((tq & 1) ? (vs & 0xFFFF0000u) : (vs << 16));
         bi = __uint_as_float((tq & 1) ? (vb & 0xFFFF0000u) : (vb << 16));
@@ -177,16 +194,28 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) load_w(clampk(kt0 + i), wr[(s0 + i) % 12]);
     };
-    load_win(0, tw_cur);
+    if constexpr (TLDS) {
+      // this thread's half (64 bytes) of its row's table, per kind; the other
+      // half is its neighbour lane's, and a wavefront's LDS accesses stay in order
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t o = (uint32_t)(whalf * 64 + i * 16);
+        *reinterpret_cast<u32x4*>(tabs + o) = __builtin_amdgcn_raw_buffer_load_b128(rs, tvo + o, 0, 0);
+        if constexpr (MODE == 0)
+          *reinterpret_cast<u32x4*>(tabs + kTabKind + o) = __builtin_amdgcn_raw_buffer_load_b128(rb, tvo + o, 0, 0);
+      }
+    } else {
+      load_win(0, tw_cur);
+    }
     load_quad(0, std::integral_constant<int, 0>{});
     load_quad(4, std::integral_constant<int, 4>{});
     tw_nxt = tw_cur;
     {
       float sc, bi;
-      entry(std::integral_constant<int, 0>{}, tw_cur, sc, bi);
+      entry(0, std::integral_constant<int, 0>{}, tw_cur, sc, bi);
       dequant_tile(pend, wr[0], sc, bi);
       write_tile(0, pend);
-      entry(std::integral_constant<int, 1>{}, tw_cur, sc, bi);
+      entry(clampk(1), std::integral_constant<int, 1>{}, tw_cur, sc, bi);
       dequant_tile(pend, wr[1], sc, bi);
     }
     lds_barrier();                                  // tile 0 is published
@@ -202,11 +231,13 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
         // the quad two ahead, into the slots of the quad before this one
         // (its last tile was dequantized three steps ago)
         load_quad(kt + 8, std::integral_constant<int, (t12 + 8) % 12>{});
-        const int q = (kt >> 2) + 1;                // next quad's windows (clamped at the end)
-        load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
+        if constexpr (!TLDS) {
+          const int q = (kt >> 2) + 1;              // next quad's windows (clamped at the end)
+          load_win(q * 4 < KT ? q : (kt >> 2), tw_nxt);
+        }
       }
       float sc, bi;
-      entry(std::integral_constant<int, (t + 2) & 3>{}, t >= 2 ? tw_nxt : tw_cur, sc, bi);
+      entry(clampk(kt + 2), std::integral_constant<int, (t + 2) & 3>{}, t >= 2 ? tw_nxt : tw_cur, sc, bi);
       dequant_tile(pend, wr[(t12 + 2) % 12], sc, bi);
       if (t == 3) tw_cur = tw_nxt;
       lds_barrier();
@@ -386,13 +417,30 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
   }
 }
 
-template <int MODE, int BITS, bool G64>
-void launch_s(const Gemm2Args& a, hipStream_t st) {
+template <int MODE, int BITS, bool G64, bool TLDS>
+void launch_k(const Gemm2Args& a, hipStream_t st) {
   const int64_t m_tiles = ceil_div(a.R, kTileRows) + a.E;      // provisioned: a tile never straddles an expert
   const int64_t total = ceil_div(ceil_div(a.N, BN), 8) * 8 * m_tiles;
   const size_t epi = (size_t)4 * 32 * BN * 2;
-  const size_t lds = epi > (size_t)(kS * kStage) ? epi : (size_t)(kS * kStage);
-  hipLaunchKernelGGL((gemm2s_kernel<MODE, BITS, G64>), dim3((unsigned)total), dim3(512), lds, st, a);
+  const size_t need = (size_t)(kS * kStage) + (TLDS ? 2 * kTabKind : 0);
+  const size_t lds = epi > need ? epi : need;
+  auto kern = gemm2s_kernel<MODE, BITS, G64, TLDS>;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(512), lds, st, a);
+}
+
+template <int MODE, int BITS, bool G64>
+void launch_s(const Gemm2Args& a, hipStream_t st) {
+  // a row's table of the whole K in one 128-byte line per kind?
+  const int64_t row_bytes = MODE == 1 ? a.K / 32 : (int64_t)(a.K / a.gs) * 2;
+  static const bool no_tlds = getenv("QMM_GEMM2S_NOTLDS") != nullptr;
+  if (row_bytes <= 128 && !no_tlds) launch_k<MODE, BITS, G64, true>(a, st);
+  else launch_k<MODE, BITS, G64, false>(a, st);
 }
 
 }  // namespace
