@@ -10,7 +10,8 @@ namespace qmm {
 
 void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int gs, int bits,
-                   int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st);
+                   int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t n_experts,
+                   int64_t n_xrows, hipStream_t st);
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
@@ -61,7 +62,9 @@ int fail(int code, const char* fmt, ...) {
 }
 
 int check_launch(const char* what) {
-  hipError_t e = hipGetLastError();
+  hipError_t e = setup_error();                   // a failed launch set-up (nothing was launched)
+  setup_error() = hipSuccess;
+  if (e == hipSuccess) e = hipGetLastError();
   if (e != hipSuccess) return fail(QMM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
   return QMM_OK;
 }
@@ -185,7 +188,7 @@ size_t route_bytes_segments(int64_t P, int64_t E) {
 // 14336 x 4096: 128 pairs 151 against 235 us, 256 pairs 239 against 244 us, 512
 // pairs 436 against 237 us.
 bool grouped_decode_pairs(int64_t P, int64_t E) {
-  static const int64_t gd_max = getenv("QMM_GD_MAX") ? atoll(getenv("QMM_GD_MAX")) : 0;
+  static const int64_t gd_max = experiment_env("QMM_GD_MAX") ? atoll(experiment_env("QMM_GD_MAX")) : 0;
   if (P < kGroupedDecodeMinPairs) return false;
   return gd_max ? P <= gd_max : P <= 16 * E && P <= 4096;
 }
@@ -237,7 +240,7 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
     int waves, rows, rows2;
     skinny_geometry(N, K, bits, &waves, &rows);
     // eight compute + four loader wavefronts where the loader kernel serves the shape
-    const bool loaders = !getenv("QMM_SKINNY_V1") && skinny2_plan(M, N, K, bits, &rows2);
+    const bool loaders = !experiment_env("QMM_SKINNY_V1") && skinny2_plan(M, N, K, bits, &rows2);
     if (loaders) rows = rows2;
     if (kernel) *kernel = QMM_KERNEL_GEMV;
     if (grid) *grid = (int)ceil_div(N, rows);
@@ -276,7 +279,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (M <= kGemvMaxM) {
     gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, batch, M, N, K, group_size,
-                  bits, mode, nullptr, nullptr, st);
+                  bits, mode, nullptr, nullptr, 0, 0, st);
     return check_launch("gemv launch");
   }
   const int wbits = mode == QMM_MODE_MXFP4 ? 4 : bits;
@@ -385,7 +388,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   if (P > INT32_MAX / 2 || N > INT32_MAX || K > INT32_MAX || E > 65535 || T * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  static const bool no_grouped_decode = getenv("QMM_NO_GROUPED_DECODE") != nullptr;
+  static const bool no_grouped_decode = experiment_env("QMM_NO_GROUPED_DECODE") != nullptr;
   if (grouped_decode_pairs(P, E) && !no_grouped_decode && workspace &&
       workspace_bytes >= route_bytes_segments(P, E) &&
       skinny2_grouped_supported(N, K, group_size, bits, mode, table_dtype, scales, biases, E)) {
@@ -404,7 +407,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   }
   if (P <= kGatherGemvMaxPairs) {
     gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, P, 1, N, K, group_size, bits,
-                  mode, lhs_idx, rhs_idx, st);
+                  mode, lhs_idx, rhs_idx, E, T, st);
     return check_launch("gather gemv launch");
   }
   const size_t need = route_bytes(P, E);

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/qmm_hip.h"
 
@@ -101,5 +102,43 @@ __device__ __forceinline__ uint32_t byte_perm(uint32_t hi, uint32_t lo, uint32_t
 }
 
 __host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- host-side helpers ------------------------------------------------------
+
+// Experiment switches (kernel overrides used while measuring).  The shipped
+// library reads no environment: they exist only in a build with
+// -DQMM_EXPERIMENTS.
+inline const char* experiment_env(const char* name) {
+#ifdef QMM_EXPERIMENTS
+  return getenv(name);
+#else
+  (void)name;
+  return nullptr;
+#endif
+}
+
+// The status of the last failed launch set-up on this thread (hipSuccess when
+// none); the C ABI turns it into QMM_ERR_HIP and clears it.
+inline hipError_t& setup_error() {
+  static thread_local hipError_t e = hipSuccess;
+  return e;
+}
+
+// Raises kernel KERN's dynamic-LDS limit.  The HIP call is made once per
+// process (the initialisation of a function-local static is thread-safe) and
+// its status is kept: every later call reports the same status, so a launch
+// behind a failed set-up is never attempted.  Returns true when the limit is set.
+template <auto KERN>
+inline bool lds_limit(size_t bytes) {
+  static const size_t set_bytes = bytes;
+  static const hipError_t rc = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(KERN), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  hipError_t r = rc;
+  if (r == hipSuccess && bytes > set_bytes)      // a later call asking for more than the first did
+    r = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (r != hipSuccess) setup_error() = r;
+  return r == hipSuccess;
+}
 
 }  // namespace qmm

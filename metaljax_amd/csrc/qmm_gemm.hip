@@ -335,13 +335,8 @@ void launch(const GemmArgs& a0, hipStream_t st) {
   const int64_t total = ceil_div(a.N, BN) * a.m_tiles;
   dim3 grid((unsigned)(ceil_div(total, 8) * 8));
   const size_t lds = 3 * (size_t)(BM + BN) * kRowBytes;
-  auto kern = gemm_kernel<MODE, BITS, BM>;
-  static bool configured = false;                 // per instantiation
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    configured = true;
-  }
+  constexpr auto kern = gemm_kernel<MODE, BITS, BM>;
+  if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds, st, a);
 }
 
@@ -352,7 +347,7 @@ void launch_bm(const GemmArgs& a, int bm, hipStream_t st) {
 }
 
 int env_int(const char* name) {
-  const char* e = getenv(name);
+  const char* e = experiment_env(name);
   return e ? atoi(e) : 0;
 }
 

@@ -496,13 +496,8 @@ void launch2_k(const Gemm2Args& a0, hipStream_t st) {
   // three weight stages; the epilogue transposes 32 x NT*32 sixteen-bit results per wavefront there
   const size_t epi = (size_t)NWAVES * 32 * NT * 32 * 2;
   const size_t lds = epi > (size_t)(kStages * kStage) ? epi : (size_t)(kStages * kStage);
-  auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG, TF, G64>;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    configured = true;
-  }
+  constexpr auto kern = gemm2_kernel<MODE, BITS, MT, NT, WMW, NWAVES, RAG, TF, G64>;
+  if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(64 * NWAVES), lds, st, a);
 }
 
@@ -536,7 +531,7 @@ int64_t prep_rows(int64_t R) { return ceil_div(R + 256, 64) * 64; }   // a tile 
 }  // namespace
 
 bool gemm2_supported(int64_t R, int64_t N, int64_t K) {
-  if (getenv("QMM_GEMM_V1")) return false;
+  if (experiment_env("QMM_GEMM_V1")) return false;
   return K > 0 && K % 64 == 0 && prep_rows(R) * K * 2 < (1ll << 32) && N * K < (1ll << 31);
 }
 
@@ -570,7 +565,7 @@ void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, 
     const int g = mode == QMM_MODE_MXFP4 ? 32 : gs;
     const bool aligned = ((K / g) * esz) % 4 == 0 && (reinterpret_cast<uintptr_t>(s) & 3u) == 0 &&
                          (mode == QMM_MODE_MXFP4 || (reinterpret_cast<uintptr_t>(b) & 3u) == 0);
-    a.tabfast = aligned && K % 256 == 0 && N * (K / g) * esz < (1ll << 31) && !getenv("QMM_G2_NOTABFAST");
+    a.tabfast = aligned && K % 256 == 0 && N * (K / g) * esz < (1ll << 31) && !experiment_env("QMM_G2_NOTABFAST");
   }
   if (gemm2s_wanted(a, mode, bits)) return gemm2s_launch(a, mode, bits, st);
   const int mt = row_tile >= 256 ? 2 : 1;

@@ -424,13 +424,8 @@ void launch_k(const Gemm2Args& a, hipStream_t st) {
   const size_t epi = (size_t)4 * 32 * BN * 2;
   const size_t need = (size_t)(kS * kStage) + (TLDS ? 2 * kTabKind : 0);
   const size_t lds = epi > need ? epi : need;
-  auto kern = gemm2s_kernel<MODE, BITS, G64, TLDS>;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    configured = true;
-  }
+  constexpr auto kern = gemm2s_kernel<MODE, BITS, G64, TLDS>;
+  if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(512), lds, st, a);
 }
 
@@ -438,7 +433,7 @@ template <int MODE, int BITS, bool G64>
 void launch_s(const Gemm2Args& a, hipStream_t st) {
   // a row's table of the whole K in one 128-byte line per kind?
   const int64_t row_bytes = MODE == 1 ? a.K / 32 : (int64_t)(a.K / a.gs) * 2;
-  static const bool no_tlds = getenv("QMM_GEMM2S_NOTLDS") != nullptr;
+  static const bool no_tlds = experiment_env("QMM_GEMM2S_NOTLDS") != nullptr;
   if (row_bytes <= 128 && !no_tlds) launch_k<MODE, BITS, G64, true>(a, st);
   else launch_k<MODE, BITS, G64, false>(a, st);
 }
@@ -449,7 +444,7 @@ void launch_s(const Gemm2Args& a, hipStream_t st) {
 // windows of bf16 (E8M0 for MXFP4) entries; everything else stays on the
 // general kernel.
 bool gemm2s_wanted(const g2::Gemm2Args& a, int mode, int bits) {
-  static const char* env = getenv("QMM_GEMM2S");   // "0": never, "1": whenever it can run
+  static const char* env = experiment_env("QMM_GEMM2S");   // "0": never, "1": whenever it can run
   if (env && env[0] == '0') return false;
   const bool can = a.row_offsets && a.E > 0 && a.tabfast && a.K % 256 == 0 &&
                    (mode == QMM_MODE_MXFP4 || (a.tab == QMM_BF16 && (bits == 4 || bits == 8)));

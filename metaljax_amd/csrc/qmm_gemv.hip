@@ -64,9 +64,14 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
   const int64_t wpr = (int64_t)a.K * BITS / 32;             // words per weight row
   const int64_t ng = (int64_t)((a.K / CH) >> a.gshift);     // table entries per row
 
-  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
-  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+  bool x_ok = true;
+  if (a.rhs_idx) {                                  // gather form: indices are data
+    if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
+    if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
+  }
+  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? (int64_t)a.M * a.K * 2 : 0);
   const auto rw = make_rsrc(a.w + wz * a.N * wpr, a.N * wpr * 4);
   const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
   const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
@@ -227,8 +232,13 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
   const int64_t wpr = (int64_t)a.K / 8;
   const int nblk = a.K / 32;                       // MX blocks per row
 
-  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  bool x_ok = true;
+  if (a.rhs_idx) {                                  // gather form: indices are data
+    if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
+    if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
+  }
   const uint16_t* xb = a.x + xz * a.M * (int64_t)a.K;
   const uint32_t* wb = a.w + wz * a.N * wpr;
   const uint8_t* sb = static_cast<const uint8_t*>(a.s) + wz * a.N * (int64_t)nblk;
@@ -246,7 +256,7 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
     wrow[t] = wb + n * wpr;
     srow[t] = sb + n * nblk;
   }
-  const bool xvalid = r < a.M;
+  const bool xvalid = r < a.M && x_ok;
   const uint16_t* xrow = xb + (int64_t)(xvalid ? r : 0) * a.K;
 
   f32x4 acc[T];
@@ -366,7 +376,7 @@ void launch_mxfp4(const GemvArgs& a, int64_t batch, Geometry g, hipStream_t st) 
 }
 
 int env_int(const char* name) {
-  const char* e = getenv(name);
+  const char* e = experiment_env(name);
   return e ? atoi(e) : 0;
 }
 
@@ -399,7 +409,8 @@ void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves) {
 // M <= 16, K % 32 == 0, K % group_size == 0, x bf16.
 void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
                    int y_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int gs, int bits,
-                   int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, hipStream_t st) {
+                   int mode, const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t n_experts,
+                   int64_t n_xrows, hipStream_t st) {
   static const int env_u = env_int("QMM_GEMV_U");
   GemvArgs a;
   a.x = static_cast<const uint16_t*>(x);
@@ -413,6 +424,8 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
   a.y_dtype = y_dtype;
   a.lhs_idx = lhs_idx;
   a.rhs_idx = rhs_idx;
+  a.n_experts = (int)n_experts;
+  a.n_xrows = (int)n_xrows;
   static const int no_skinny = env_int("QMM_NO_SKINNY");
   if (!no_skinny && skinny_supported(N, K, gs, bits, mode, tab, s, b)) {
     // big weights: the kernel with loader wavefronts (QMM_SKINNY_V1 keeps the

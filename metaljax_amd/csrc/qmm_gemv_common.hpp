@@ -55,8 +55,13 @@ struct GemvArgs {
   int gshift;          // log2(group_size / CH)
   int y_dtype;
   // gather form: batch entry z multiplies x[lhs_idx[z]] by w[rhs_idx[z]]
+  // (rhs_idx set = gather form; then n_experts / n_xrows bound the indices: a
+  // pair whose expert is outside [0, n_experts) writes nothing, a row outside
+  // [0, n_xrows) reads as zeros)
   const int32_t* lhs_idx;
   const int32_t* rhs_idx;
+  int n_experts = 0;
+  int n_xrows = 0;
   // grouped decode (loader-wavefront kernel, direct variants): workgroup row
   // blockIdx.y takes segment y of `segments` ([0] = count, then (expert, first
   // sorted position, rows <= 16) triples): it multiplies the rows

@@ -485,7 +485,7 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
 static int64_t mx_rows(int64_t R) { return ceil_div(R + TM, TM) * TM; }
 
 bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K) {
-  if (getenv("QMM_NO_MXFP4_MFMA")) return false;
+  if (experiment_env("QMM_NO_MXFP4_MFMA")) return false;
   return K > 0 && K % 512 == 0 && N * (K / 2) < (1ll << 31) && mx_rows(R) * K * 3 / 2 < (1ll << 32) &&
          mx_rows(R) * 4 * 8 < (1ll << 31);
 }
@@ -524,12 +524,7 @@ void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, i
   a.m_tiles = (int)(ceil_div(R, TM) + (row_offsets ? E : 0));
   a.n_tiles = (int)ceil_div(N, TN);
   const int grid = (int)(ceil_div((int64_t)a.m_tiles * a.n_tiles, 8) * 8), block = 256;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mxfp4_mfma_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    attr_set = true;
-  }
+  if (!lds_limit<mxfp4_mfma_kernel>(kLds)) return;
   hipLaunchKernelGGL(mxfp4_mfma_kernel, dim3(grid), dim3(block), kLds, st, a);
 }
 

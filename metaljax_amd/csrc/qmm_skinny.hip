@@ -90,9 +90,14 @@ __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a,
   const int64_t ng = (int64_t)(a.K / 64) >> GSHIFT;             // table entries per row
   const int slices = a.K / KS;
 
-  const int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
+  int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
-  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+  bool x_ok = true;
+  if (a.rhs_idx) {                                  // gather form: indices are data
+    if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
+    if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
+  }
+  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? (int64_t)a.M * a.K * 2 : 0);
   const auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
   const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * 2, a.N * ng * 2);
   const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * 2, a.N * ng * 2);
@@ -284,7 +289,7 @@ void launch_g(const GemvArgs& a, int64_t batch, int waves, int rows_per_wg, hipS
 }
 
 int env_int(const char* name) {
-  const char* e = getenv(name);
+  const char* e = experiment_env(name);
   return e ? atoi(e) : 0;
 }
 

@@ -197,6 +197,11 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 
   int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  bool x_ok = true;
+  if (a.rhs_idx) {                                  // gather form: indices are data
+    if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
+    if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
+  }
   // Rows of activations of this workgroup: a.M, or in the grouped form (direct
   // variants only) those of segment blockIdx.y.
   int M = a.M;
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   if (wave >= CW) {
     // ------------------------------------------------------------ loaders ----
     const int lw = wave - CW;
-    const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, (int64_t)a.M * a.K * 2);
+    const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? (int64_t)a.M * a.K * 2 : 0);
     const auto rw = make_rsrc(reinterpret_cast<const char*>(a.w) + wz * a.N * wpr, a.N * wpr);
     const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * ES, a.N * ng * ES);
     const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * ES, a.N * ng * ES);
@@ -435,7 +440,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
     const int tab_row = (wave >> 2) * (WIDE ? 2048 : 1024) + (wave & 3) * 256 + r * 16;   // this lane's table row inside a kind
     const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
-    const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, xrows * a.K * 2);
+    const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? xrows * a.K * 2 : 0);
     auto xrow = [&](int m) -> int64_t {
       if (m >= M) return -1;
       if (!src_row) return m;
@@ -746,13 +751,8 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (GSHIFT == 5 ? 2 : 1);
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
   const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
-  auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
-  static bool configured = false;                 // one flag per instantiation
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    configured = true;
-  }
+  constexpr auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
+  if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);
 }
 
@@ -792,7 +792,7 @@ int device_cus() {
 // where the ring variant (at most 64 rows a workgroup) would need a second
 // round of workgroups (28672 x 4096 at M = 16: 17 against 22 us).
 bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
-  static const char* const env = getenv("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
+  static const char* const env = experiment_env("QMM_SKINNY2_XD");   // 0 | 1 overrides the choice (experiments)
   static const int force = env ? atoi(env) : -1;
   if (force >= 0) return force != 0;
   const int64_t per = ceil_div(N, (int64_t)device_cus());
@@ -928,7 +928,7 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
 // MXFP4 decode on the direct variants: K a multiple of 512 with at least eight
 // slices, scale rows dword-aligned (they are fetched as 16-byte runs).
 bool skinny2_mx_supported(int64_t N, int64_t K, const void* s) {
-  static const bool off = getenv("QMM_NO_SKINNY_MX") != nullptr;
+  static const bool off = experiment_env("QMM_NO_SKINNY_MX") != nullptr;
   if (off || K % 512 || K / 512 < 8) return false;
   if (reinterpret_cast<uintptr_t>(s) & 3u) return false;
   return N * (K / 2) < 0x7FFFFFFFll;                          // 32-bit lane offsets

@@ -60,14 +60,18 @@ def pair_indices(indices):
     return tidx, eidx
 
 
-def emit_dot(x, arrays, mode, gs, bits, tidx, eidx, experts, out_dtype=None):
+def emit_dot(x, arrays, mode, gs, bits, tidx, eidx, experts, out_dtype=None, has_perm=False):
     """y[p] = x[tidx[p]] . dequant(W[eidx[p]])^T -> [P, N]
     (reference moe.py:1283-1340, the mx.gather_qmm call at :1320).
-    `arrays` are a pack's arrays (w, scales[, biases]) with the expert axis
-    leading; `x` is [T, K] (or [P, K] with tidx None)."""
+    `arrays` are a pack's arrays (w, scales[, biases][, perm]) with the expert
+    axis leading; `x` is [T, K] (or [P, K] with tidx None).  A pack built over
+    a permuted contraction axis carries the permutation last: the activations
+    are gathered through it first (reference moe.py:1316-1317)."""
     from . import kernels
     w, scales = arrays[0], arrays[1]
     biases = arrays[2] if mode == "affine" else None
+    if has_perm:
+        x = kernels.take_k(x, arrays[-1])
     w, scales = split_experts([w, scales], experts)
     if biases is not None:
         (biases,) = split_experts([biases], experts)
@@ -93,7 +97,8 @@ def expert_dispatch(interp, match, x, indices, weights):
     for d in match.bshape:
         experts *= d
     tidx, eidx = pair_indices(indices)
-    y = emit_dot(x, arrays, match.mode, match.gs, match.bits, tidx, eidx, experts)
+    y = emit_dot(x, arrays, match.mode, match.gs, match.bits, tidx, eidx, experts,
+                 out_dtype=qmm._torch_dtype(match.out_dtype), has_perm=match.has_perm)
     STATS["dispatches"] += 1
     return combine(y, weights)
 

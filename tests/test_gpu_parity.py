@@ -972,3 +972,171 @@ def test_gather_qmm_few_pairs_grouped_by_expert_mxfp4(k, pairs, e):
     y = out_f32(K.gather_qmm(xd, wd, sd, None, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
                              group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32))
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+@pytest.mark.parametrize("pairs,n,k,mode", [
+    (3, 2048, 4096, "affine"),      # below four pairs: independent products on the loader-wavefront kernel
+    (32, 2048, 4096, "affine"),     # no workspace: the same, 32 launches' worth of pairs
+    (32, 300, 1024, "affine"),      # two K-slices: the self-loading kernel
+    (32, 72, 96, "affine"),         # the general decode kernel
+    (32, 72, 256, "mxfp4"),         # the general MXFP4 decode kernel
+])
+def test_gather_qmm_independent_decode_products_check_their_indices(pairs, n, k, mode):
+    """Pairs that run as independent decode products (no expert sort): an
+    expert index outside [0, E) leaves the pair's output row as it was, a row
+    index outside [0, T) multiplies zeros -- what the sorted paths do."""
+    from metaljax_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(pairs + n + k)
+    e, t = 4, 6
+    if mode == "affine":
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 32 if k == 96 else 64, lead=(e,))
+        gs = 32 if k == 96 else 64
+    else:
+        _, words, s, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+        b, bd, gs = None, None, 32
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    lhs[1] = t                   # one past the last row
+    if pairs > 3:
+        lhs[7], rhs[5], rhs[9] = -1, e, -2
+    else:
+        rhs[2] = e + 5
+    y = torch.full((pairs, n), 7.0, dtype=torch.float32, device=DEV)
+    ld, rd = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    rc = lib.qmm_gather_qmm(xd.data_ptr(), _lib.BF16, wd.data_ptr(), sd.data_ptr(),
+                            None if bd is None else bd.data_ptr(), _lib.BF16, y.data_ptr(), _lib.F32,
+                            ld.data_ptr(), rd.data_ptr(), pairs, t, e, n, k, gs, 4,
+                            0 if mode == "affine" else 1, None, 0,
+                            torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc)
+    got = y.cpu().numpy()
+    for i in range(pairs):
+        if not 0 <= rhs[i] < e:
+            np.testing.assert_array_equal(got[i], np.full(n, 7.0, np.float32))
+        elif not 0 <= lhs[i] < t:
+            np.testing.assert_array_equal(got[i], np.zeros(n, np.float32))
+        else:
+            bi = None if b is None else b[rhs[i]]
+            want = O.qmm(x[lhs[i]][None], words[rhs[i]], s[rhs[i]], bi, gs, 4, mode)[0]
+            assert O.rel_l2(got[i], want) <= 2e-5, i
+
+
+# ------------------------------------- the named configurations at full size ----
+
+def _report(name, **figures):
+    """Measured distances of a full-size configuration, shown with `pytest -s`
+    / in the captured output of a failure, and kept for the session summary."""
+    line = name + ": " + ", ".join(f"{k} = {v:.3e}" for k, v in figures.items())
+    print(line)
+    FULL_SIZE_REPORT.append(line)
+
+
+FULL_SIZE_REPORT = []
+
+
+def test_c3_prefill_full_size_against_the_oracle():
+    """C3 whole (x [2048, 4096] x int8 g64 [4096, 4096]) against the C oracle:
+    float32 output against the bf16-rounded weight tile (the tile the kernel
+    stages is that rounding, so only accumulation order differs), bf16 output
+    against the exactly reconstructed weight at the 1e-2 bar; the float32
+    output's distance from the exact-weight product is measured and reported
+    (one bf16 rounding per weight: about 2^-9 / sqrt(3) = 1.1e-3)."""
+    wl = synth.make(3)
+    x, w, s, b, _ = synth.to_device(wl)
+    want_tile = C.qmm(wl.x, wl.w, wl.scales, wl.biases, 64, 8, "affine", round_tile_bf16=True)
+    want_exact = C.qmm(wl.x, wl.w, wl.scales, wl.biases, 64, 8, "affine", round_tile_bf16=False)
+    y32 = out_f32(K.quantized_matmul(x, w, s, b, group_size=64, bits=8, out_dtype=torch.float32))
+    y16 = out_f32(K.quantized_matmul(x, w, s, b, group_size=64, bits=8))
+    d_tile, d_exact, d16 = O.rel_l2(y32, want_tile), O.rel_l2(y32, want_exact), O.rel_l2(y16, want_exact)
+    _report("C3 full size", f32_vs_bf16_tile=d_tile, f32_vs_exact_weight=d_exact, bf16_vs_exact_weight=d16)
+    assert d_tile <= 2e-5
+    assert d_exact <= 3e-3
+    assert d16 <= TOL_BF16_OUT
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
+def test_c4_mxfp4_full_size_against_the_oracle():
+    """C4 whole (x [256, 8192] x MXFP4 [8192, 8192]) against the C oracle on the
+    exact weight (E2M1 x 2^e is exact in every float type)."""
+    wl = synth.make(4)
+    x, w, s, _, _ = synth.to_device(wl)
+    want = C.qmm(wl.x, wl.w, wl.scales, None, 32, 4, "mxfp4", round_tile_bf16=False)
+    y32 = out_f32(K.quantized_matmul(x, w, s, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    y16 = out_f32(K.quantized_matmul(x, w, s, None, group_size=32, bits=4, mode="mxfp4"))
+    d32, d16 = O.rel_l2(y32, want), O.rel_l2(y16, want)
+    _report("C4 full size", f32_vs_exact_weight=d32, bf16_vs_exact_weight=d16)
+    assert d32 <= TOL_F32_OUT
+    assert d16 <= TOL_BF16_OUT
+
+
+def test_c5_moe_full_size_against_the_oracle():
+    """C5 whole (1024 routed rows, 8 experts of int4 g64 [14336, 4096]): the
+    sorted-rows form in float32 and bf16, expert by expert, and the gathered
+    form on the unsorted (token, expert) pairs of the same routing."""
+    wl = synth.make(5)
+    x, w, s, b, ro = synth.to_device(wl)
+    ro_h = wl.row_offsets
+    assert wl.x.shape == (1024, 4096) and wl.w.shape == (8, 14336, 512)
+    want_tile = C.grouped_qmm(wl.x, wl.w, wl.scales, wl.biases, ro_h, 64, 4, "affine", round_tile_bf16=True)
+    want_exact = C.grouped_qmm(wl.x, wl.w, wl.scales, wl.biases, ro_h, 64, 4, "affine", round_tile_bf16=False)
+    y32 = out_f32(K.grouped_qmm(x, w, s, b, ro, group_size=64, bits=4, out_dtype=torch.float32))
+    y16 = out_f32(K.grouped_qmm(x, w, s, b, ro, group_size=64, bits=4))
+    for e in range(8):
+        lo, hi = ro_h[e], ro_h[e + 1]
+        assert hi > lo
+        assert O.rel_l2(y32[lo:hi], want_tile[lo:hi]) <= 2e-5, e
+        assert O.rel_l2(y16[lo:hi], want_exact[lo:hi]) <= TOL_BF16_OUT, e
+    _report("C5 full size", f32_vs_bf16_tile=O.rel_l2(y32, want_tile),
+            f32_vs_exact_weight=O.rel_l2(y32, want_exact), bf16_vs_exact_weight=O.rel_l2(y16, want_exact))
+    assert O.rel_l2(y32, want_exact) <= 3e-3
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+    # gathered form: pair p = 2 * token + j reads x_tokens[token] and expert experts[token, j];
+    # sorted row r holds pair pair_of_row[r]
+    ex = wl.extras
+    tokens = ex["tokens"]
+    xt = torch.from_numpy(ex["x_tokens"].view(np.int16)).to(DEV).view(torch.bfloat16)
+    lhs = torch.arange(tokens, dtype=torch.int32, device=DEV).repeat_interleave(2)
+    rhs = torch.from_numpy(ex["experts"].reshape(-1)).to(DEV)
+    yg = out_f32(K.gather_qmm(xt, w, s, b, lhs, rhs, group_size=64, bits=4, out_dtype=torch.float32))
+    assert yg.shape == (1024, 14336)
+    np.testing.assert_array_equal(yg[ex["pair_of_row"]], y32)       # row for row the same arithmetic
+    assert O.rel_l2(yg[ex["pair_of_row"]], want_tile) <= 2e-5
+
+
+@pytest.mark.parametrize("bits,gs,k,mode", [
+    (4, 64, 4352, "affine"),     # 68 entries a row: 136 bytes
+    (4, 32, 2304, "affine"),     # 72 entries
+    (8, 64, 4352, "affine"),
+    (8, 32, 2304, "affine"),
+    (4, 32, 4352, "mxfp4"),      # 136 scale bytes a row, K % 512 != 0: the bf16 kernels
+])
+def test_grouped_qmm_short_experts_with_table_rows_longer_than_a_cache_line(bits, gs, k, mode):
+    """The split-role kernel stages a tile's scale / bias rows in LDS only when
+    a row's table fits one 128-byte line; longer rows (these) take the 16-byte
+    windows per quad of K-tiles instead."""
+    rng = np.random.default_rng(bits * 1000 + gs + k)
+    sizes = np.array([130, 0, 96, 161, 17])
+    e, n = len(sizes), 136
+    if mode == "affine":
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, lead=(e,))
+    else:
+        _, words, s, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+        b, bd = None, None
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    assert r // e <= 144 and k % 256 == 0
+    x, xd = make_x(rng, r, k)
+    want = O.grouped_qmm(x, words, s, b, ro, gs, bits, mode, weight_rounding="bf16")
+    ro_d = torch.from_numpy(ro).to(DEV)
+    y32 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=gs, bits=bits, mode=mode,
+                                out_dtype=torch.float32))
+    y16 = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=gs, bits=bits, mode=mode))
+    for i in range(e):
+        lo, hi = ro[i], ro[i + 1]
+        if hi > lo:
+            assert O.rel_l2(y32[lo:hi], want[lo:hi]) <= 2e-5, (i, O.rel_l2(y32[lo:hi], want[lo:hi]))
+            assert O.rel_l2(y16[lo:hi], want[lo:hi]) <= TOL_BF16_OUT, i
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
