@@ -22,7 +22,10 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
 
 def _compile(src: str) -> str:
     obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + ".o")
-    cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    # QMM_EXPERIMENTS=1: a measuring build whose kernel choice can be overridden
+    # through QMM_* environment switches; the normal build reads no environment
+    extra = ["-DQMM_EXPERIMENTS"] if os.environ.get("QMM_EXPERIMENTS") == "1" else []
+    cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode:

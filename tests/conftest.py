@@ -27,3 +27,14 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The distances the full-size configuration tests measured (they are
+    captured output otherwise)."""
+    mod = sys.modules.get("tests.test_gpu_parity") or sys.modules.get("test_gpu_parity")
+    lines = getattr(mod, "FULL_SIZE_REPORT", None) if mod else None
+    if lines:
+        terminalreporter.write_sep("-", "full-size configurations: measured rel-L2")
+        for line in lines:
+            terminalreporter.write_line(line)
