@@ -95,6 +95,25 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
                    int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* qmm_gather_qmm for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  Same arguments and results as
+ * qmm_gather_qmm without the workspace pair: the expert sort's arrays, the
+ * segment list and the re-laid activation copy live in a device array of
+ * QMM_STATIC_SCRATCH_BYTES that is part of the library's code object (every
+ * GPU the library runs on holds one until the process ends).  A call whose
+ * qmm_gather_workspace_bytes(P, E, N, K) exceeds that size fails with
+ * QMM_ERR_WORKSPACE and launches nothing.  The call allocates and frees
+ * nothing.  Every call on a GPU uses that GPU's one array: calls that overlap
+ * on one GPU (different streams, or threads) race; calls in stream order do
+ * not, and each call initialises what it reads. */
+#define QMM_STATIC_SCRATCH_BYTES (16u << 20)
+int qmm_gather_qmm_static(const void* x, int x_dtype, const void* w, const void* scales,
+                          const void* biases, int table_dtype, void* y, int y_dtype,
+                          const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
+                          int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
+                          void* stream);
+
 /* The sorted-rows form of the same product (rows of x already grouped by
  * expert): rows [row_offsets[e], row_offsets[e+1]) use expert e's weight.
  * row_offsets int32 [E+1] on the device, non-decreasing, row_offsets[0] = 0,

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libqmm_hip.so")
 QMM_OK = 0
 ERR_NAMES = {1: "BAD_ARGUMENT", 2: "BAD_SHAPE", 3: "UNSUPPORTED", 4: "WORKSPACE", 5: "HIP"}
 F32, BF16, F16 = 0, 1, 2
+STATIC_SCRATCH_BYTES = 16 << 20      # QMM_STATIC_SCRATCH_BYTES of include/qmm_hip.h
 MODE_AFFINE, MODE_MXFP4 = 0, 1
 KERNEL_GEMV, KERNEL_GEMM, KERNEL_MXFP4_MFMA = 1, 2, 3
 
@@ -23,7 +24,7 @@ KERNEL_GEMV, KERNEL_GEMM, KERNEL_MXFP4_MFMA = 1, 2, 3
 SYMBOLS = (
     "qmm_abi_version", "qmm_last_error", "qmm_quantized_matmul", "qmm_workspace_bytes",
     "qmm_gather_workspace_bytes", "qmm_plan", "qmm_gather_qmm", "qmm_grouped_qmm",
-    "qmm_dequantize", "qmm_unpack_codes", "qmm_pack_codes", "qmm_take_k",
+    "qmm_gather_qmm_static", "qmm_dequantize", "qmm_unpack_codes", "qmm_pack_codes", "qmm_take_k",
 )
 
 
@@ -70,6 +71,8 @@ def load():
     lib.qmm_plan.argtypes = [i64, i64, i64, ci, ci, ci, ip, ip, ip]
     lib.qmm_gather_qmm.argtypes = [vp, ci, vp, vp, vp, ci, vp, ci, vp, vp, i64, i64, i64, i64,
                                    i64, ci, ci, ci, vp, sz, vp]
+    lib.qmm_gather_qmm_static.argtypes = [vp, ci, vp, vp, vp, ci, vp, ci, vp, vp, i64, i64, i64,
+                                          i64, i64, ci, ci, ci, vp]
     lib.qmm_grouped_qmm.argtypes = [vp, ci, vp, vp, vp, ci, vp, ci, vp, i64, i64, i64, i64, ci,
                                     ci, ci, vp, sz, vp]
     lib.qmm_dequantize.argtypes = [vp, vp, vp, ci, vp, ci, i64, i64, ci, ci, ci, vp]

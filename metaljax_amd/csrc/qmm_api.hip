@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 
 #include "qmm_common.hpp"
 
@@ -191,6 +192,34 @@ bool grouped_decode_pairs(int64_t P, int64_t E) {
   static const int64_t gd_max = experiment_env("QMM_GD_MAX") ? atoll(experiment_env("QMM_GD_MAX")) : 0;
   if (P < kGroupedDecodeMinPairs) return false;
   return gd_max ? P <= gd_max : P <= 16 * E && P <= 4096;
+}
+
+// ---- scratch of the allocation-free entry point ------------------------------
+// Part of the code object: each GPU that loads the library holds its own copy
+// at its own address.  In host code the name is only a handle for
+// hipGetSymbolAddress; the address it yields is what kernels are given.
+__device__ __align__(256) unsigned char scratch[QMM_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// The current device's scratch address (looked up once per device).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(QMM_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(QMM_ERR_HIP, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(QMM_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return QMM_OK;
 }
 
 }  // namespace
@@ -440,6 +469,29 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   gemm_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
                 group_size, bits, mode, st);
   return check_launch("gather gemm launch");
+}
+
+int qmm_gather_qmm_static(const void* x, int x_dtype, const void* w, const void* scales,
+                          const void* biases, int table_dtype, void* y, int y_dtype,
+                          const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
+                          int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
+                          void* stream) {
+  if (P < 0 || T < 0 || E < 0 || N < 0 || K < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
+  const size_t need = qmm_gather_workspace_bytes(P, E, N, K);
+  if (need > (size_t)QMM_STATIC_SCRATCH_BYTES)
+    return fail(QMM_ERR_WORKSPACE,
+                "gather_qmm_static: %lld pairs over %lld experts of [%lld, %lld] need %zu scratch "
+                "bytes, the static scratch holds %zu (use qmm_gather_qmm with a workspace)",
+                (long long)P, (long long)E, (long long)N, (long long)K, need,
+                (size_t)QMM_STATIC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  if (need) {
+    const int rc = static_scratch(&ptr);
+    if (rc) return rc;
+  }
+  return qmm_gather_qmm(x, x_dtype, w, scales, biases, table_dtype, y, y_dtype, lhs_idx, rhs_idx, P,
+                        T, E, N, K, group_size, bits, mode, ptr, need ? (size_t)QMM_STATIC_SCRATCH_BYTES : 0,
+                        stream);
 }
 
 int qmm_dequantize(const void* w, const void* scales, const void* biases, int table_dtype,

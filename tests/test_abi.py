@@ -46,6 +46,10 @@ def test_header_cites_the_reference_for_every_entry_point():
         if name in ("qmm_abi_version", "qmm_last_error", "qmm_workspace_bytes",
                     "qmm_gather_workspace_bytes", "qmm_plan"):
             continue
+        if name == "qmm_gather_qmm_static":      # says that the reference has no such call
+            head = text[:text.index(name + "(")]
+            assert "No counterpart in the reference" in head[head.rindex("/*"):]
+            continue
         head = text[:text.index(name + "(")]
         comment = head[head.rindex("/*"):]
         assert re.search(r"\.py:\d+", comment), f"{name}: no reference citation"
@@ -115,3 +119,16 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libqmm_hip.so"))
     with pytest.raises(_lib.QmmLibraryError):
         _lib.load()
+
+
+def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):
+    """qmm_gather_qmm_static refuses, on the host and before any device work,
+    a product whose scratch need exceeds the array built into the library."""
+    text = open(HEADER).read()
+    assert re.search(r"#define QMM_STATIC_SCRATCH_BYTES \(16u << 20\)", text)
+    assert _lib.STATIC_SCRATCH_BYTES == 16 << 20
+    p, e, n, k = 4096, 8, 14336, 4096                 # the re-laid activations alone are 32 MiB
+    assert lib.qmm_gather_workspace_bytes(p, e, n, k) > _lib.STATIC_SCRATCH_BYTES
+    rc = lib.qmm_gather_qmm_static(None, _lib.BF16, None, None, None, _lib.BF16, None, _lib.BF16,
+                                   None, None, p, p, e, n, k, 64, 4, 0, None)
+    assert rc == 4 and b"static scratch" in lib.qmm_last_error()

@@ -1,0 +1,105 @@
+"""qmm_gather_qmm_static (the entry point that allocates nothing: its scratch
+is a device array inside the library) against qmm_gather_qmm with a caller's
+workspace, through the C ABI: the same kernels on the same inputs, so the
+outputs are compared bit for bit, and against the oracle.  Calls run back to
+back on one stream, a larger product first and smaller ones after it, so a
+later call meets the earlier one's leftovers in the scratch."""
+
+import numpy as np
+import pytest
+import torch
+
+from metaljax_amd import _lib
+from oracle import qmm_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _bf16(a):
+    return torch.from_numpy(O.f32_to_bf16_bits(a).view(np.int16)).to(DEV).view(torch.bfloat16)
+
+
+def _case(rng, e, n, k, t, pairs, mode):
+    codes = rng.integers(0, 16, size=(e, n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, 4)
+    if mode == "affine":
+        s = O.round_bf16(rng.uniform(0.005, 0.02, (e, n, k // 64)).astype(np.float32))
+        b = O.round_bf16(-8 * s)
+        sd, bd, gs = _bf16(s), _bf16(b), 64
+    else:
+        s = rng.integers(120, 131, size=(e, n, k // 32)).astype(np.uint8)
+        b, sd, bd, gs = None, torch.from_numpy(s).to(DEV), None, 32
+    x = O.round_bf16(rng.standard_normal((t, k)).astype(np.float32))
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    dev = dict(x=_bf16(x), w=torch.from_numpy(words.view(np.int32)).to(DEV), s=sd, b=bd,
+               lhs=torch.from_numpy(lhs).to(DEV), rhs=torch.from_numpy(rhs).to(DEV))
+    return dict(e=e, n=n, k=k, t=t, p=pairs, mode=mode, gs=gs, x=x, words=words, s=s, b=b,
+                lhs=lhs, rhs=rhs, dev=dev)
+
+
+def _call(lib, c, static, y_dtype=torch.float32):
+    d = c["dev"]
+    y = torch.full((c["p"], c["n"]), 3.0, dtype=y_dtype, device=DEV)
+    yd = _lib.F32 if y_dtype == torch.float32 else _lib.BF16
+    head = (d["x"].data_ptr(), _lib.BF16, d["w"].data_ptr(), d["s"].data_ptr(),
+            None if d["b"] is None else d["b"].data_ptr(), _lib.BF16, y.data_ptr(), yd,
+            d["lhs"].data_ptr(), d["rhs"].data_ptr(), c["p"], c["t"], c["e"], c["n"], c["k"],
+            c["gs"], 4, 0 if c["mode"] == "affine" else 1)
+    st = torch.cuda.current_stream().cuda_stream
+    if static:
+        rc = lib.qmm_gather_qmm_static(*head, st)
+    else:
+        nbytes = int(lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"]))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=DEV)
+        rc = lib.qmm_gather_qmm(*head, ws.data_ptr() if nbytes else None, nbytes, st)
+    _lib.check(rc)
+    return y
+
+
+def test_static_scratch_calls_match_the_workspace_entry_point_call_after_call():
+    lib = _lib.load()
+    rng = np.random.default_rng(2024)
+    cases = [
+        _case(rng, 6, 200, 512, 400, 800, "affine"),      # prefill kernels: sort + re-laid activations
+        _case(rng, 6, 200, 512, 90, 150, "affine"),       # the same path, smaller, over the leftovers
+        _case(rng, 4, 2100, 4096, 9, 24, "affine"),       # grouped decode: sort + segment list
+        _case(rng, 4, 2100, 4096, 5, 8, "affine"),        # smaller again
+        _case(rng, 3, 136, 1024, 100, 300, "mxfp4"),      # block-scaled matrix cores: split activations
+        _case(rng, 4, 200, 512, 2, 3, "affine"),          # below four pairs: no scratch at all
+    ]
+    allocated = None
+    for i, c in enumerate(cases):
+        print("case", i, c["mode"], c["p"], "pairs", flush=True)
+        want = _call(lib, c, static=False)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        got = _call(lib, c, static=True)
+        got16 = _call(lib, c, static=True, y_dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), i
+        assert torch.equal(got16, want.to(torch.bfloat16)), i
+        rounding = "bf16" if (c["p"] > 64 and c["mode"] == "affine") else "f32"
+        ref = O.gather_qmm(c["x"][:, None, :], c["words"], c["s"], c["b"], c["lhs"], c["rhs"],
+                           c["gs"], 4, c["mode"], weight_rounding=rounding)[:, 0]
+        tol = 1e-3 if (c["mode"] == "mxfp4" and c["p"] > 64) else 2e-5
+        assert O.rel_l2(got.cpu().numpy(), ref) <= tol, i
+        # torch's allocator saw only the two outputs
+        allocated = torch.cuda.memory_allocated() - before
+        assert allocated <= 2 * (got.numel() * 4 + got16.numel() * 2) + (1 << 20)
+
+
+def test_static_scratch_limit_is_an_error_and_launches_nothing():
+    lib = _lib.load()
+    rng = np.random.default_rng(7)
+    c = _case(rng, 2, 64, 8192, 8, 1100, "affine")       # 1100 pairs x K = 8192: the re-laid copy alone is 21 MiB
+    assert lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"]) > _lib.STATIC_SCRATCH_BYTES
+    with pytest.raises(_lib.QmmError) as err:
+        _call(lib, c, static=True)
+    assert err.value.code == 4 and "static scratch" in str(err.value)
+    # the workspace form serves the same call
+    y = _call(lib, c, static=False)
+    ref = O.gather_qmm(c["x"][:, None, :], c["words"], c["s"], c["b"], c["lhs"], c["rhs"], 64, 4,
+                       weight_rounding="bf16")[:, 0]
+    assert O.rel_l2(y.cpu().numpy(), ref) <= 2e-5
