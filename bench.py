@@ -199,6 +199,9 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a 64 MiB read + 64 MiB write elementwise kernel five times, "
                          "for scaling FETCH_SIZE / WRITE_SIZE counter readings")
+    ap.add_argument("--probe", action="store_true",
+                    help="time read-only and empty launches instead (what one launch over the "
+                         "headline's bytes can reach on this GPU whatever its arithmetic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU; --gpus {args.gpus} is not supported "
@@ -216,6 +219,10 @@ def main():
         for _ in range(5):
             torch.bitwise_not(src, out=dst)
         torch.cuda.synchronize()
+    if args.probe:
+        from metaljax_amd import profiling
+        print(json.dumps({"probe": profiling.stream_probe()}))
+        return 0
     if args.shape:
         print(json.dumps({args.shape: bench_once(int(args.shape[1]))}))
         return 0

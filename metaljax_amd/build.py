@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libqmm_hip.so")
-SOURCES = ["qmm_api.hip", "qmm_gemv.hip", "qmm_skinny.hip", "qmm_skinny2.hip", "qmm_gemm.hip", "qmm_gemm2.hip", "qmm_gemm2s.hip", "qmm_mxfp4.hip", "qmm_util.hip"]
+SOURCES = ["qmm_api.hip", "qmm_gemv.hip", "qmm_skinny.hip", "qmm_skinny2.hip", "qmm_skinny3.hip", "qmm_gemm.hip", "qmm_gemm2.hip", "qmm_gemm2s.hip", "qmm_mxfp4.hip", "qmm_util.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wno-unused-function"]
@@ -47,7 +47,23 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    build_probe(verbose)
     return LIB
+
+
+PROBE_LIB = os.path.join(LIBDIR, "libqmm_probe.so")
+
+
+def build_probe(verbose: bool = False) -> str:
+    """The measuring kernels of `bench.py --probe` (read-only and empty
+    launches), a library of their own: not part of the quantized-matmul ABI."""
+    cmd = ["hipcc", *FLAGS, "-shared", os.path.join(CSRC, "probe_stream.hip"), "-o", PROBE_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode:
+        raise RuntimeError(f"hipcc failed on probe_stream.hip:\n{r.stderr}")
+    if verbose:
+        print(f"built {PROBE_LIB}")
+    return PROBE_LIB
 
 
 if __name__ == "__main__":

@@ -635,11 +635,66 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           if (active) chunk_sums();
         }
       };
+      // More than eight rows of activations: the direct load above makes every
+      // lane a cache-line request of its own (sixteen rows a quarter line each
+      // per instruction), which at sixteen rows costs more than it saves.
+      // Here the slice comes in with whole-line loads instead -- instruction
+      // (c, h) fetches the 128 bytes of chunk c of rows 8h .. 8h+7 -- all of
+      // them requested at once, and each chunk takes a round trip through a
+      // 2 KB wave-private LDS patch into operand order (piece p of row r at
+      // position p ^ ((r >> 1) & 7): both the 16-lane write and read passes
+      // touch every bank once).
+      auto fetch_x_staged = [&](int p, bool active) __attribute__((always_inline)) {
+        unsigned char* stg = smem + 4 * (kItem + kTab) + wave * 2048;
+        const int srow = lane >> 3, sp = lane & 7;
+        u32x4 raw[CPS][2];
+        uint32_t lo[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int64_t xr = active ? xrow(8 * h + srow) : -1;
+          lo[h] = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)sp * 16u : kOutOfRange;
+        }
+        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
+#pragma unroll
+        for (int c = 0; c < CPS; ++c)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo[h], so + (uint32_t)(c * 128), 0);
+        const uint32_t wr0 = (uint32_t)(srow * 128 + ((sp ^ ((srow >> 1) & 7)) << 4));          // rows 0-7
+        const uint32_t wr1 = (uint32_t)((srow + 8) * 128 + ((sp ^ (((srow + 8) >> 1) & 7)) << 4));
+        const uint32_t rkey = (uint32_t)((r >> 1) & 7);
+#pragma unroll
+        for (int c = 0; c < CPS; ++c) {
+          *reinterpret_cast<u32x4*>(stg + wr0) = raw[c][0];
+          *reinterpret_cast<u32x4*>(stg + wr1) = raw[c][1];
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const uint32_t pc = (uint32_t)(kg * 2 + j);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + r * 128 + ((pc ^ rkey) << 4));
+            if constexpr (BITS == 4 && !MX) xa[c][j] = pair_stride4(v);
+            else xa[c][j] = __builtin_bit_cast(bf16x8, v);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        if constexpr (!MX) {
+          if (active) chunk_sums();
+        }
+      };
       if constexpr (XD == 1) {
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
         const bool active = wave < slices;        // uniform
-        fetch_x(0, active, xlane);
+        if constexpr (!WIDE) {                    // (wide table rows leave no LDS for the staging patches)
+          if (M > 8) fetch_x_staged(0, active);
+          else fetch_x(0, active, xlane);
+        } else {
+          fetch_x(0, active, xlane);
+        }
 #pragma nounroll
         for (int g = 0; g < ntiles; ++g) {
           item_barrier();
@@ -750,7 +805,9 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
   constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (GSHIFT == 5 ? 2 : 1);
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
-  const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind);
+  // (one-pass direct variant: plus a 2 KB patch a compute wavefront for staging activations)
+  const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind) +
+                     (XD == 1 && GSHIFT != 5 ? (size_t)CW * 2048 : 0);
   constexpr auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);
@@ -796,7 +853,12 @@ bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   static const int force = env ? atoi(env) : -1;
   if (force >= 0) return force != 0;
   const int64_t per = ceil_div(N, (int64_t)device_cus());
-  if (M > 8 && per <= 64) return false;
+  // More than eight rows of activations on a weight of at most 64 rows per
+  // compute unit: with one pass over K the direct variant stages the
+  // activations through LDS patches (whole-line loads) and is ahead of the
+  // ring (4096 x 14336 at M = 16: 12.1 against 12.9 us a launch, 4096 x 4096:
+  // 6.5 against 7.6); with several passes the ring variant stays.
+  if (M > 8 && per <= 64 && K * bits / 8 / 256 != 8) return false;
   // Several passes over K: the next pass's activations are fetched when the
   // pass begins, which costs about 0.8 us a pass; measured against the other
   // kernels at M = 4 (us): 28672 x 8192 30.8 / 38.4, 57344 x 8192 61 / 79,
@@ -855,7 +917,10 @@ void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int r
                       int tab, bool force_direct) {
   GemvArgs a = a0;
   a.gshift = (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : tab == QMM_F32 ? 5 : 0);
-  const bool xd = force_direct || direct_x(a.M, a.N, a.K, bits);
+  bool xd = force_direct || direct_x(a.M, a.N, a.K, bits);
+  // float32 tables with groups of 64 fill the LDS with table rows: no room for
+  // the staging patches, and direct loads of more than eight rows lose to the ring
+  if (xd && !force_direct && a.M > 8 && rows <= 64 && tab == QMM_F32 && gs == 64) xd = false;
   if (xd) {                                       // up to eight tiles' sums in registers over several passes
     const bool one_pass = a.K * bits / 8 / 256 <= 8;
     if (one_pass) {

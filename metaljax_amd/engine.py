@@ -4,10 +4,23 @@ execute it on buffers (reference src/metaljax/engine.py:325, :385).
 Only what the quantized-matmul path needs is here: `compile_program` parses
 the module text, `execute` runs the packing prologue and then the program.
 The PJRT plugin, buffer donation/aliasing and the trace cache of the reference
-engine are outside this package; the entry points a PJRT plugin calls by name
-(`buffer_from_host`, `buffer_to_host`, `buffer_pointer`, `device_kind`,
-`stablehlo_version`; reference src/metaljax/engine.py:133-159, :549-591) are
-kept as a thin surface over host arrays and device tensors.
+engine are outside this package.  What the plugin calls by name keeps its name,
+argument meaning and result type (reference plugin/metal_pjrt.cc):
+
+    compile_program(code, fmt, options) -> object with name, fingerprint,
+        num_outputs, num_params, out_types (PJRT_Buffer_Type integers),
+        out_dims, donated_params                       metal_pjrt.cc:547-580
+    execute(executable, [buffer]) -> [buffer]; a buffer has data, type_enum,
+        dims, nbytes                                   metal_pjrt.cc:284-299, :990-1010
+    buffer_from_host(memoryview, type_enum, dims, byte_strides, offset)
+                                                       metal_pjrt.cc:662-664
+    to_host(buffer) -> bytes                           metal_pjrt.cc:1168-1172
+    buffer_pointer(buffer) -> int                      metal_pjrt.cc:1125
+    device_kind() -> str, stablehlo_version() -> [int] metal_pjrt.cc:382, :440
+
+The reference's executables also carry `forwarded_outputs`-style donation
+plumbing inside `execute`; here `donated_params` is reported and donation is
+not acted on (every output is a fresh buffer).
 """
 
 from __future__ import annotations
@@ -77,13 +90,24 @@ def buffer_from_host(data, type_enum: int, dims, byte_strides=None, offset: int 
     return Buffer(from_numpy(arr, el), type_enum, dims)
 
 
-def buffer_to_host(buf) -> bytes:
-    """The bytes of a Buffer (or of any runtime value) in its element type."""
+def to_host(buf) -> bytes:
+    """The bytes of a Buffer (or of any runtime value) in its element type,
+    row-major (reference engine.py:154-159; what the plugin's ToHostBuffer
+    copies out, metal_pjrt.cc:1168-1172)."""
     h = host(buf.data if isinstance(buf, Buffer) else buf)
     if h.el == "bf16":
         from .packing import f32_to_bf16_bits
         return f32_to_bf16_bits(np.ascontiguousarray(h.a, np.float32)).tobytes()
     return np.ascontiguousarray(h.a).tobytes()
+
+
+buffer_to_host = to_host        # the name earlier callers of this package used
+
+
+def to_numpy(buf):
+    """A result as (numpy array, element type); bf16 comes back as float32 values."""
+    h = host(buf.data if isinstance(buf, Buffer) else buf)
+    return h.a, h.el
 
 
 def buffer_pointer(buf) -> int:
@@ -118,8 +142,9 @@ class Executable:
         self.fingerprint = fingerprint
         self.num_params = len(interp.main.body.args)
         self.num_outputs = len(interp.main.result_types)
-        self.out_types = [t.el for t in interp.main.result_types]
-        self.out_type_enums = [_EL_ENUM.get(t.el, 0) for t in interp.main.result_types]
+        # PJRT_Buffer_Type integers, as the plugin reads them (metal_pjrt.cc:558)
+        self.out_types = [_EL_ENUM.get(t.el, 0) for t in interp.main.result_types]
+        self.out_els = [t.el for t in interp.main.result_types]
         self.out_dims = [list(t.shape) for t in interp.main.result_types]
         self.donated_params = sorted(interp.donated_args)
         self.generation = 0                 # bumped whenever the rewrite set changes
@@ -146,10 +171,8 @@ def execute(ex: Executable, buffers):
     if qmm.ENABLED:
         if qmm.prologue(ex.interp, args):
             ex.invalidate_traces()
-    return ex.interp.run(args)
-
-
-def to_host(buf):
-    """A result as (numpy array, element type); bf16 comes back as float32 values."""
-    h = host(buf)
-    return h.a, h.el
+    outs = ex.interp.run(args)
+    # every output as a buffer object (data, type_enum, dims, nbytes), which is
+    # what the plugin wraps (metal_pjrt.cc:990-1010); `data` is a device tensor
+    # for a fused dot's result, a host array otherwise
+    return [Buffer(v, t, d) for v, t, d in zip(outs, ex.out_types, ex.out_dims)]

@@ -107,6 +107,8 @@ def host(v) -> HostArray:
     """Any runtime value as a HostArray (device tensors are copied back)."""
     if isinstance(v, HostArray):
         return v
+    if hasattr(v, "type_enum") and hasattr(v, "data"):      # an engine buffer
+        return host(v.data)
     import torch
     if isinstance(v, torch.Tensor):
         if v.dtype == torch.bfloat16:

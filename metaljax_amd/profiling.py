@@ -48,6 +48,67 @@ def _short(name: str) -> str:
     return name.split("(")[0][:64]
 
 
+def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
+    """What a single launch reaches on this GPU whatever its arithmetic: the
+    per-launch time (HIP events around a graph replay, like the benchmark's
+    decode leg) of read-only launches over `nbytes` in several geometries, each
+    cycling through distinct buffers of more than twice the last-level cache
+    so that every launch streams from HBM, and of empty launches of the decode
+    kernel's geometry.  Returns a dict of results."""
+    import ctypes
+    import os
+
+    import torch
+    here = os.path.dirname(os.path.abspath(__file__))
+    lib = ctypes.CDLL(os.path.join(here, "lib", "libqmm_probe.so"))
+    vp, ci, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+    lib.probe_read.argtypes = [vp, i64, vp, ci, ci, ci, ci, vp]
+    lib.probe_empty.argtypes = [vp, ci, ci, ci, vp]
+    n_sets = (2 * (256 << 20)) // nbytes + 1
+    bufs = [torch.randint(-2**31, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda")
+            for _ in range(n_sets)]
+    sink = torch.zeros(4096, dtype=torch.int32, device="cuda")
+
+    def timed(launch):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            st = stream.cuda_stream
+            for i in range(n_sets):
+                launch(i, st)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for i in range(n_sets):
+                    launch(i, st)
+            g.replay()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n = max(1, reps // n_sets)
+            a.record(stream)
+            for _ in range(n):
+                g.replay()
+            b.record(stream)
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) * 1e3 / (n * n_sets)
+
+    out = {"bytes": nbytes, "buffers": n_sets, "read": {}, "empty": {}}
+    for blocks, threads, unroll, lds in ((256, 1024, 8, 0), (256, 768, 8, 0), (256, 768, 8, 147456),
+                                         (512, 512, 8, 0), (1024, 256, 8, 0), (2048, 256, 4, 0),
+                                         (4096, 256, 2, 0), (8192, 256, 1, 0)):
+        def launch(i, st, b=blocks, t=threads, u=unroll, l=lds):
+            rc = lib.probe_read(bufs[i].data_ptr(), nbytes, sink.data_ptr(), b, t, u, l, st)
+            assert rc == 0, rc
+        us = timed(launch)
+        out["read"][f"{blocks}x{threads} unroll {unroll} lds {lds}"] = {
+            "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1)}
+    for blocks, threads, lds in ((256, 768, 147456), (256, 768, 0), (256, 256, 0)):
+        def launch(i, st, b=blocks, t=threads, l=lds):
+            rc = lib.probe_empty(sink.data_ptr(), b, t, l, st)
+            assert rc == 0, rc
+        out["empty"][f"{blocks}x{threads} lds {lds}"] = {"us": round(timed(launch), 2)}
+    return out
+
+
 def main(argv):
     path = argv[1]
     total = sum(r[7] for r in kernel_stats(path)) or 1

@@ -27,7 +27,8 @@ def compare(text, args, exact, packs=1):
     lit = I.Interpreter(text)
     want = I.host(lit.run(args)[0]).a.astype(np.float32)
     ex = engine.compile_program(text)
-    (y,) = engine.execute(ex, args)
+    (buf,) = engine.execute(ex, args)
+    y = buf.data
     assert isinstance(y, torch.Tensor) and y.is_cuda          # the fused op ran on the device
     got = y.float().cpu().numpy()
     assert qmm.stats()["packs"] == packs and qmm.stats()["fallbacks"] == 0

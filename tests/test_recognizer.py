@@ -402,37 +402,58 @@ def test_emit_fails_loudly_without_a_gpu():
 
 # ------------------------------------------------------- engine surface ----
 
-def test_engine_surface_names_a_pjrt_plugin_calls():
-    """compile_program / execute / buffer_from_host / buffer_to_host /
-    buffer_pointer / device_kind / stablehlo_version and the executable's
-    attributes (reference src/metaljax/engine.py:133-175, :549-591)."""
+def test_engine_surface_is_what_the_pjrt_plugin_calls_by_name():
+    """Names, argument meaning and result types as the reference's plugin uses
+    them: compile_program(code, fmt, options) -> object whose name /
+    fingerprint are str, num_outputs / num_params ints, out_types a list of
+    PJRT_Buffer_Type integers, out_dims a list of int lists, donated_params a
+    list of ints (plugin/metal_pjrt.cc:547-580); execute(exec, [buffer]) -> a
+    list of num_outputs objects with data, type_enum, dims, nbytes (:284-299,
+    :990-1010); buffer_from_host(memoryview, type_enum, dims, byte_strides,
+    offset) (:662-664); buffer_pointer(buffer) -> int (:1125); to_host(buffer)
+    -> bytes of nbytes length (:1168-1172); device_kind() -> str,
+    stablehlo_version() -> ints (:382, :440)."""
     import numpy as np
     from metaljax_amd import engine
     text = T.float_dot(8, 16, 4, el="f32")          # y = x @ (w * r[:, None]): w [8,16], r [8], x [4,8]
     ex = engine.compile_program(text.encode(), "mlir", None)
-    assert ex.name == "main" and len(ex.fingerprint) == 64
-    assert ex.num_params == 3 and ex.num_outputs == 1
+    assert isinstance(ex.name, str) and ex.name == "main"
+    assert isinstance(ex.fingerprint, str) and len(ex.fingerprint) == 64
+    assert (ex.num_params, ex.num_outputs) == (3, 1)
+    f32 = engine.PJRT_TYPES.index("F32")
+    assert f32 == 11 and engine.PJRT_TYPES.index("BF16") == 13       # PJRT_Buffer_Type values of the C API
+    assert ex.out_types == [f32] and all(type(t) is int for t in ex.out_types)
     assert ex.out_dims == [[4, 16]] and ex.donated_params == []
-    assert ex.out_type_enums == [engine.PJRT_TYPES.index("F32")]
     rng = np.random.default_rng(0)
     w = rng.standard_normal((8, 16)).astype(np.float32)
     r = rng.standard_normal((8,)).astype(np.float32)
     x = rng.standard_normal((4, 8)).astype(np.float32)
-    f32 = engine.PJRT_TYPES.index("F32")
     # a transposed host view arrives with strides
     wt = np.ascontiguousarray(w.T)
     bw = engine.buffer_from_host(memoryview(wt), f32, [8, 16], [4, 4 * 8], 0)
-    br = engine.buffer_from_host(memoryview(r), f32, [8], None)
-    bx = engine.buffer_from_host(memoryview(x), f32, [4, 8], None)
+    br = engine.buffer_from_host(memoryview(r), f32, [8], None, 0)
+    bx = engine.buffer_from_host(memoryview(x), f32, [4, 8], None, 0)
     assert bx.nbytes == x.nbytes and bx.dims == [4, 8] and bx.type_enum == f32
-    assert engine.buffer_pointer(bx) != 0
-    (y,) = engine.execute(ex, [bw, br, bx])
-    got = np.frombuffer(engine.buffer_to_host(y), np.float32).reshape(4, 16)
+    ptr = engine.buffer_pointer(bx)
+    assert type(ptr) is int and ptr != 0
+    outs = engine.execute(ex, [bw, br, bx])
+    assert isinstance(outs, list) and len(outs) == ex.num_outputs
+    y = outs[0]
+    assert y.type_enum == f32 and y.dims == [4, 16] and y.nbytes == 4 * 16 * 4
+    assert hasattr(y, "data")
+    raw = engine.to_host(y)
+    assert type(raw) is bytes and len(raw) == y.nbytes
+    got = np.frombuffer(raw, np.float32).reshape(4, 16)
     np.testing.assert_allclose(got, x @ (w * r[:, None]), rtol=1e-5, atol=1e-5)
+    # an output buffer is a valid input of the next execute
+    (y2,) = engine.execute(ex, [bw, br, bx])
+    assert engine.to_host(y2) == raw
     # bf16 bytes round-trip as 16-bit patterns
     bits = np.array([0x3F80, 0xC000, 0x0000], np.uint16)
-    bf = engine.buffer_from_host(memoryview(bits), engine.PJRT_TYPES.index("BF16"), [3], None)
-    assert engine.buffer_to_host(bf) == bits.tobytes()
-    with pytest.raises(TypeError, match="Unsupported"):
-        engine.buffer_from_host(None, engine.PJRT_TYPES.index("C64"), [1], None)
-    assert isinstance(engine.device_kind(), str) and len(engine.stablehlo_version()) == 3
+    bf = engine.buffer_from_host(memoryview(bits), engine.PJRT_TYPES.index("BF16"), [3], None, 0)
+    assert bf.nbytes == 6 and engine.to_host(bf) == bits.tobytes()
+    with pytest.raises(TypeError, match="Unsupported"):      # "Unsupported" in the class or text -> UNIMPLEMENTED (:185-226)
+        engine.buffer_from_host(None, engine.PJRT_TYPES.index("C64"), [1], None, 0)
+    assert isinstance(engine.device_kind(), str)
+    ver = engine.stablehlo_version()
+    assert len(ver) == 3 and all(type(v) is int for v in ver)
