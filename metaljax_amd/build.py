@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libqmm_hip.so")
-SOURCES = ["qmm_api.hip", "qmm_gemv.hip", "qmm_skinny.hip", "qmm_skinny2.hip", "qmm_skinny3.hip", "qmm_gemm.hip", "qmm_gemm2.hip", "qmm_gemm2s.hip", "qmm_mxfp4.hip", "qmm_util.hip"]
+SOURCES = ["qmm_api.hip", "qmm_gemv.hip", "qmm_skinny.hip", "qmm_skinny2.hip", "qmm_gemm.hip", "qmm_gemm2.hip", "qmm_gemm2s.hip", "qmm_mxfp4.hip", "qmm_util.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wno-unused-function"]

@@ -386,9 +386,6 @@ bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                       const void* b);
 void skinny_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int tab, hipStream_t st);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
-bool skinny3_wanted(int64_t M, int64_t N, int64_t K, int gs, int bits, int* rows_per_wg);
-void skinny3_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows_per_wg,
-                      hipStream_t st);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
 void skinny2_dispatch(const GemvArgs& a0, int64_t batch, int gs, int bits, int rows, hipStream_t st,
                       int tab, bool force_direct);
@@ -435,7 +432,6 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
     // self-loading one everywhere, for comparison)
     static const int v1 = env_int("QMM_SKINNY_V1");
     int rows;
-    if (skinny3_wanted(M, N, K, gs, bits, &rows)) return skinny3_dispatch(a, batch, gs, bits, rows, st);
     if (!v1 && skinny2_plan(M, N, K, bits, &rows)) skinny2_dispatch(a, batch, gs, bits, rows, st, tab, false);
     else skinny_dispatch(a, batch, gs, bits, tab, st);
     return;
