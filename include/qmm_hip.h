@@ -14,7 +14,10 @@
  *
  * Layouts (identical to what the reference hands mx.quantized_matmul,
  * reference src/metaljax/qmm.py:2469-2501 and :206-282):
- *   x        [batch, M, K] row-major, dtype x_dtype
+ *   x        [batch, M, K] row-major, dtype x_dtype (bf16, or float16 / float32:
+ *            those are split, exactly, into two / three bf16 terms that are
+ *            multiplied like bf16 activations and added in float32 -- the
+ *            workspace queries take x_dtype for that)
  *   w        affine: uint32 [batch, N, K*bits/32]; element i of a row at bits
  *            [i*bits, (i+1)*bits) of the row's little-endian stream.
  *            mxfp4:  the same stream of 4-bit E2M1 codes (uint32 [N, K/8] ==
@@ -76,8 +79,9 @@ size_t qmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int g
  * expert sort's arrays, plus the segment list of the grouped decode (up to
  * 16 pairs an expert on average: one decode product per expert and sixteen
  * pairs) or the re-laid activation copy of the prefill kernel (more pairs).
- * With less the call still runs, on a slower kernel. */
-size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K);
+ * With less the call still runs, on a slower kernel (bf16 activations; float16
+ * and float32 activations need the whole of it). */
+size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K, int x_dtype);
 
 /* The kernel family and launch geometry the dispatcher would choose. */
 int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode,
@@ -102,7 +106,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
  * segment list and the re-laid activation copy live in a device array of
  * QMM_STATIC_SCRATCH_BYTES that is part of the library's code object (every
  * GPU the library runs on holds one until the process ends).  A call whose
- * qmm_gather_workspace_bytes(P, E, N, K) exceeds that size fails with
+ * qmm_gather_workspace_bytes(P, E, N, K, x_dtype) exceeds that size fails with
  * QMM_ERR_WORKSPACE and launches nothing.  The call allocates and frees
  * nothing.  Every call on a GPU uses that GPU's one array: calls that overlap
  * on one GPU (different streams, or threads) race; calls in stream order do

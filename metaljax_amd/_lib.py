@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libqmm_hip.so")
 
 QMM_OK = 0
+ABI_VERSION = 2
 ERR_NAMES = {1: "BAD_ARGUMENT", 2: "BAD_SHAPE", 3: "UNSUPPORTED", 4: "WORKSPACE", 5: "HIP"}
 F32, BF16, F16 = 0, 1, 2
 STATIC_SCRATCH_BYTES = 16 << 20      # QMM_STATIC_SCRATCH_BYTES of include/qmm_hip.h
@@ -66,7 +67,7 @@ def load():
                                          ci, ci, ci, vp, sz, vp]
     lib.qmm_workspace_bytes.argtypes = [i64, i64, i64, i64, ci, ci, ci, ci]
     lib.qmm_workspace_bytes.restype = sz
-    lib.qmm_gather_workspace_bytes.argtypes = [i64, i64, i64, i64]
+    lib.qmm_gather_workspace_bytes.argtypes = [i64, i64, i64, i64, ci]
     lib.qmm_gather_workspace_bytes.restype = sz
     lib.qmm_plan.argtypes = [i64, i64, i64, ci, ci, ci, ip, ip, ip]
     lib.qmm_gather_qmm.argtypes = [vp, ci, vp, vp, vp, ci, vp, ci, vp, vp, i64, i64, i64, i64,
@@ -81,6 +82,9 @@ def load():
     lib.qmm_take_k.argtypes = [vp, ci, vp, vp, i64, i64, vp]
     for name in SYMBOLS:
         getattr(lib, name)
+    if lib.qmm_abi_version() != ABI_VERSION:
+        raise QmmLibraryError(f"{LIB_PATH} has ABI version {lib.qmm_abi_version()}, this binding "
+                              f"speaks {ABI_VERSION}: rebuild it with `python -m metaljax_amd.build`")
     _lib = lib
     return lib
 

@@ -49,6 +49,11 @@ void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void
                       hipStream_t st);
 void take_dispatch(const void* x, int x_dtype, const int32_t* perm, void* out, int64_t rows,
                    int64_t K, hipStream_t st);
+void split_terms_dispatch(const void* x, int x_dtype, void* out, int64_t batch, int64_t rows,
+                          int64_t K, const int32_t* src_row, int64_t x_rows, hipStream_t st);
+void sum_terms_dispatch(const void* part, int terms, void* y, int y_dtype, int64_t batch,
+                        int64_t rows, int64_t N, const int32_t* offsets,
+                        const int32_t* expert_of_row, int64_t E, hipStream_t st);
 
 namespace {
 
@@ -108,8 +113,8 @@ int check_quant(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const
 
 int check_io(const void* x, int x_dtype, void* y, int y_dtype) {
   if (!x || !y) return fail(QMM_ERR_BAD_ARGUMENT, "null activation or output pointer");
-  if (x_dtype != QMM_BF16)
-    return fail(QMM_ERR_UNSUPPORTED, "activation dtype %d (bf16 built)", x_dtype);
+  if (x_dtype != QMM_BF16 && x_dtype != QMM_F16 && x_dtype != QMM_F32)
+    return fail(QMM_ERR_UNSUPPORTED, "activation dtype %d", x_dtype);
   if (y_dtype != QMM_BF16 && y_dtype != QMM_F32 && y_dtype != QMM_F16)
     return fail(QMM_ERR_UNSUPPORTED, "output dtype %d", y_dtype);
   if (!aligned16(x)) return fail(QMM_ERR_BAD_ARGUMENT, "activation pointer not 16-byte aligned");
@@ -194,6 +199,40 @@ bool grouped_decode_pairs(int64_t P, int64_t E) {
   return gd_max ? P <= gd_max : P <= 16 * E && P <= 4096;
 }
 
+// ---- float16 / float32 activations ---------------------------------------------
+// The kernels multiply bf16 operands.  Wider activations are split, exactly,
+// into bf16 terms (float16: two, float32: three), every term is multiplied
+// like a bf16 activation (products exact, float32 accumulate) and the terms'
+// float32 results are added, largest first, before the one rounding to the
+// output type.  In the dense decode case the terms ride as extra rows of the
+// same launch (terms x M <= 16: the weight is still streamed once).
+int act_terms(int x_dtype) { return x_dtype == QMM_F32 ? 3 : x_dtype == QMM_F16 ? 2 : 1; }
+
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// Scratch of the bf16 dense / grouped product over `rows` rows.  `exact`: the
+// activation terms must stay exact, so MXFP4 weights take the bf16 kernels
+// (their FP6 activation terms would round).
+size_t dense_scratch(int64_t rows, int64_t N, int64_t K, int mode, bool exact) {
+  if (mode == QMM_MODE_MXFP4 && !exact && rows > kGemvMaxM && mxfp4_mfma_supported(rows, N, K))
+    return mxfp4_workspace_bytes(rows, K);
+  if (rows > kGemvMaxM && gemm2_supported(rows, N, K)) return gemm2_workspace_bytes(rows, K);
+  return 0;
+}
+
+size_t gather_scratch(int64_t P, int64_t E, int64_t N, int64_t K, bool exact) {
+  if (P < kGroupedDecodeMinPairs) return 0;
+  const size_t decode = grouped_decode_pairs(P, E) ? route_bytes_segments(P, E) : 0;
+  if (P <= kGatherGemvMaxPairs) return decode;    // the expert sort of the grouped decode
+  // the expert sort's arrays, then (when the register-operand kernel serves
+  // the shape) the re-laid copy of the gathered activation rows
+  size_t relaid = gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0;
+  if (!exact && mxfp4_mfma_supported(P, N, K) && mxfp4_workspace_bytes(P, K) > relaid)
+    relaid = mxfp4_workspace_bytes(P, K);          // the mode is not known here: the larger of the two
+  const size_t gemm = route_bytes(P, E) + relaid;
+  return gemm > decode ? gemm : decode;
+}
+
 // ---- scratch of the allocation-free entry point ------------------------------
 // Part of the code object: each GPU that loads the library holds its own copy
 // at its own address.  In host code the name is only a handle for
@@ -229,28 +268,28 @@ using namespace qmm;
 
 extern "C" {
 
-int qmm_abi_version(void) { return 1; }
+int qmm_abi_version(void) { return 2; }
 
 const char* qmm_last_error(void) { return g_err; }
 
-size_t qmm_workspace_bytes(int64_t, int64_t M, int64_t N, int64_t K, int, int, int mode, int) {
-  if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K))
-    return mxfp4_workspace_bytes(M, K);
-  if (M > kGemvMaxM && gemm2_supported(M, N, K)) return gemm2_workspace_bytes(M, K);
-  return 0;
+size_t qmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int, int, int mode,
+                           int x_dtype) {
+  const int terms = act_terms(x_dtype);
+  if (terms == 1) return dense_scratch(M, N, K, mode, false);
+  // terms as bf16 rows, their float32 products, then the scratch of the bf16
+  // product: over terms x M stacked rows (dense) or over M rows (grouped)
+  if (batch < 1) batch = 1;
+  const size_t stacked = dense_scratch(terms * M, N, K, mode, true), plain = dense_scratch(M, N, K, mode, true);
+  return align256((size_t)(batch * terms * M * K) * 2) + align256((size_t)(batch * terms * M * N) * 4) +
+         (stacked > plain ? stacked : plain);
 }
 
-size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K) {
-  if (P < kGroupedDecodeMinPairs) return 0;
-  const size_t decode = grouped_decode_pairs(P, E) ? route_bytes_segments(P, E) : 0;
-  if (P <= kGatherGemvMaxPairs) return decode;    // the expert sort of the grouped decode
-  // the expert sort's arrays, then (when the register-operand kernel serves
-  // the shape) the re-laid copy of the gathered activation rows
-  size_t relaid = gemm2_supported(P, N, K) ? gemm2_workspace_bytes(P, K) : 0;
-  if (mxfp4_mfma_supported(P, N, K) && mxfp4_workspace_bytes(P, K) > relaid)
-    relaid = mxfp4_workspace_bytes(P, K);          // the mode is not known here: the larger of the two
-  const size_t gemm = route_bytes(P, E) + relaid;
-  return gemm > decode ? gemm : decode;
+size_t qmm_gather_workspace_bytes(int64_t P, int64_t E, int64_t N, int64_t K, int x_dtype) {
+  const int terms = act_terms(x_dtype);
+  if (terms == 1) return gather_scratch(P, E, N, K, false);
+  // the gathered rows' terms, their float32 products, the bf16 product's scratch
+  return align256((size_t)(terms * P * K) * 2) + align256((size_t)(terms * P * N) * 4) +
+         gather_scratch(P, E, N, K, true);
 }
 
 int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode, int* kernel,
@@ -291,11 +330,12 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
   return QMM_OK;
 }
 
-int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* scales,
-                         const void* biases, int table_dtype, void* y, int y_dtype,
-                         int64_t batch, int64_t M, int64_t N, int64_t K, int group_size,
-                         int bits, int mode, void* workspace, size_t workspace_bytes,
-                         void* stream) {
+// The three products on bf16 activations.  `exact`: the activations are exact
+// terms of a wider type (MXFP4 weights then take the bf16 kernels).
+static int dense_bf16(const void* x, int x_dtype, const void* w, const void* scales,
+                      const void* biases, int table_dtype, void* y, int y_dtype, int64_t batch,
+                      int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode,
+                      void* workspace, size_t workspace_bytes, void* stream, bool exact) {
   if (batch < 0 || M < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
   if (batch == 0 || M == 0 || N == 0) return QMM_OK;
   if (K == 0) return fail(QMM_ERR_BAD_SHAPE, "K=0");
@@ -316,7 +356,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
   const int64_t ng = mode == QMM_MODE_MXFP4 ? K / 32 : K / group_size;
   const int tabsz = mode == QMM_MODE_MXFP4 ? 1 : (table_dtype == QMM_F32 ? 4 : 2);
   const int ysz = y_dtype == QMM_F32 ? 4 : 2;
-  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(M, N, K)) {
+  if (mode == QMM_MODE_MXFP4 && !exact && mxfp4_mfma_supported(M, N, K)) {
     // block-scaled matrix cores; the activations are split into the workspace first
     const size_t need = mxfp4_workspace_bytes(M, K);
     if (!workspace || workspace_bytes < need)
@@ -368,11 +408,11 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
   return QMM_OK;
 }
 
-int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scales,
-                    const void* biases, int table_dtype, void* y, int y_dtype,
-                    const int32_t* row_offsets, int64_t R, int64_t E, int64_t N, int64_t K,
-                    int group_size, int bits, int mode, void* workspace, size_t workspace_bytes,
-                    void* stream) {
+static int grouped_bf16(const void* x, int x_dtype, const void* w, const void* scales,
+                        const void* biases, int table_dtype, void* y, int y_dtype,
+                        const int32_t* row_offsets, int64_t R, int64_t E, int64_t N, int64_t K,
+                        int group_size, int bits, int mode, void* workspace, size_t workspace_bytes,
+                        void* stream, bool exact) {
   if (R < 0 || E < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
   if (R == 0 || N == 0 || E == 0) return QMM_OK;
   if (!row_offsets) return fail(QMM_ERR_BAD_ARGUMENT, "null row_offsets");
@@ -382,7 +422,7 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   if (rc) return rc;
   if (R > INT32_MAX || N > INT32_MAX || K > INT32_MAX || E > 65535 || R * K >= (1ll << 30))
     return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
-  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(R, N, K) && workspace &&
+  if (mode == QMM_MODE_MXFP4 && !exact && mxfp4_mfma_supported(R, N, K) && workspace &&
       workspace_bytes >= mxfp4_workspace_bytes(R, K) && aligned16(workspace) && aligned16(scales)) {
     // MXFP4 experts on the block-scaled matrix cores
     mxfp4_mfma_dispatch(x, w, scales, y, y_dtype, row_offsets, nullptr, nullptr, R, R, E, N, K,
@@ -402,11 +442,11 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
   return check_launch("grouped gemm launch");
 }
 
-int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales,
-                   const void* biases, int table_dtype, void* y, int y_dtype,
-                   const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
-                   int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
-                   void* workspace, size_t workspace_bytes, void* stream) {
+static int gather_bf16(const void* x, int x_dtype, const void* w, const void* scales,
+                       const void* biases, int table_dtype, void* y, int y_dtype,
+                       const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
+                       int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
+                       void* workspace, size_t workspace_bytes, void* stream, bool exact) {
   if (P < 0 || T < 0 || E < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
   if (P == 0 || N == 0) return QMM_OK;
   if (!rhs_idx) return fail(QMM_ERR_BAD_ARGUMENT, "null rhs_idx");
@@ -451,7 +491,7 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
                      ro, cursor, src_row, out_row, static_cast<int32_t*>(nullptr));
   rc = check_launch("route launch");
   if (rc) return rc;
-  if (mode == QMM_MODE_MXFP4 && mxfp4_mfma_supported(P, N, K) &&
+  if (mode == QMM_MODE_MXFP4 && !exact && mxfp4_mfma_supported(P, N, K) &&
       workspace_bytes >= need + mxfp4_workspace_bytes(P, K) && aligned16(workspace) &&
       aligned16(scales)) {
     mxfp4_mfma_dispatch(x, w, scales, y, y_dtype, ro, src_row, out_row, P, T, E, N, K,
@@ -471,13 +511,104 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
   return check_launch("gather gemm launch");
 }
 
+int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* scales,
+                         const void* biases, int table_dtype, void* y, int y_dtype,
+                         int64_t batch, int64_t M, int64_t N, int64_t K, int group_size,
+                         int bits, int mode, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  const int terms = act_terms(x_dtype);
+  if (terms == 1 || batch <= 0 || M <= 0 || N <= 0 || K <= 0 || !x)
+    return dense_bf16(x, x_dtype, w, scales, biases, table_dtype, y, y_dtype, batch, M, N, K,
+                      group_size, bits, mode, workspace, workspace_bytes, stream, false);
+  // bf16 terms as extra rows: x2 [batch, terms * M, K] -> p2 [batch, terms * M, N] -> y
+  if (!aligned16(x)) return fail(QMM_ERR_BAD_ARGUMENT, "activation pointer not 16-byte aligned");
+  if (batch * terms * M * K >= (1ll << 30))
+    return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  const size_t xs = align256((size_t)(batch * terms * M * K) * 2);
+  const size_t ps = align256((size_t)(batch * terms * M * N) * 4);
+  const size_t inner = dense_scratch(terms * M, N, K, mode, true);
+  if (!workspace || workspace_bytes < xs + ps + inner || !aligned16(workspace))
+    return fail(QMM_ERR_WORKSPACE, "float16 / float32 activations need %zu aligned workspace bytes, got %zu",
+                xs + ps + inner, workspace ? workspace_bytes : (size_t)0);
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  split_terms_dispatch(x, x_dtype, ws, batch, M, K, nullptr, 0, st);
+  int rc = check_launch("activation split launch");
+  if (rc) return rc;
+  rc = dense_bf16(ws, QMM_BF16, w, scales, biases, table_dtype, ws + xs, QMM_F32, batch, terms * M, N, K,
+                  group_size, bits, mode, inner ? ws + xs + ps : nullptr, inner, stream, true);
+  if (rc) return rc;
+  if (!y) return fail(QMM_ERR_BAD_ARGUMENT, "null output pointer");
+  sum_terms_dispatch(ws + xs, terms, y, y_dtype, batch, M, N, nullptr, nullptr, 0, st);
+  return check_launch("term sum launch");
+}
+
+int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scales,
+                    const void* biases, int table_dtype, void* y, int y_dtype,
+                    const int32_t* row_offsets, int64_t R, int64_t E, int64_t N, int64_t K,
+                    int group_size, int bits, int mode, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+  const int terms = act_terms(x_dtype);
+  if (terms == 1 || R <= 0 || E <= 0 || N <= 0 || K <= 0 || !x || !row_offsets || !y)
+    return grouped_bf16(x, x_dtype, w, scales, biases, table_dtype, y, y_dtype, row_offsets, R, E, N, K,
+                        group_size, bits, mode, workspace, workspace_bytes, stream, false);
+  // one grouped product per bf16 term (the rows keep their expert order)
+  if (!aligned16(x)) return fail(QMM_ERR_BAD_ARGUMENT, "activation pointer not 16-byte aligned");
+  const size_t xs = align256((size_t)(terms * R * K) * 2), ps = align256((size_t)(terms * R * N) * 4);
+  const size_t inner = dense_scratch(R, N, K, mode, true);
+  if (!workspace || workspace_bytes < xs + ps + inner || !aligned16(workspace))
+    return fail(QMM_ERR_WORKSPACE, "float16 / float32 activations need %zu aligned workspace bytes, got %zu",
+                xs + ps + inner, workspace ? workspace_bytes : (size_t)0);
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  split_terms_dispatch(x, x_dtype, ws, 1, R, K, nullptr, 0, st);
+  int rc = check_launch("activation split launch");
+  for (int t = 0; t < terms && !rc; ++t)
+    rc = grouped_bf16(ws + (size_t)t * R * K * 2, QMM_BF16, w, scales, biases, table_dtype,
+                      ws + xs + (size_t)t * R * N * 4, QMM_F32, row_offsets, R, E, N, K, group_size, bits,
+                      mode, inner ? ws + xs + ps : nullptr, inner, stream, true);
+  if (rc) return rc;
+  sum_terms_dispatch(ws + xs, terms, y, y_dtype, 1, R, N, row_offsets, nullptr, E, st);
+  return check_launch("term sum launch");
+}
+
+int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales,
+                   const void* biases, int table_dtype, void* y, int y_dtype,
+                   const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
+                   int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  const int terms = act_terms(x_dtype);
+  if (terms == 1 || P <= 0 || T < 0 || E < 0 || N <= 0 || K <= 0 || !x || !rhs_idx || !y)
+    return gather_bf16(x, x_dtype, w, scales, biases, table_dtype, y, y_dtype, lhs_idx, rhs_idx, P, T, E,
+                       N, K, group_size, bits, mode, workspace, workspace_bytes, stream, false);
+  // the pairs' rows are gathered while they are split; every term is then a
+  // gathered product over rows already in pair order
+  const size_t xs = align256((size_t)(terms * P * K) * 2), ps = align256((size_t)(terms * P * N) * 4);
+  const size_t inner = gather_scratch(P, E, N, K, true);
+  if (!workspace || workspace_bytes < xs + ps + inner || !aligned16(workspace))
+    return fail(QMM_ERR_WORKSPACE, "float16 / float32 activations need %zu aligned workspace bytes, got %zu",
+                xs + ps + inner, workspace ? workspace_bytes : (size_t)0);
+  if (terms * P * K >= (1ll << 30)) return fail(QMM_ERR_BAD_SHAPE, "shape exceeds kernel index range");
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  split_terms_dispatch(x, x_dtype, ws, 1, P, K, lhs_idx, T, st);      // lhs_idx null: row p of x
+  int rc = check_launch("activation split launch");
+  for (int t = 0; t < terms && !rc; ++t)
+    rc = gather_bf16(ws + (size_t)t * P * K * 2, QMM_BF16, w, scales, biases, table_dtype,
+                     ws + xs + (size_t)t * P * N * 4, QMM_F32, nullptr, rhs_idx, P, P, E, N, K, group_size,
+                     bits, mode, inner ? ws + xs + ps : nullptr, inner, stream, true);
+  if (rc) return rc;
+  sum_terms_dispatch(ws + xs, terms, y, y_dtype, 1, P, N, nullptr, rhs_idx, E, st);
+  return check_launch("term sum launch");
+}
+
 int qmm_gather_qmm_static(const void* x, int x_dtype, const void* w, const void* scales,
                           const void* biases, int table_dtype, void* y, int y_dtype,
                           const int32_t* lhs_idx, const int32_t* rhs_idx, int64_t P, int64_t T,
                           int64_t E, int64_t N, int64_t K, int group_size, int bits, int mode,
                           void* stream) {
   if (P < 0 || T < 0 || E < 0 || N < 0 || K < 0) return fail(QMM_ERR_BAD_ARGUMENT, "negative shape");
-  const size_t need = qmm_gather_workspace_bytes(P, E, N, K);
+  const size_t need = qmm_gather_workspace_bytes(P, E, N, K, x_dtype);
   if (need > (size_t)QMM_STATIC_SCRATCH_BYTES)
     return fail(QMM_ERR_WORKSPACE,
                 "gather_qmm_static: %lld pairs over %lld experts of [%lld, %lld] need %zu scratch "

@@ -102,6 +102,63 @@ __global__ __launch_bounds__(kBlock) void take_kernel(const T* __restrict__ x,
   out[i] = x[r * k + perm[j]];
 }
 
+// float16 / float32 activations as exact sums of bf16 terms (float16: 11
+// significant bits = 8 + 3; float32: 24 = 8 + 8 + 8), term t of batch entry z,
+// row m at out[z][t][m][:]: the matrix cores then multiply bf16 operands and
+// every product stays exact.  x [batch, rows, K]; out bf16 [batch, TERMS, rows, K].
+template <int TERMS, typename T>
+__global__ void split_terms_kernel(const T* __restrict__ x, uint16_t* __restrict__ out,
+                                   int64_t rows_k, int64_t k, int64_t total,
+                                   const int32_t* __restrict__ src_row, int64_t x_rows) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t z = i / rows_k, j = i - z * rows_k;
+  int64_t src = i;
+  bool ok = true;
+  if (src_row) {                                   // rows gathered: out row j / k is x row src_row[j / k]
+    const int64_t row = j / k, sr = src_row[row];
+    ok = sr >= 0 && sr < x_rows;                   // a row outside x gathers zeros
+    src = sr * k + (j - row * k);
+  }
+  float v = 0.f;
+  if (ok) {
+    if constexpr (sizeof(T) == 4) v = x[src];
+    else v = f16_bits_to_f32(x[src]);
+  }
+  uint16_t* o = out + z * TERMS * rows_k + j;
+#pragma unroll
+  for (int t = 0; t < TERMS; ++t) {
+    const uint32_t hi = __float_as_uint(v) & 0xFFFF0000u;       // truncation: the remainder is exact
+    o[(int64_t)t * rows_k] = (uint16_t)(hi >> 16);
+    v -= __uint_as_float(hi);
+  }
+}
+
+// y[z][m][n] = sum_t part[z][t][m][n] (float32 partial products, added in term
+// order: largest first), rounded once to the output type.  Rows that the
+// product did not compute are left alone: rows outside [offsets[0], offsets[E])
+// of a grouped product, pairs whose expert index is outside [0, E) of a
+// gathered one.
+template <int TERMS>
+__global__ void sum_terms_kernel(const float* __restrict__ part, void* __restrict__ y, int y_dtype,
+                                 int64_t rows_n, int64_t n, int64_t total,
+                                 const int32_t* __restrict__ offsets,
+                                 const int32_t* __restrict__ expert_of_row, int E) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t z = i / rows_n, j = i - z * rows_n;
+  if (offsets || expert_of_row) {
+    const int64_t row = j / n;
+    if (offsets && (row < offsets[0] || row >= offsets[E])) return;
+    if (expert_of_row && (expert_of_row[row] < 0 || expert_of_row[row] >= E)) return;
+  }
+  const float* p = part + z * TERMS * rows_n + j;
+  float v = p[0];
+#pragma unroll
+  for (int t = 1; t < TERMS; ++t) v += p[(int64_t)t * rows_n];
+  store_out(y, i, v, y_dtype);
+}
+
 inline unsigned blocks_for(int64_t n) { return (unsigned)ceil_div(n, kBlock); }
 
 }  // namespace
@@ -141,6 +198,38 @@ void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void
   if (words == 0) return;
   if (bits == 4) hipLaunchKernelGGL((dequant_kernel<0, 4>), dim3(blocks_for(words)), dim3(kBlock), 0, st, wp, s, b, tab, out, out_dtype, words, wpr, gs);
   else hipLaunchKernelGGL((dequant_kernel<0, 8>), dim3(blocks_for(words)), dim3(kBlock), 0, st, wp, s, b, tab, out, out_dtype, words, wpr, gs);
+}
+
+// x (float16 / float32) [batch, rows, K] -> bf16 terms [batch, terms, rows, K];
+// with src_row (batch = 1): out row r = x row src_row[r] of x [x_rows, K]
+void split_terms_dispatch(const void* x, int x_dtype, void* out, int64_t batch, int64_t rows,
+                          int64_t K, const int32_t* src_row, int64_t x_rows, hipStream_t st) {
+  const int64_t total = batch * rows * K;
+  if (total == 0) return;
+  uint16_t* o = static_cast<uint16_t*>(out);
+  if (x_dtype == QMM_F32)
+    hipLaunchKernelGGL((split_terms_kernel<3, float>), dim3(blocks_for(total)), dim3(kBlock), 0, st,
+                       static_cast<const float*>(x), o, rows * K, K, total, src_row, x_rows);
+  else
+    hipLaunchKernelGGL((split_terms_kernel<2, uint16_t>), dim3(blocks_for(total)), dim3(kBlock), 0, st,
+                       static_cast<const uint16_t*>(x), o, rows * K, K, total, src_row, x_rows);
+}
+
+// part float32 [batch, terms, rows, N] -> y [batch, rows, N]; `offsets` ([E+1],
+// grouped form) / `expert_of_row` ([rows], gathered form) name the rows that
+// were computed (null: all of them)
+void sum_terms_dispatch(const void* part, int terms, void* y, int y_dtype, int64_t batch,
+                        int64_t rows, int64_t N, const int32_t* offsets,
+                        const int32_t* expert_of_row, int64_t E, hipStream_t st) {
+  const int64_t total = batch * rows * N;
+  if (total == 0) return;
+  const float* p = static_cast<const float*>(part);
+  if (terms == 3)
+    hipLaunchKernelGGL(sum_terms_kernel<3>, dim3(blocks_for(total)), dim3(kBlock), 0, st, p, y, y_dtype,
+                       rows * N, N, total, offsets, expert_of_row, (int)E);
+  else
+    hipLaunchKernelGGL(sum_terms_kernel<2>, dim3(blocks_for(total)), dim3(kBlock), 0, st, p, y, y_dtype,
+                       rows * N, N, total, offsets, expert_of_row, (int)E);
 }
 
 void take_dispatch(const void* x, int x_dtype, const int32_t* perm, void* out, int64_t rows,

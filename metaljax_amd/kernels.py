@@ -54,7 +54,7 @@ def quantized_matmul(x, w, scales, biases=None, transpose=True, group_size=64, b
                      mode="affine", out_dtype=None):
     """y[..., M, N] = x[..., M, K] @ dequant(w)[..., N, K]^T, float32 accumulate.
 
-    x [M,K] or [B,M,K] (bf16); w uint32 [(B,)N,K*bits/32] (or the same bytes
+    x [M,K] or [B,M,K] (bf16, float16 or float32); w uint32 [(B,)N,K*bits/32] (or the same bytes
     as uint8); scales/biases [(B,)N,K/group_size] (bf16/f16/f32), for mxfp4
     uint8 E8M0 [(B,)N,K/32] and biases None.  Result dtype = out_dtype or x's.
     """
@@ -151,7 +151,7 @@ def gather_qmm(x, w, scales, biases=None, lhs_indices=None, rhs_indices=None, tr
     y = torch.empty((p, n), dtype=out_dtype, device=x.device)
     x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
     biases = None if biases is None else biases.contiguous()
-    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k))
+    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k, _dt(x.dtype)))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
     tab = _dt(scales.dtype) if mode == "affine" else BF16
     rc = lib.qmm_gather_qmm(_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab,

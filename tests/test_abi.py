@@ -89,18 +89,18 @@ def test_plan_of_the_decode_variants(lib):
 def test_gather_workspace_covers_the_grouped_decode(lib):
     """From four pairs up to sixteen an expert the workspace holds the expert
     sort and the segment list; below four pairs nothing is needed."""
-    assert lib.qmm_gather_workspace_bytes(2, 8, 14336, 4096) == 0
-    few = lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096)
+    assert lib.qmm_gather_workspace_bytes(2, 8, 14336, 4096, _lib.BF16) == 0
+    few = lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096, _lib.BF16)
     sort_only = ((2 * 8 + 1 + 2 * 16) * 4 + 255) // 256 * 256
     assert few >= sort_only and few % 256 == 0
-    assert lib.qmm_gather_workspace_bytes(128, 8, 14336, 4096) >= lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096)
+    assert lib.qmm_gather_workspace_bytes(128, 8, 14336, 4096, _lib.BF16) >= lib.qmm_gather_workspace_bytes(16, 8, 14336, 4096, _lib.BF16)
 
 
 def test_workspace_queries_need_no_device(lib):
     assert lib.qmm_workspace_bytes(1, 16, 14336, 4096, 64, 4, 0, _lib.BF16) == 0
-    need = lib.qmm_gather_workspace_bytes(1024, 8, 14336, 4096)
+    need = lib.qmm_gather_workspace_bytes(1024, 8, 14336, 4096, _lib.BF16)
     assert need > 0 and need % 4 == 0
-    assert lib.qmm_gather_workspace_bytes(0, 8, 64, 64) >= 0
+    assert lib.qmm_gather_workspace_bytes(0, 8, 64, 64, _lib.BF16) >= 0
 
 
 def test_argument_errors_are_reported_before_any_launch(lib):
@@ -128,7 +128,7 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):
     assert re.search(r"#define QMM_STATIC_SCRATCH_BYTES \(16u << 20\)", text)
     assert _lib.STATIC_SCRATCH_BYTES == 16 << 20
     p, e, n, k = 4096, 8, 14336, 4096                 # the re-laid activations alone are 32 MiB
-    assert lib.qmm_gather_workspace_bytes(p, e, n, k) > _lib.STATIC_SCRATCH_BYTES
+    assert lib.qmm_gather_workspace_bytes(p, e, n, k, _lib.BF16) > _lib.STATIC_SCRATCH_BYTES
     rc = lib.qmm_gather_qmm_static(None, _lib.BF16, None, None, None, _lib.BF16, None, _lib.BF16,
                                    None, None, p, p, e, n, k, 64, 4, 0, None)
     assert rc == 4 and b"static scratch" in lib.qmm_last_error()

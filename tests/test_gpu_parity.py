@@ -74,7 +74,7 @@ def make_x(rng, m, k):
 
 def test_library_reports_loaded():
     from metaljax_amd import _lib
-    assert _lib.load().qmm_abi_version() == 1
+    assert _lib.load().qmm_abi_version() == _lib.ABI_VERSION
 
 
 @pytest.mark.parametrize("bits", [2, 4, 8])
@@ -748,7 +748,7 @@ def test_gather_qmm_with_only_the_sort_workspace_still_runs():
     x, xd = make_x(rng, t, k)
     rhs = rng.integers(0, e, size=t).astype(np.int32)
     rd = torch.from_numpy(rhs).to(DEV)
-    full = int(lib.qmm_gather_workspace_bytes(t, e, n, k))
+    full = int(lib.qmm_gather_workspace_bytes(t, e, n, k, _lib.BF16))
     small = ((2 * e + 1 + 2 * t) * 4 + 255) // 256 * 256
     assert full > small
     ws = torch.empty(small, dtype=torch.uint8, device=DEV)
@@ -863,7 +863,7 @@ def test_unsupported_and_bad_shapes_raise_without_launching():
     with pytest.raises(K.UnsupportedQmm):
         K.quantized_matmul(x, w, s, s, group_size=16, bits=4)
     with pytest.raises(K.UnsupportedQmm):
-        K.quantized_matmul(x.float(), w, s, s, group_size=64, bits=4)
+        K.quantized_matmul(x.double(), w, s, s, group_size=64, bits=4)     # float64 activations
     with pytest.raises(K.QmmError):
         K.quantized_matmul(x, w, s, None, group_size=64, bits=4)       # affine without biases
     with pytest.raises(K.QmmError):
@@ -939,7 +939,7 @@ def test_gather_qmm_few_pairs_invalid_indices_touch_nothing():
     from metaljax_amd import _lib
     lib = _lib.load()
     p = len(lhs)
-    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k))
+    nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k, _lib.BF16))
     assert nbytes > 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
     y = torch.full((p, n), 7.0, dtype=torch.float32, device=DEV)
@@ -1140,3 +1140,98 @@ def test_grouped_qmm_short_experts_with_table_rows_longer_than_a_cache_line(bits
             assert O.rel_l2(y32[lo:hi], want[lo:hi]) <= 2e-5, (i, O.rel_l2(y32[lo:hi], want[lo:hi]))
             assert O.rel_l2(y16[lo:hi], want[lo:hi]) <= TOL_BF16_OUT, i
     np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
+# ------------------------------------------ float16 / float32 activations ----
+
+def _x_of(rng, m, k, el):
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if el == "f16":
+        x = x.astype(np.float16)
+        return x.astype(np.float32), torch.from_numpy(x).to(DEV)
+    return x, torch.from_numpy(x).to(DEV)
+
+
+@pytest.mark.parametrize("el", ["f32", "f16"])
+@pytest.mark.parametrize("bits,gs,m,n,k", [
+    (4, 64, 1, 300, 4096),      # three / two terms as rows of one decode launch (loader-wavefront kernel)
+    (4, 64, 5, 2100, 4096),     # float32: 15 rows, still one decode launch
+    (8, 64, 3, 200, 512),       # the self-loading kernel
+    (4, 32, 2, 72, 96),         # the general decode kernel
+    (4, 64, 8, 136, 1024),      # float32: 24 stacked rows -> the prefill kernel; float16: 16 -> decode
+    (4, 128, 40, 200, 512),     # prefill
+    (8, 64, 130, 136, 1024),
+])
+def test_float16_and_float32_activations_affine(el, bits, gs, m, n, k):
+    """Activations wider than bf16 are split exactly into bf16 terms, so the
+    product keeps the accuracy of the kernel that runs it: the exactly
+    reconstructed weight where the stacked rows fit the decode kernel, the
+    bf16-rounded weight tile on the prefill kernels."""
+    rng = np.random.default_rng(bits * 100 + gs + m + k)
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    x, xd = _x_of(rng, m, k, el)
+    terms = 3 if el == "f32" else 2
+    rounding = "f32" if terms * m <= 16 else "bf16"
+    want = O.qmm(x, words, s, b, gs, bits, weight_rounding=rounding)
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits)        # result in the activations' type
+    assert y.dtype == xd.dtype
+    assert O.rel_l2(out_f32(y), want) <= (2e-5 if el == "f32" else 1e-3)
+
+
+@pytest.mark.parametrize("el", ["f32", "f16"])
+@pytest.mark.parametrize("m,n,k", [(2, 72, 256), (4, 1200, 4096), (64, 136, 1024), (40, 200, 768)])
+def test_float16_and_float32_activations_mxfp4(el, m, n, k):
+    """MXFP4 weights are exact in bf16, so with exact activation terms the
+    whole product is float32-accurate on every path (the reference's float32
+    cases, tests/test_qmm_mxfp4.py:453: rtol 1e-5)."""
+    rng = np.random.default_rng(m + n + k)
+    _, words, sb, wd, sd = make_mxfp4(rng, n, k)
+    x, xd = _x_of(rng, m, k, el)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+
+
+def test_float32_activations_batched():
+    rng = np.random.default_rng(11)
+    bsz, m, n, k = 3, 2, 96, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(bsz,))
+    x = rng.standard_normal((bsz, m, k)).astype(np.float32)
+    xd = torch.from_numpy(x).to(DEV)
+    want = np.stack([O.qmm(x[i], words[i], s[i], b[i], 64, 4) for i in range(bsz)])
+    y = out_f32(K.quantized_matmul(xd, wd, sd, bd, group_size=64, bits=4))
+    assert y.shape == (bsz, m, n)
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
+@pytest.mark.parametrize("el", ["f32", "f16"])
+def test_float16_and_float32_activations_grouped_and_gathered(el):
+    """The expert-indexed forms on wider activations: one product per bf16
+    term; rows outside the offsets and pairs naming no expert stay untouched."""
+    rng = np.random.default_rng(5 + len(el))
+    e, n, k = 4, 136, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    sizes = np.array([70, 0, 33, 20])
+    ro = np.concatenate([[3], 3 + np.cumsum(sizes)]).astype(np.int32)     # rows 0-2 and the last four belong to no expert
+    r = int(ro[-1]) + 4
+    x, xd = _x_of(rng, r, k, el)
+    want = O.grouped_qmm(x, words, s, b, ro, 64, 4, weight_rounding="bf16")
+    given = torch.full((r, n), 7.0, dtype=torch.float32, device=DEV)
+    K.grouped_qmm(xd, wd, sd, bd, torch.from_numpy(ro).to(DEV), group_size=64, bits=4, out=given)
+    got = out_f32(given)
+    assert (got[:3] == 7.0).all() and (got[ro[-1]:] == 7.0).all()
+    assert O.rel_l2(got[3:ro[-1]], want[3:ro[-1]]) <= 2e-5
+    # gathered: many pairs (prefill kernels), few pairs (grouped decode), three pairs (independent products)
+    for pairs, rounding in ((300, "bf16"), (24, "f32"), (3, "f32")):
+        lhs = rng.integers(0, r, size=pairs).astype(np.int32)
+        rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+        rhs_dev = rhs.copy()
+        rhs_dev[1] = e + 2                                   # names no expert
+        wantg = O.gather_qmm(x[:, None, :], words, s, b, lhs, rhs, 64, 4, weight_rounding=rounding)[:, 0]
+        yg = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs_dev).to(DEV),
+                                  group_size=64, bits=4, out_dtype=torch.float32))
+        good = np.arange(pairs) != 1
+        assert O.rel_l2(yg[good], wantg[good]) <= 2e-5, (pairs, O.rel_l2(yg[good], wantg[good]))

@@ -51,7 +51,7 @@ def _call(lib, c, static, y_dtype=torch.float32):
     if static:
         rc = lib.qmm_gather_qmm_static(*head, st)
     else:
-        nbytes = int(lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"]))
+        nbytes = int(lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"], _lib.BF16))
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=DEV)
         rc = lib.qmm_gather_qmm(*head, ws.data_ptr() if nbytes else None, nbytes, st)
     _lib.check(rc)
@@ -94,7 +94,7 @@ def test_static_scratch_limit_is_an_error_and_launches_nothing():
     lib = _lib.load()
     rng = np.random.default_rng(7)
     c = _case(rng, 2, 64, 8192, 8, 1100, "affine")       # 1100 pairs x K = 8192: the re-laid copy alone is 21 MiB
-    assert lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"]) > _lib.STATIC_SCRATCH_BYTES
+    assert lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"], _lib.BF16) > _lib.STATIC_SCRATCH_BYTES
     with pytest.raises(_lib.QmmError) as err:
         _call(lib, c, static=True)
     assert err.value.code == 4 and "static scratch" in str(err.value)
