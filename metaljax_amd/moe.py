@@ -117,3 +117,7 @@ def emit_bytes(g) -> int:
 
 def emit(interp, g, env):
     return g.run(interp, env)
+
+
+def plan_dispatches(interp, st):
+    return []

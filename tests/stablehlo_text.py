@@ -269,3 +269,103 @@ def random_mxfp4(shape_nk, seed=0, lo=117, hi=127):
     grid = np.array(list(E2M1) + [-v for v in E2M1], np.float32)
     w = grid[codes] * np.repeat(np.ldexp(np.float32(1), sb.astype(np.int32) - 127), 32, axis=-1)
     return codes, blocks, sb, w.astype(np.float32)
+
+
+# ---------------------------------------------- weights stored rows-first ----
+
+def affine_grouped(n, k, gs, t, interleave=False, el="bf16"):
+    """`tk,nk->tn` over a sub-channel weight whose group axis is split out of K
+    (what a packed checkpoint stores; reference tests/test_qmm.py:991-1027):
+    codes i8 [N, K] viewed as [N, K/gs, gs] -- or, interleaved, [N, gs, K/gs],
+    which scatters each group's columns across K at stride K/gs -- one scale /
+    zero pair per group broadcast over the group, reshaped back to [N, K].
+    The contraction runs over the LAST axis, so the weight can be packed by
+    blocks of rows."""
+    ng = k // gs
+    split = (n, gs, ng) if interleave else (n, ng, gs)
+    where = "[0, 2]" if interleave else "[0, 1]"
+    s3, q3 = _t(split, el), _t(split, "i8")
+    return f"""
+module @jit_affine_grouped {{
+  func.func public @main(%q: {_t((n, k), "i8")}, %scale: {_t((n, ng), "f32")}, %zero: {_t((n, ng), "i8")}, %x: {_t((t, k), el)}) -> {_t((t, n), el)} {{
+    %qs = stablehlo.reshape %q : ({_t((n, k), "i8")}) -> {q3}
+    %qf = stablehlo.convert %qs : ({q3}) -> {s3}
+    %sc = stablehlo.convert %scale : ({_t((n, ng), "f32")}) -> {_t((n, ng), el)}
+    %sb = stablehlo.broadcast_in_dim %sc, dims = {where} : ({_t((n, ng), el)}) -> {s3}
+    %zc = stablehlo.convert %zero : ({_t((n, ng), "i8")}) -> {_t((n, ng), el)}
+    %zb = stablehlo.broadcast_in_dim %zc, dims = {where} : ({_t((n, ng), el)}) -> {s3}
+    %d = stablehlo.subtract %qf, %zb : {s3}
+    %w3 = stablehlo.multiply %d, %sb : {s3}
+    %w = stablehlo.reshape %w3 : ({s3}) -> {_t((n, k), el)}
+    %y = stablehlo.dot_general %x, %w, contracting_dims = [1] x [1] : ({_t((t, k), el)}, {_t((n, k), el)}) -> {_t((t, n), el)}
+    return %y : {_t((t, n), el)}
+  }}
+}}
+"""
+
+
+def affine_grouped_data(n, k, gs, seed, interleave=False):
+    """Seeded codes / scales / zero points of `affine_grouped` and the exact
+    float32 weight (reference tests/test_qmm.py:991-1010: same draws)."""
+    rng = np.random.default_rng(seed)
+    ng = k // gs
+    q = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    scale = ((rng.random((n, ng)).astype(np.float32) + 0.5) * 0.05)
+    zero = rng.integers(-3, 4, size=(n, ng)).astype(np.int8)
+    g = (np.arange(k) % ng) if interleave else (np.arange(k) // gs)
+    ref = np.take(scale, g, axis=1) * (q.astype(np.float32) - np.take(zero, g, axis=1))
+    return q, scale, zero, ref
+
+
+def dense_mxfp4_rows(n, k, t, el="bf16"):
+    """dense_mxfp4 as jax lowers `jnp.take`: the E2M1 decode is a private
+    @_take callee (index wrap with full-extent splats, then a gather that
+    batches over the indices), and every op keeps N as the leading axis
+    (reference tests/test_qmm_mxfp4.py:282-298, :908-916)."""
+    h = k // 2
+    vals = ", ".join(("-" if np.signbit(v) else "") + f"{abs(v):.6e}"
+                     for v in np.array(list(E2M1) + [-v for v in E2M1], np.float64))
+    bl, sb = _t((n, h), "ui8"), _t((n, k // 32), "ui8")
+    idx, idx3 = _t((n, k), "i32"), _t((n, k, 1), "i32")
+    return f"""
+module @jit_dense_mxfp4_rows {{
+  func.func public @main(%blocks: {bl}, %scales: {sb}, %x: {_t((t, k), el)}) -> {_t((t, n), el)} {{
+    %vt = stablehlo.constant dense<[{vals}]> : tensor<16x{el}>
+    %stab = stablehlo.constant dense<"{_e8m0_table_hex()}"> : tensor<256xf32>
+    %m15s = stablehlo.constant dense<15> : tensor<ui8>
+    %m15 = stablehlo.broadcast_in_dim %m15s, dims = [] : (tensor<ui8>) -> {bl}
+    %s4s = stablehlo.constant dense<4> : tensor<ui8>
+    %s4 = stablehlo.broadcast_in_dim %s4s, dims = [] : (tensor<ui8>) -> {bl}
+    %lo = stablehlo.and %blocks, %m15 : {bl}
+    %hi = stablehlo.shift_right_logical %blocks, %s4 : {bl}
+    %lo3 = stablehlo.reshape %lo : ({bl}) -> {_t((n, h, 1), "ui8")}
+    %hi3 = stablehlo.reshape %hi : ({bl}) -> {_t((n, h, 1), "ui8")}
+    %nb = stablehlo.concatenate %lo3, %hi3, dim = 2 : ({_t((n, h, 1), "ui8")}, {_t((n, h, 1), "ui8")}) -> {_t((n, h, 2), "ui8")}
+    %nib = stablehlo.reshape %nb : ({_t((n, h, 2), "ui8")}) -> {_t((n, k), "ui8")}
+    %ni = stablehlo.convert %nib : ({_t((n, k), "ui8")}) -> {idx}
+    %v = func.call @_take(%vt, %ni) : (tensor<16x{el}>, {idx}) -> {_t((n, k), el)}
+    %sbi0 = stablehlo.convert %scales : ({sb}) -> {_t((n, k // 32), "i32")}
+    %sbi = stablehlo.reshape %sbi0 : ({_t((n, k // 32), "i32")}) -> {_t((n, k // 32, 1), "i32")}
+    %s32 = "stablehlo.gather"(%stab, %sbi) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1>}}> : (tensor<256xf32>, {_t((n, k // 32, 1), "i32")}) -> {_t((n, k // 32), "f32")}
+    %scd = stablehlo.convert %s32 : ({_t((n, k // 32), "f32")}) -> {_t((n, k // 32), el)}
+    %scb = stablehlo.broadcast_in_dim %scd, dims = [0, 1] : ({_t((n, k // 32), el)}) -> {_t((n, k // 32, 32), el)}
+    %v3 = stablehlo.reshape %v : ({_t((n, k), el)}) -> {_t((n, k // 32, 32), el)}
+    %w3 = stablehlo.multiply %v3, %scb : {_t((n, k // 32, 32), el)}
+    %wt = stablehlo.reshape %w3 : ({_t((n, k // 32, 32), el)}) -> {_t((n, k), el)}
+    %y = stablehlo.dot_general %x, %wt, contracting_dims = [1] x [1] : ({_t((t, k), el)}, {_t((n, k), el)}) -> {_t((t, n), el)}
+    return %y : {_t((t, n), el)}
+  }}
+  func.func private @_take(%table: tensor<16x{el}>, %i: {idx}) -> {_t((n, k), el)} {{
+    %zs = stablehlo.constant dense<0> : tensor<i32>
+    %z = stablehlo.broadcast_in_dim %zs, dims = [] : (tensor<i32>) -> {idx}
+    %ns = stablehlo.constant dense<16> : tensor<i32>
+    %nn = stablehlo.broadcast_in_dim %ns, dims = [] : (tensor<i32>) -> {idx}
+    %neg = stablehlo.compare LT, %i, %z, SIGNED : ({idx}, {idx}) -> {_t((n, k), "i1")}
+    %wrap = stablehlo.add %i, %nn : {idx}
+    %sel = stablehlo.select %neg, %wrap, %i : {_t((n, k), "i1")}, {idx}
+    %i3 = stablehlo.reshape %sel : ({idx}) -> {idx3}
+    %r = "stablehlo.gather"(%table, %i3) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1>}}> : (tensor<16x{el}>, {idx3}) -> {_t((n, k), el)}
+    return %r : {_t((n, k), el)}
+  }}
+}}
+"""

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import stablehlo_text as T
-from metaljax_amd import engine, interpreter as I, ir, packing, qmm
+from metaljax_amd import engine, interpreter as I, ir, packing, packs, qmm
 from oracle import qmm_oracle as O
 
 
@@ -156,11 +156,9 @@ def test_mxfp4_chain_packs_bit_exactly(el):
     lit = qmm._eval(ex.interp, st.matches[0].root.operands[1], env)
     np.testing.assert_array_equal(lit.a, w)
     qmm.prologue(ex.interp, args)
-    if el == "f32":
-        # float32 activations are outside what the kernels serve: the weight
-        # packs, the kernel check disables the dot
-        assert qmm.stats()["fallbacks"] == 1 and st.matches[0].disabled
-        return
+    # float32 chains are served like bf16 ones (the library splits float32
+    # activations into exact bf16 terms)
+    assert st.matches[0].act_dtype == el and not st.matches[0].disabled
     assert qmm.stats() == {**{k_: 0 for k_ in qmm.STATS}, "recognized": 1, "packs": 1, "mxfp4": 1}
     pk = st.matches[0].packs[0]
     np.testing.assert_array_equal(np.asarray(pk.w), O.pack_codes(codes, 4))
@@ -304,7 +302,7 @@ def test_packs_are_keyed_by_buffer_identity_and_repack_storms_give_up(monkeypatc
     qmm.prologue(ex.interp, args2)                          # new weight buffers: repack, no stale pack
     assert qmm.stats()["packs"] == 2 and ex.interp._qmm.matches[0].repacks == 2
     assert qmm.stats()["shared"] == 1                       # same bytes: the arrays are shared
-    monkeypatch.setattr(qmm, "_MAX_REPACKS", 3)
+    monkeypatch.setattr(packs, "MAX_REPACKS", 3)
     keep = []
     for i in range(3):
         keep.append(host_args_dense(packed.copy(), scale, zero, g_idx, x))
@@ -457,3 +455,127 @@ def test_engine_surface_is_what_the_pjrt_plugin_calls_by_name():
     assert isinstance(engine.device_kind(), str)
     ver = engine.stablehlo_version()
     assert len(ver) == 3 and all(type(v) is int for v in ver)
+
+
+# --------------------------------------------------- packing by row blocks ----
+
+def _packs_built(monkeypatch, text, args, block_elems):
+    """Pack `text`'s weights on fresh copies of `args` with a given block size;
+    returns (pack arrays, stats).  Both pack tables are cleared first: two
+    builds of one weight are identical and would otherwise alias each other,
+    and comparing an array with itself proves nothing."""
+    qmm._SHARED.clear()
+    qmm._BUILT.clear()
+    qmm.reset_stats()
+    monkeypatch.setattr(packs, "BLOCK_ELEMS", block_elems)
+    ex = engine.compile_program(text)
+    fresh = [I.HostArray(np.array(a.a, copy=True), a.el) for a in args]
+    qmm.prologue(ex.interp, fresh)
+    st = ex.interp._qmm
+    built = [[np.array(np.asarray(a.bits if isinstance(a, packing.BF16Array) else a)) for a in pk.arrays()]
+             for mt in st.matches for pk in mt.packs[:1]]
+    return built, qmm.stats(), st
+
+
+def _same_packs(a, b):
+    assert len(a) == len(b)
+    for pa, pb in zip(a, b):
+        assert len(pa) == len(pb)
+        for x, y in zip(pa, pb):
+            assert x.dtype == y.dtype and x.shape == y.shape
+            np.testing.assert_array_equal(x, y)
+
+
+def test_blocked_affine_pack_is_bit_identical(monkeypatch):
+    """Packing an affine weight by blocks of rows gives the bits a whole
+    evaluation gives: codes, scale and bias tables (reference
+    tests/test_qmm.py:1029-1057).  The codes are walked twice when blocked
+    (the offset is one number for the whole weight)."""
+    n, k, gs, t = 256, 128, 64, 3
+    q, scale, zero, ref = T.affine_grouped_data(n, k, gs, 21)
+    x = T.bf16_round(np.random.default_rng(22).standard_normal((t, k)).astype(np.float32) * 0.3)
+    args = [I.from_numpy(q), I.from_numpy(scale), I.from_numpy(zero), I.from_numpy(x, "bf16")]
+    text = T.affine_grouped(n, k, gs, t)
+    whole, st_w, _ = _packs_built(monkeypatch, text, args, 1 << 40)
+    small, st_b, state = _packs_built(monkeypatch, text, args, 1 << 10)     # 8 rows a block
+    assert st_w["packs"] == st_b["packs"] == 1 and st_w["fallbacks"] == st_b["fallbacks"] == 0
+    assert st_w["blocked"] == 0 and st_b["blocked"] == 1
+    assert state.matches[0].packs[0].blocked
+    _same_packs(whole, small)
+    pk = state.matches[0].packs[0]
+    assert (pk.gs, pk.bits, pk.perm) == (gs, 4, None)
+    # the packed weight is the graph's weight: scale * (q - zero) with bf16 scales
+    want = T.bf16_round(scale)[:, np.arange(k) // gs] * (q.astype(np.float32) - zero[:, np.arange(k) // gs])
+    np.testing.assert_allclose(dequant_pack(pk), want, rtol=1e-6, atol=1e-7)
+
+
+def test_blocked_affine_falls_back_when_groups_interleave(monkeypatch):
+    """Groups scattered along K: the permutation that gathers them is a
+    property of the whole contraction axis, so the blocked pass gives up and
+    the weight packs from a whole evaluation -- the same pack the unblocked
+    path builds (reference tests/test_qmm.py:1060-1090)."""
+    n, k, gs, t = 128, 128, 64, 2
+    q, scale, zero, ref = T.affine_grouped_data(n, k, gs, 23, interleave=True)
+    x = T.bf16_round(np.random.default_rng(24).standard_normal((t, k)).astype(np.float32) * 0.3)
+    args = [I.from_numpy(q), I.from_numpy(scale), I.from_numpy(zero), I.from_numpy(x, "bf16")]
+    text = T.affine_grouped(n, k, gs, t, interleave=True)
+    whole, st_w, _ = _packs_built(monkeypatch, text, args, 1 << 40)
+    small, st_b, state = _packs_built(monkeypatch, text, args, 1 << 10)
+    assert st_b["packs"] == 1 and st_b["blocked"] == 0 and st_b["perms"] == 1 and st_b["fallbacks"] == 0
+    assert st_w["perms"] == 1
+    _same_packs(whole, small)
+    assert state.matches[0].has_perm
+
+
+def test_blocked_mxfp4_pack_is_bit_identical_through_a_take_callee(monkeypatch):
+    """The E2M1 decode as jax lowers it -- a private @_take callee whose body
+    is declared for the full extent -- evaluated inside the callee, block by
+    block (reference tests/test_qmm_mxfp4.py:895-928)."""
+    n, k, t = 96, 128, 4
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=5)
+    x = T.bf16_round(np.random.default_rng(6).standard_normal((t, k)).astype(np.float32))
+    text = T.dense_mxfp4_rows(n, k, t)
+    assert "@_take" in text
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")]
+    whole, st_w, _ = _packs_built(monkeypatch, text, args, 1 << 40)
+    small, st_b, state = _packs_built(monkeypatch, text, args, 1 << 11)     # 16 rows a block
+    assert st_w["blocked"] == 0 and st_b["blocked"] == 1 and st_b["mxfp4"] == 1
+    _same_packs(whole, small)
+    pk = state.matches[0].packs[0]
+    np.testing.assert_array_equal(np.asarray(pk.w), O.pack_codes(codes, 4))
+    np.testing.assert_array_equal(np.asarray(pk.scales), sb)
+    # the literal run of the same module agrees with the exact weight
+    lit = I.host(I.Interpreter(text).run(args)[0]).a
+    np.testing.assert_allclose(lit, T.bf16_round(x @ w.T), rtol=2e-2, atol=1e-2 * np.abs(x @ w.T).max())
+
+
+def test_a_chain_that_is_not_row_local_packs_whole(monkeypatch):
+    """A reshape that folds N into other axes (the decode over a flat index
+    list) is not row-local: blocks are refused and the pack is the whole
+    evaluation's.  A weight stored K-first cannot be blocked by rows at all."""
+    n, k, t = 48, 128, 5
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=1)
+    x = T.bf16_round(np.random.default_rng(2).standard_normal((t, k)).astype(np.float32))
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")]
+    whole, _, _ = _packs_built(monkeypatch, T.dense_mxfp4(n, k, t), args, 1 << 40)
+    small, st_b, _ = _packs_built(monkeypatch, T.dense_mxfp4(n, k, t), args, 1 << 9)
+    assert st_b["packs"] == 1 and st_b["blocked"] == 0 and st_b["fallbacks"] == 0
+    _same_packs(whole, small)
+    kk, nn, m = 128, 64, 2
+    q, packed, scale, zero, g_idx, _ = T.quantize(kk, nn, 64)
+    ex = engine.compile_program(T.dense_sub(kk, nn, 2, m))
+    st = qmm.analyze(ex.interp)
+    monkeypatch.setattr(packs, "BLOCK_ELEMS", 1 << 8)
+    src = packs.WeightRows(ex.interp, st.matches[0], host_args_dense(packed, scale, zero, g_idx, np.zeros((m, kk), np.float32)))
+    assert not src.blocked() and src.blocks() == [(0, kk)]
+
+
+def test_block_size_comes_from_the_environment():
+    import os
+    import subprocess
+    import sys
+    ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = "from metaljax_amd import packs; print(packs.BLOCK_ELEMS)"
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True,
+                         env={**os.environ, "METALJAX_QMM_BLOCK": "4096"}, cwd=ROOT)
+    assert out.stdout.strip() == "4096", out.stderr
