@@ -504,6 +504,32 @@ def _reduce(interp, op, ins, env):
     return settle(fn(src, axis=dims), el)
 
 
+def top_k(a: np.ndarray, k: int):
+    """(values, int32 indices) of the k largest entries along the last axis,
+    largest first, equal values in index order."""
+    order = np.argsort(-a, axis=-1, kind="stable")[..., :k]
+    return np.take_along_axis(a, order, axis=-1), order.astype(np.int32)
+
+
+@register("chlo.top_k")
+def _top_k(interp, op, ins, env):
+    a = host(ins[0])
+    k = op.attrs.get("k", op.results[0].type.shape[-1])
+    vals, idx = top_k(a.a.astype(np.float32 if a.el in ("bf16", "f16") else a.a.dtype), k)
+    return [settle(vals, op.results[0].type.el), settle(idx, op.results[1].type.el)]
+
+
+@register("stablehlo.composite")
+def _composite(interp, op, ins, env):
+    """A composite runs as what it names when that is known here (a top-k
+    arrives wrapped like this after a portable-artifact round trip), else as
+    its decomposition."""
+    if op.attrs.get("name") == "chlo.top_k":
+        return _top_k(interp, op, ins, env)
+    f = interp.module.funcs[str(op.attrs["decomposition"]).lstrip("@")]
+    return interp.run_block(f.body, dict(zip(f.body.args, ins)))
+
+
 @register("func.call")
 def _call(interp, op, ins, env):
     f = interp.module.funcs[op.attrs["callee"]]

@@ -527,6 +527,19 @@ class _Parser:
             self.expect("punct", ")")
             _, outs = self.fn_type()
             return Op("func.call", operands, outs, {"callee": callee}, [])
+        if name == "chlo.top_k":
+            # `chlo.top_k(%x, k = 2) : tensor<..> -> (tensor<..>, tensor<..>)`
+            self.expect("punct", "(")
+            operands = [self.lookup(self.expect("ssa")[1])]
+            self.expect("punct", ",")
+            self.expect("id", "k")
+            self.expect("punct", "=")
+            k = int(self.expect("num")[1])
+            self.expect("punct", ")")
+            self.expect("punct", ":")
+            self.type_()
+            self.expect("arrow")
+            return Op(name, operands, self.type_list(), {"k": k}, [])
         if not name.startswith("stablehlo."):
             return self.opaque_op(name)
         if short == "constant":

@@ -128,24 +128,34 @@ def grouped_qmm(x, w, scales, biases, row_offsets, group_size=64, bits=4, mode="
 
 def gather_qmm(x, w, scales, biases=None, lhs_indices=None, rhs_indices=None, transpose=True,
                group_size=64, bits=4, mode="affine", out_dtype=None):
-    """y[p] = x[lhs_indices[p]] @ dequant(w[rhs_indices[p]])^T, one row per pair.
+    """y[p] = x[lhs_indices[p]] @ dequant(w[rhs_indices[p]])^T for every pair p.
 
-    x [T,K] (or [T,1,K]); w [E,N,...]; indices int32 [P] in any order.
-    Returns [P,N] (or [P,1,N] when x was 3-D), like mx.gather_qmm with M=1.
+    x [T,K] -> y [P,N], or x [T,M,K] (M activation rows per entry, as
+    mx.gather_qmm takes it, reference src/metaljax/moe.py:1293-1301) ->
+    y [P,M,N]; w [E,N,...]; indices int32 [P] in any order; lhs_indices None
+    means pair p reads entry p.  With M rows per entry every pair becomes M
+    one-row pairs of the same expert (rows lhs*M .. lhs*M + M - 1 of the
+    flattened activations), which is what the library multiplies.
     """
     if not transpose:
         raise UnsupportedQmm(3, "only transpose=True is built")
     _need_cuda(x, w, scales, biases, lhs_indices, rhs_indices)
     lib = _lib.load()
-    three_d = x.dim() == 3
-    if three_d:
-        if x.shape[1] != 1:
-            raise UnsupportedQmm(3, "gather_qmm serves one activation row per pair")
-        x = x[:, 0]
     (e,), n, k = _weight_dims(w, bits, mode)
-    t = x.shape[0]
     rhs = rhs_indices.to(torch.int32).contiguous()
     lhs = None if lhs_indices is None else lhs_indices.to(torch.int32).contiguous()
+    rows, with_rows = 1, x.dim() == 3
+    if with_rows:
+        rows = x.shape[1]
+        x = x.reshape(x.shape[0] * rows, x.shape[2])
+        if rows > 1:
+            step = torch.arange(rows, device=rhs.device, dtype=torch.int32)
+            first = (torch.arange(rhs.numel(), device=rhs.device, dtype=torch.int32) if lhs is None else lhs) * rows
+            lhs = (first[:, None] + step[None, :]).reshape(-1).contiguous()
+            rhs = rhs.repeat_interleave(rows).contiguous()
+    elif x.dim() != 2:
+        raise _lib.QmmError(2, f"x must be [T, K] or [T, M, K], got {tuple(x.shape)}")
+    t = x.shape[0]
     p = rhs.numel()
     out_dtype = out_dtype or x.dtype
     y = torch.empty((p, n), dtype=out_dtype, device=x.device)
@@ -158,7 +168,7 @@ def gather_qmm(x, w, scales, biases=None, lhs_indices=None, rhs_indices=None, tr
                             _ptr(y), _dt(out_dtype), _ptr(lhs), _ptr(rhs), p, t, e, n, k,
                             group_size, bits, _MODE[mode], _ptr(ws), nbytes, _stream(x))
     _lib.check(rc)
-    return y[:, None, :] if three_d else y
+    return y.reshape(p // rows, rows, n) if with_rows else y
 
 
 def dequantize(w, scales, biases=None, group_size=64, bits=4, mode="affine",

@@ -168,9 +168,10 @@ def prologue(interp, args) -> bool:
         arrays = pk.arrays()
         m.slot, m.nvals = len(layout), len(arrays)
         layout += arrays
-    for dispatch in st.moe:
-        if not dispatch.disabled and dispatch.match.disabled:
-            dispatch.disabled = rewrite_changed = True      # its expert weight runs literally: so does the dispatch
+    if st.moe:
+        from . import moe
+        if moe.prologue(interp, st):            # a dispatch whose weight did not pack, or that fails its check, runs densely
+            rewrite_changed = True
     if rewrite_changed:
         st.rebuild()
         interp.invalidate_plans()
@@ -242,7 +243,10 @@ def to_device(v):
     if h.el == "bf16":
         bits = packing.f32_to_bf16_bits(h.a).view(np.int16)
         return torch.from_numpy(np.ascontiguousarray(bits)).cuda().view(torch.bfloat16)
-    return torch.from_numpy(np.ascontiguousarray(h.a)).cuda()
+    a = np.ascontiguousarray(h.a)
+    if not a.flags.writeable:                   # torch refuses to wrap read-only storage without a warning
+        a = a.copy()
+    return torch.from_numpy(a).cuda()
 
 
 def emit(interp, m, env):

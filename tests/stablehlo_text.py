@@ -369,3 +369,124 @@ module @jit_dense_mxfp4_rows {{
   }}
 }}
 """
+
+
+# ------------------------------------------------- a dense MoE dispatch ----
+
+def _tagged_mxfp4_weight(tag, blocks, scales, lead, n, k, el):
+    """`_mxfp4_weight` with every SSA name suffixed by `tag` and the two
+    inputs named `blocks` / `scales`: defines %wt<tag> [lead.., N, K]."""
+    import re
+    text = _mxfp4_weight(lead, n, k, el)
+    text = text.replace("%blocks", "%BLOCKS").replace("%scales", "%SCALES")
+    text = re.sub(r"%([a-z][a-z0-9]*)\b", lambda mo: f"%{mo.group(1)}{tag}", text)
+    return text.replace("%BLOCKS", blocks).replace("%SCALES", scales)
+
+
+def moe_block_mxfp4(E, T, H, I, K, el="f32", composite=False):
+    """The gpt-oss expert block as the reference's test writes it (reference
+    tests/test_moe.py:60-66, :500-511): every expert runs on every token,
+
+        gu   = einsum("th,emh->etm", x, Wgu) + bgu        Wgu MXFP4 [E, 2I, H]
+        act  = (clip(up) + 1) * (g * sigmoid(1.702 g)),   g = clip(gate); gate / up = gu[..., 0::2] / [..., 1::2]
+        y    = einsum("etm,ehm->eth", act, Wd) + bd       Wd MXFP4 [E, H, I]
+        out  = sum_e y[e] * S[:, e],  S = sum_k one_hot(idx) * softmax(top_k values)
+
+    `composite`: the top-k as a stablehlo.composite (what reaches a plugin)."""
+    f = el
+    tk = ((f'%tk:2 = stablehlo.composite "chlo.top_k" %logits {{composite_attributes = {{k = {K} : i64}}, '
+           f'decomposition = @chlo.top_k.impl, version = 1 : i32}} : ({_t((T, E), f)}) -> '
+           f'({_t((T, K), f)}, {_t((T, K), "i32")})\n    %vals = stablehlo.convert %tk#0 : ({_t((T, K), f)}) -> {_t((T, K), f)}\n'
+           f'    %idx = stablehlo.convert %tk#1 : ({_t((T, K), "i32")}) -> {_t((T, K), "i32")}')
+          if composite else
+          f'%vals, %idx = chlo.top_k(%logits, k = {K}) : {_t((T, E), f)} -> ({_t((T, K), f)}, {_t((T, K), "i32")})')
+    etm, eti, eth = _t((E, T, 2 * I), f), _t((E, T, I), f), _t((E, T, H), f)
+    tke = (T, K, E)
+    return f"""
+module @jit_moe_block {{
+  func.func public @main(%x: {_t((T, H), f)}, %wr: {_t((H, E), f)}, %br: {_t((E,), f)}, %guc: {_t((E, 2 * I, H // 2), "ui8")}, %gus: {_t((E, 2 * I, H // 32), "ui8")}, %dc: {_t((E, H, I // 2), "ui8")}, %ds: {_t((E, H, I // 32), "ui8")}, %bgu: {_t((E, 2 * I), f)}, %bd: {_t((E, H), f)}) -> {_t((T, H), f)} {{{_tagged_mxfp4_weight("g", "%guc", "%gus", (E,), 2 * I, H, f)}{_tagged_mxfp4_weight("d", "%dc", "%ds", (E,), H, I, f)}
+    %zero = stablehlo.constant dense<0.000000e+00> : tensor<{f}>
+    %ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>
+    %gu0 = stablehlo.dot_general %x, %wtg, contracting_dims = [1] x [2] : ({_t((T, H), f)}, {_t((E, 2 * I, H), f)}) -> {_t((T, E, 2 * I), f)}
+    %gu1 = stablehlo.transpose %gu0, dims = [1, 0, 2] : ({_t((T, E, 2 * I), f)}) -> {etm}
+    %bgub = stablehlo.broadcast_in_dim %bgu, dims = [0, 2] : ({_t((E, 2 * I), f)}) -> {etm}
+    %gu = stablehlo.add %gu1, %bgub : {etm}
+    %gate0 = stablehlo.slice %gu [0:{E}, 0:{T}, 0:{2 * I}:2] : ({etm}) -> {eti}
+    %up0 = stablehlo.slice %gu [0:{E}, 0:{T}, 1:{2 * I}:2] : ({etm}) -> {eti}
+    %big = stablehlo.constant dense<-1.000000e+09> : tensor<{f}>
+    %p7 = stablehlo.constant dense<7.000000e+00> : tensor<{f}>
+    %m7 = stablehlo.constant dense<-7.000000e+00> : tensor<{f}>
+    %gate = stablehlo.clamp %big, %gate0, %p7 : (tensor<{f}>, {eti}, tensor<{f}>) -> {eti}
+    %up = stablehlo.clamp %m7, %up0, %p7 : (tensor<{f}>, {eti}, tensor<{f}>) -> {eti}
+    %c17s = stablehlo.constant dense<1.702000e+00> : tensor<{f}>
+    %c17 = stablehlo.broadcast_in_dim %c17s, dims = [] : (tensor<{f}>) -> {eti}
+    %ones = stablehlo.constant dense<1.000000e+00> : tensor<{f}>
+    %one = stablehlo.broadcast_in_dim %ones, dims = [] : (tensor<{f}>) -> {eti}
+    %ga = stablehlo.multiply %gate, %c17 : {eti}
+    %sg = stablehlo.logistic %ga : {eti}
+    %glu = stablehlo.multiply %gate, %sg : {eti}
+    %up1 = stablehlo.add %up, %one : {eti}
+    %act = stablehlo.multiply %up1, %glu : {eti}
+    %y0 = stablehlo.dot_general %act, %wtd, batching_dims = [0] x [0], contracting_dims = [2] x [2] : ({eti}, {_t((E, H, I), f)}) -> {eth}
+    %bdb = stablehlo.broadcast_in_dim %bd, dims = [0, 2] : ({_t((E, H), f)}) -> {eth}
+    %y = stablehlo.add %y0, %bdb : {eth}
+    %lg = stablehlo.dot_general %x, %wr, contracting_dims = [1] x [0] : ({_t((T, H), f)}, {_t((H, E), f)}) -> {_t((T, E), f)}
+    %brb = stablehlo.broadcast_in_dim %br, dims = [1] : ({_t((E,), f)}) -> {_t((T, E), f)}
+    %logits = stablehlo.add %lg, %brb : {_t((T, E), f)}
+    {tk}
+    %v32 = stablehlo.convert %vals : ({_t((T, K), f)}) -> {_t((T, K), "f32")}
+    %mx = stablehlo.reduce(%v32 init: %ninf) applies stablehlo.maximum across dimensions = [1] : ({_t((T, K), "f32")}, tensor<f32>) -> {_t((T,), "f32")}
+    %mxb = stablehlo.broadcast_in_dim %mx, dims = [0] : ({_t((T,), "f32")}) -> {_t((T, K), "f32")}
+    %sh = stablehlo.subtract %v32, %mxb : {_t((T, K), "f32")}
+    %ex = stablehlo.exponential %sh : {_t((T, K), "f32")}
+    %z32 = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+    %sm = stablehlo.reduce(%ex init: %z32) applies stablehlo.add across dimensions = [1] : ({_t((T, K), "f32")}, tensor<f32>) -> {_t((T,), "f32")}
+    %smb = stablehlo.broadcast_in_dim %sm, dims = [0] : ({_t((T,), "f32")}) -> {_t((T, K), "f32")}
+    %w32 = stablehlo.divide %ex, %smb : {_t((T, K), "f32")}
+    %w = stablehlo.convert %w32 : ({_t((T, K), "f32")}) -> {_t((T, K), f)}
+    %idxb = stablehlo.broadcast_in_dim %idx, dims = [0, 1] : ({_t((T, K), "i32")}) -> {_t(tke, "i32")}
+    %io = stablehlo.iota dim = 2 : {_t(tke, "i32")}
+    %eq = stablehlo.compare EQ, %idxb, %io, SIGNED : ({_t(tke, "i32")}, {_t(tke, "i32")}) -> {_t(tke, "i1")}
+    %hot = stablehlo.convert %eq : ({_t(tke, "i1")}) -> {_t(tke, f)}
+    %wb = stablehlo.broadcast_in_dim %w, dims = [0, 1] : ({_t((T, K), f)}) -> {_t(tke, f)}
+    %hw = stablehlo.multiply %hot, %wb : {_t(tke, f)}
+    %s = stablehlo.reduce(%hw init: %zero) applies stablehlo.add across dimensions = [1] : ({_t(tke, f)}, tensor<{f}>) -> {_t((T, E), f)}
+    %st = stablehlo.transpose %s, dims = [1, 0] : ({_t((T, E), f)}) -> {_t((E, T), f)}
+    %sb = stablehlo.broadcast_in_dim %st, dims = [0, 1] : ({_t((E, T), f)}) -> {eth}
+    %ys = stablehlo.multiply %y, %sb : {eth}
+    %out = stablehlo.reduce(%ys init: %zero) applies stablehlo.add across dimensions = [0] : ({eth}, tensor<{f}>) -> {_t((T, H), f)}
+    return %out : {_t((T, H), f)}
+  }}
+}}
+"""
+
+
+def make_mxfp4_experts(rows, k, E, seed):
+    """([E, rows, k/2] packed codes, [E, rows, k/32] E8M0 bytes, the exact
+    float32 weight) -- the generator of reference tests/test_moe.py:487-497."""
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 16, size=(E, rows, k)).astype(np.uint8)
+    exps = rng.integers(120, 128, size=(E, rows, k // 32)).astype(np.uint8)
+    packed = (codes[..., 0::2] | (codes[..., 1::2] << 4)).astype(np.uint8)
+    grid = np.array(list(E2M1) + [-v for v in E2M1], np.float32)
+    scale = np.exp2(exps.astype(np.float32) - 127.0)
+    ref = (grid[codes].reshape(E, rows, k // 32, 32) * scale[..., None]).reshape(E, rows, k)
+    return packed, exps, ref.astype(np.float32)
+
+
+def moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd, k):
+    """The block on exactly dequantized weights, in float64 numpy."""
+    x, wr, br, bgu, bd = (np.asarray(a, np.float64) for a in (x, wr, br, bgu, bd))
+    gu = np.einsum("th,emh->etm", x, gu_ref.astype(np.float64)) + bgu[:, None, :]
+    gate = np.clip(gu[..., ::2], -1e9, 7.0)
+    up = np.clip(gu[..., 1::2], -7.0, 7.0)
+    act = (up + 1) * (gate / (1.0 + np.exp(-1.702 * gate)))
+    y = np.einsum("etm,ehm->eth", act, d_ref.astype(np.float64)) + bd[:, None, :]
+    logits = (x @ wr + br).astype(np.float32)
+    order = np.argsort(-logits, axis=-1, kind="stable")[:, :k]
+    vals = np.take_along_axis(logits, order, -1).astype(np.float64)
+    w = np.exp(vals - vals.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    s = np.zeros_like(logits, dtype=np.float64)
+    np.put_along_axis(s, order, w, -1)
+    return np.einsum("eth,te->th", y, s)

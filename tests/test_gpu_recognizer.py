@@ -132,8 +132,6 @@ def test_gathered_expert_dispatch_over_a_recognized_pack():
     st = qmm.analyze(ex.interp)
     qmm.prologue(ex.interp, [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(xe, "bf16")])
     mt = st.matches[0]
-    dot = moe.Dot(mt)
-    assert mt.absorbed
     rng = np.random.default_rng(5)
     x = T.bf16_round(rng.standard_normal((t, k)).astype(np.float32))
     logits = rng.standard_normal((t, e)).astype(np.float32)
@@ -142,12 +140,78 @@ def test_gathered_expert_dispatch_over_a_recognized_pack():
     p = p / p.sum(1, keepdims=True)
     wts = np.take_along_axis(p, idx, 1)
     xd = qmm.to_device(I.from_numpy(x, "bf16"))
-    y = moe.expert_dispatch(ex.interp, dot.match, xd, torch.from_numpy(idx).cuda(),
+    y = moe.expert_dispatch(ex.interp, mt, xd, torch.from_numpy(idx).cuda(),
                             torch.from_numpy(wts).cuda())
     want = np.zeros((t, n), np.float32)
     for i in range(t):
         for j in range(topk):
             want[i] += wts[i, j] * (x[i] @ w[idx[i, j]].T)
     got = y.float().cpu().numpy()
-    assert moe.stats() == {"gather_qmm": 1, "dispatches": 1}
+    assert moe.stats()["gather_qmm"] == 1 and moe.stats()["dispatches"] == 1
     assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-2
+
+
+
+@pytest.mark.parametrize("E,K", [(4, 2), (8, 4)])
+@pytest.mark.parametrize("Tk", [1, 3])
+def test_mxfp4_experts_gathered(E, K, Tk):
+    """The gpt-oss block end to end (reference tests/test_moe.py:514-557):
+    the dense dispatch is recognized, both projections run as expert-indexed
+    quantized products on the device, the routing-weighted sum follows there,
+    and the result matches the dense block on exactly dequantized weights
+    (float32 graph: rtol 3e-5) and the literal run of the same module."""
+    import stablehlo_text as S
+    moe.reset_stats()
+    H, Ii = 64, 32
+    rng = np.random.default_rng(E)
+    gu_c, gu_s, gu_ref = S.make_mxfp4_experts(2 * Ii, H, E, seed=E)
+    d_c, d_s, d_ref = S.make_mxfp4_experts(H, Ii, E, seed=E + 1)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    wr = (rng.standard_normal((H, E)) / 8).astype(np.float32)
+    br = rng.standard_normal(E).astype(np.float32)
+    bgu = (rng.standard_normal((E, 2 * Ii)) / 8).astype(np.float32)
+    bd = (rng.standard_normal((E, H)) / 8).astype(np.float32)
+    text = S.moe_block_mxfp4(E, Tk, H, Ii, K)
+    args = [I.from_numpy(a) for a in (x, wr, br, gu_c, gu_s, d_c, d_s, bgu, bd)]
+    ex = engine.compile_program(text)
+    (buf,) = engine.execute(ex, args)
+    st, qst = moe.stats(), qmm.stats()
+    assert st["recognized"] == 1 and st["verified"] == 1 and st["fallbacks"] == 0, st
+    assert st["gather_qmm"] >= 2 and st["dispatches"] == 1, st       # both projections read packs
+    assert qst["mxfp4"] == 2 and qst["fallbacks"] == 0, qst
+    assert isinstance(buf.data, torch.Tensor) and buf.data.is_cuda
+    got = buf.data.float().cpu().numpy()
+    want = S.moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd, K)
+    np.testing.assert_allclose(got, want, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+    lit = I.host(I.Interpreter(text).run(args)[0]).a
+    np.testing.assert_allclose(got, lit, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+    # a second execute on the same buffers packs nothing new
+    engine.execute(ex, args)
+    assert qmm.stats()["packs"] == 2 and moe.stats()["dispatches"] == 2
+
+
+def test_gather_qmm_with_several_rows_per_pair():
+    """x [T, M, K]: every pair multiplies M rows (mx.gather_qmm's general
+    form, reference src/metaljax/moe.py:1293-1301)."""
+    from metaljax_amd import kernels as K
+    from oracle import qmm_oracle as O
+    rng = np.random.default_rng(3)
+    e, n, k, t, m, pairs = 3, 72, 256, 5, 4, 7
+    codes = rng.integers(0, 16, size=(e, n, k), dtype=np.uint8)
+    words = O.pack_codes(codes, 4)
+    s = O.round_bf16(rng.uniform(0.005, 0.02, (e, n, k // 64)).astype(np.float32))
+    b = O.round_bf16(-8 * s)
+    x = O.round_bf16(rng.standard_normal((t, m, k)).astype(np.float32))
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    dev = lambda a: torch.from_numpy(O.f32_to_bf16_bits(a).view(np.int16)).cuda().view(torch.bfloat16)
+    y = K.gather_qmm(dev(x), torch.from_numpy(words.view(np.int32)).cuda(), dev(s), dev(b),
+                     torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), group_size=64, bits=4,
+                     out_dtype=torch.float32)
+    assert tuple(y.shape) == (pairs, m, n)
+    want = O.gather_qmm(x, words, s, b, lhs, rhs, 64, 4)
+    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-5
+    y0 = K.gather_qmm(dev(x[:pairs]), torch.from_numpy(words.view(np.int32)).cuda(), dev(s), dev(b), None,
+                      torch.from_numpy(rhs[:t]).cuda(), group_size=64, bits=4, out_dtype=torch.float32)
+    want0 = O.gather_qmm(x, words, s, b, np.arange(t), rhs[:t], 64, 4)
+    assert O.rel_l2(y0.cpu().numpy(), want0) <= 2e-5

@@ -579,3 +579,103 @@ def test_block_size_comes_from_the_environment():
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True,
                          env={**os.environ, "METALJAX_QMM_BLOCK": "4096"}, cwd=ROOT)
     assert out.stdout.strip() == "4096", out.stderr
+
+
+# ------------------------------------------------------- expert dispatch ----
+
+def _moe_inputs(E, T, H, Ii, seed=None):
+    rng = np.random.default_rng(E if seed is None else seed)
+    gu_c, gu_s, gu_ref = T_.make_mxfp4_experts(2 * Ii, H, E, seed=E)
+    d_c, d_s, d_ref = T_.make_mxfp4_experts(H, Ii, E, seed=E + 1)
+    x = (rng.standard_normal((T, H)) / 8).astype(np.float32)
+    wr = (rng.standard_normal((H, E)) / 8).astype(np.float32)
+    br = rng.standard_normal(E).astype(np.float32)
+    bgu = (rng.standard_normal((E, 2 * Ii)) / 8).astype(np.float32)
+    bd = (rng.standard_normal((E, H)) / 8).astype(np.float32)
+    return (x, wr, br, gu_c, gu_s, d_c, d_s, bgu, bd), (gu_ref, d_ref)
+
+
+T_ = T
+
+
+@pytest.mark.parametrize("composite", [False, True])
+def test_dense_moe_block_is_planned_over_pairs(composite):
+    """The gpt-oss block (reference tests/test_moe.py:500-557): one dispatch,
+    both expert projections read quantized packs, the router is proven and
+    checked on synthetic logits, and the dense [tokens, experts] scores and
+    their one-hot are no longer computed."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    ex = engine.compile_program(T.moe_block_mxfp4(E, Tk, H, Ii, K, composite=composite))
+    st = qmm.analyze(ex.interp)
+    assert [m.mode for m in st.matches] == ["mxfp4", "mxfp4"] and all(m.absorbed for m in st.matches)
+    assert len(st.moe) == 1 and moe.stats()["recognized"] == 1
+    g = st.moe[0]
+    assert (g.E, g.T, g.K, g.P, g.out_shape) == (E, Tk, K, Tk * K, [Tk, H])
+    assert g.matches == st.matches and g.plan.dots == 2
+    r = g.router
+    assert r.indices.type.shape == (Tk, K) and r.weights.type.shape == (Tk, K) and moe.is_top_k(r.top_k)
+    # the rewrite: the root is the dispatch, the dots and the router's dense tail are skipped
+    assert st.roots == {g.key: g}
+    names = {k.op.name for k in g.skip_keys}
+    assert {"stablehlo.dot_general", "stablehlo.compare", "stablehlo.iota", "stablehlo.logistic"} <= names
+    by_name = {v.name: v for b in ir.walk_blocks(ex.interp.main.body) for o in b.ops for v in o.results}
+    assert by_name["s"] in g.skip_keys and by_name["hw"] in g.skip_keys          # scores and one-hot product
+    assert by_name["w"] not in g.skip_keys and by_name["logits"] not in g.skip_keys
+    assert set(qmm.emit_reads(g)) >= {r.indices, r.weights, by_name["bd"] if "bd" in by_name else r.weights}
+    args, _ = _moe_inputs(E, Tk, H, Ii)
+    changed = qmm.prologue(ex.interp, [I.from_numpy(a) for a in args])
+    assert changed is False and moe.stats()["verified"] == 1 and moe.stats()["fallbacks"] == 0
+    assert qmm.stats()["mxfp4"] == 2 and qmm.stats()["packs"] == 2
+
+
+def test_a_router_that_is_not_a_top_k_scatter_is_refused():
+    from metaljax_amd import moe
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    # the one-hot compares with LT instead of EQ: not a scatter of the selection
+    bad = text.replace("stablehlo.compare EQ, %idxb, %io", "stablehlo.compare LT, %idxb, %io")
+    ex = engine.compile_program(bad)
+    st = qmm.analyze(ex.interp)
+    assert st.moe == [] and not any(m.absorbed for m in st.matches) and len(st.roots) == 2
+    # the expert outputs are also returned: a region value read outside the region
+    shared = text.replace("-> tensor<3x64xf32> {", "-> (tensor<3x64xf32>, tensor<4x3x64xf32>) {", 1).replace(
+        "return %out : tensor<3x64xf32>", "return %out, %y : tensor<3x64xf32>, tensor<4x3x64xf32>")
+    st = qmm.analyze(engine.compile_program(shared).interp)
+    assert st.moe == []
+
+
+def test_a_dispatch_that_fails_its_check_runs_densely(monkeypatch):
+    """Verification closes a structurally accepted but wrong reading: here the
+    check itself is made to fail, and the dispatch is disabled, its matches
+    emit their own dense products again."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    E, Tk, H, Ii, K = 4, 1, 64, 32, 2          # one token: the decode step
+    ex = engine.compile_program(T.moe_block_mxfp4(E, Tk, H, Ii, K))
+    st = qmm.analyze(ex.interp)
+    assert len(st.moe) == 1
+
+    def broken(interp, g):
+        raise moe.Reject("scores differ")
+    monkeypatch.setattr(moe, "verify", broken)
+    args, _ = _moe_inputs(E, Tk, H, Ii)
+    assert qmm.prologue(ex.interp, [I.from_numpy(a) for a in args]) is True
+    assert st.moe[0].disabled and moe.stats()["fallbacks"] == 1
+    assert not any(m.absorbed for m in st.matches) and set(st.roots) == {m.key for m in st.matches}
+
+
+def test_router_check_catches_a_misplaced_weight(monkeypatch):
+    """`verify` compares the evaluated scores with the scatter of the matched
+    weights at the matched indices: a router record pointing at other weights
+    (what a misread axis would amount to) fails it."""
+    from metaljax_amd import moe
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    ex = engine.compile_program(T.moe_block_mxfp4(E, Tk, H, Ii, K))
+    g = qmm.analyze(ex.interp).moe[0]
+    moe.verify(ex.interp, g)                               # the true reading passes
+    by_name = {v.name: v for o in ex.interp.main.body.ops for v in o.results}
+    g.router.weights = by_name["ex"]                       # un-normalised exponentials
+    with pytest.raises(moe.Reject):
+        moe.verify(ex.interp, g)
