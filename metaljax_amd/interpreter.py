@@ -460,14 +460,73 @@ def _gather(interp, op, ins, env):
     return HostArray(out.reshape(_ty(op).shape), operand.el)
 
 
+# ---- the literal dot on the device -----------------------------------------
+# A dot the recognizer left alone (or gave back) still belongs on the GPU when
+# there is one, as in the reference, whose literal dot is a device matmul
+# (reference src/metaljax/ops/linalg.py:91-142): operands widened to float32,
+# one library matmul (float32 accumulate), one rounding to the result type.
+_DEVICE_DOT_ELS = {"bf16": "bfloat16", "f16": "float16", "f32": "float32"}
+_DEVICE_DOT_MIN_MACS = 1 << 22         # below this the copies cost more than the product
+
+
+def _device_dot_pays(ins, lc, ty) -> bool:
+    """Is there a GPU, and is the product large enough (or an operand already
+    there) for the device to be the place to run it?"""
+    try:
+        import torch
+    except ImportError:
+        return False
+    if not torch.cuda.is_available():
+        return False
+    if any(isinstance(x, torch.Tensor) and x.is_cuda for x in ins):
+        return True
+    a = ins[0]
+    shape = tuple(a.shape) if isinstance(a, torch.Tensor) else host(a).a.shape
+    k = 1
+    for d in lc:
+        k *= shape[d]
+    return ty.size * k >= _DEVICE_DOT_MIN_MACS
+
+
+def _as_device_f32(v):
+    import torch
+    if isinstance(v, torch.Tensor):
+        return v.cuda().float()
+    h = host(v)
+    return torch.from_numpy(np.array(h.a, dtype=np.float32)).cuda()
+
+
+def _dot_general_device(ins, lb, rb, lc, rc, ty):
+    import torch
+    A, B = _as_device_f32(ins[0]), _as_device_f32(ins[1])
+    af = [d for d in range(A.dim()) if d not in lb and d not in lc]
+    bf = [d for d in range(B.dim()) if d not in rb and d not in rc]
+    A = A.permute(lb + af + lc)
+    B = B.permute(rb + bf + rc)
+    nb = len(lb)
+    bs = tuple(A.shape[:nb])
+    k = 1
+    for d in A.shape[nb + len(af):]:
+        k *= d
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        out = torch.matmul(A.reshape(bs + (-1, k)), B.reshape(bs + (-1, k)).transpose(-1, -2))
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    return out.reshape(tuple(ty.shape)).to(getattr(torch, _DEVICE_DOT_ELS[ty.el]))
+
+
 @register("stablehlo.dot_general")
 def _dot_general(interp, op, ins, env):
     """The literal dot: operands widened to float32 (float64 for f64), product
     accumulated there, one rounding to the result type (reference
     src/metaljax/ops/linalg.py:91-142)."""
-    a, b = host(ins[0]), host(ins[1])
     lb, rb, lc, rc = ir.dot_dims(op)
     ty = _ty(op)
+    if ty.el in _DEVICE_DOT_ELS and _device_dot_pays(ins, lc, ty):
+        return _dot_general_device(ins, lb, rb, lc, rc, ty)
+    a, b = host(ins[0]), host(ins[1])
     ct = np.float64 if ty.el == "f64" else (np.float32 if is_float(ty.el) else np.int64)
     A, B = a.a.astype(ct), b.a.astype(ct)
     af = [d for d in range(A.ndim) if d not in lb and d not in lc]

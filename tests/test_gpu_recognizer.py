@@ -215,3 +215,23 @@ def test_gather_qmm_with_several_rows_per_pair():
                       torch.from_numpy(rhs[:t]).cuda(), group_size=64, bits=4, out_dtype=torch.float32)
     want0 = O.gather_qmm(x, words, s, b, np.arange(t), rhs[:t], 64, 4)
     assert O.rel_l2(y0.cpu().numpy(), want0) <= 2e-5
+
+
+def test_a_dot_left_to_the_interpreter_runs_on_the_device():
+    """A dot that is not rewritten (here: an ordinary float projection) is one
+    library matmul on the GPU, float32 accumulate, rounded once to the result
+    type -- the literal dot of reference src/metaljax/ops/linalg.py:91-142."""
+    k, n, m = 512, 384, 64
+    rng = np.random.default_rng(9)
+    w = T.bf16_round(rng.standard_normal((k, n)).astype(np.float32))
+    r = T.bf16_round(rng.standard_normal((k,)).astype(np.float32))
+    x = T.bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    ex = engine.compile_program(T.float_dot(k, n, m))
+    (buf,) = engine.execute(ex, [I.from_numpy(w, "bf16"), I.from_numpy(r, "bf16"), I.from_numpy(x, "bf16")])
+    assert qmm.stats()["recognized"] == 0
+    assert isinstance(buf.data, torch.Tensor) and buf.data.is_cuda and buf.data.dtype == torch.bfloat16
+    want = x.astype(np.float64) @ T.bf16_round(w * r[:, None]).astype(np.float64)
+    got = buf.data.float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2 * np.abs(want).max())
+    from metaljax_amd.packing import f32_to_bf16_bits
+    assert engine.to_host(buf) == f32_to_bf16_bits(got).tobytes()
