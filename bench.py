@@ -119,27 +119,52 @@ def bench_decode_random(m, n, k, bits=4, mode="affine", tables="bf16", steps=200
             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
 
-def bench_once(cfg, steps=20, warmup=3):
-    """A short timing of one of the other named shapes (weights are reused, so
-    they may sit in the last-level cache; these shapes are compute-bound)."""
+def _rel_l2(got, want):
+    import numpy as np
+    d = np.linalg.norm(got.astype(np.float64) - want.astype(np.float64))
+    return float(d / max(np.linalg.norm(want.astype(np.float64)), 1e-30))
+
+
+def oracle_check(wl, y, exact_weight):
+    """rel-L2 of one output of a timed leg against the C oracle, outside the
+    timed region.  `exact_weight`: against the exactly reconstructed weight,
+    else against the weight tile rounded once to bf16 (what the prefill kernels
+    stage)."""
+    from oracle import c_oracle as C
+    if wl.row_offsets is not None:
+        want = C.grouped_qmm(wl.x, wl.w, wl.scales, wl.biases, wl.row_offsets, wl.group_size, wl.bits,
+                             wl.mode, round_tile_bf16=not exact_weight)
+    else:
+        want = C.qmm(wl.x, wl.w, wl.scales, wl.biases, wl.group_size, wl.bits, wl.mode,
+                     round_tile_bf16=not exact_weight)
+    return _rel_l2(y.float().cpu().numpy(), want)
+
+
+def bench_once(cfg, steps=40, warmup=4, check=True):
+    """One of the other named shapes (C3 prefill, C4 MXFP4, C5 grouped): graph
+    replay over rotating weight sets, like the decode legs, so that every
+    launch streams its weights from HBM; the time includes the activation
+    re-layout / split kernel that precedes the product.  One output is checked
+    against the C oracle outside the timed region."""
     import torch
     from metaljax_amd import kernels as K, synth
     wl = synth.make(cfg)
     x, w, s, b, ro = synth.to_device(wl)
-    if cfg == 5:
-        # every row belongs to an expert, so the output buffer is reused as it is
-        # (a fresh one would be zero-filled first, for rows outside the offsets)
-        y5 = torch.empty((x.shape[0], wl.N), dtype=x.dtype, device=x.device)
-        fn = lambda: K.grouped_qmm(x, w, s, b, ro, group_size=64, bits=4, out=y5)
-    else:
-        fn = lambda: K.quantized_matmul(x, w, s, b, group_size=wl.group_size, bits=wl.bits, mode=wl.mode)
-    for _ in range(warmup):
-        fn()
-    ms = _events_ms(lambda: [fn() for _ in range(steps)], torch.cuda.current_stream())
+    per_set = w.numel() * 4 + s.numel() * s.element_size() * (2 if b is not None else 1)
+    n_sets = max(2, (2 * LLC_BYTES) // per_set + 1)
+    sets = [(w, s, b)] + [(w.clone(), s.clone(), None if b is None else b.clone()) for _ in range(n_sets - 1)]
+    ys = [torch.empty((x.shape[0], wl.N), dtype=torch.bfloat16, device="cuda") for _ in range(n_sets)]
+
+    def make_call(i):
+        wi, si, bi = sets[i]
+        if cfg == 5:        # every row of C5 belongs to an expert, so the output needs no zero fill
+            return K.BoundGrouped(x, wi, si, bi, ro, ys[i], group_size=64, bits=4)
+        return K.BoundQmm(x, wi, si, bi, ys[i], group_size=wl.group_size, bits=wl.bits, mode=wl.mode)
+    ms = run_rotating(make_call, n_sets, steps, warmup)
     us = ms * 1e3 / steps
     tf = wl.flops / us / 1e6
     out = {"workload": wl.name, "us": round(us, 2), "TFLOP/s": round(tf, 1),
-           "GB/s": round(wl.algorithmic_bytes / us / 1e3, 1)}
+           "GB/s": round(wl.algorithmic_bytes / us / 1e3, 1), "weight_sets": n_sets}
     if wl.mode == "mxfp4":
         # block-scaled matrix cores: each useful MFMA is issued twice (two FP6
         # activation terms), so both the useful and the issued rate are given
@@ -149,7 +174,34 @@ def bench_once(cfg, steps=20, warmup=3):
         out["issued_frac_of_fp4_mfma_peak"] = round(2 * tf / PEAK_TFLOPS["fp4"], 4)
     else:
         out["frac_of_bf16_mfma_peak"] = round(tf / PEAK_TFLOPS["bf16"], 4)
+    if check:
+        # bf16 outputs: distance from the exact-weight product (the 1e-2 bar),
+        # and for the bf16-tile kernels from the rounded-tile product as well
+        out["rel_l2_vs_exact_weight"] = float(f"{oracle_check(wl, ys[0], True):.3e}")
+        if wl.mode == "affine":
+            out["rel_l2_vs_bf16_tile"] = float(f"{oracle_check(wl, ys[0], False):.3e}")
+        assert out["rel_l2_vs_exact_weight"] <= 1e-2, out
     return out
+
+
+def bench_dense_bf16(m, n, k, steps=40, experts=1):
+    """The same box's library matmul on bf16 operands of a named shape
+    (x [M, K] x W [N, K]^T, `experts` of them one after another): the practical
+    ceiling for a kernel that must also dequantize."""
+    import torch
+    n_sets = max(2, (2 * LLC_BYTES) // (experts * n * k * 2) + 1)
+    ws = [torch.randn((experts, n, k), device="cuda", dtype=torch.bfloat16) for _ in range(n_sets)]
+    x = torch.randn((experts, m, k), device="cuda", dtype=torch.bfloat16)
+    ys = [torch.empty((experts, m, n), device="cuda", dtype=torch.bfloat16) for _ in range(n_sets)]
+
+    def step(i):
+        torch.bmm(x, ws[i].transpose(1, 2), out=ys[i])
+    for i in range(n_sets):
+        step(i)
+    ms = _events_ms(lambda: [step(i % n_sets) for i in range(steps)], torch.cuda.current_stream())
+    us = ms * 1e3 / steps
+    tf = 2.0 * experts * m * n * k / us / 1e6
+    return {"us": round(us, 2), "TFLOP/s": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / PEAK_TFLOPS["bf16"], 4)}
 
 
 def cpu_baseline(wl, budget_s=4.0):
@@ -224,9 +276,11 @@ def main():
         print(json.dumps({"probe": profiling.stream_probe()}))
         return 0
     if args.shape:
-        print(json.dumps({args.shape: bench_once(int(args.shape[1]))}))
+        print(json.dumps({args.shape: bench_once(int(args.shape[1]), check=not args.no_cpu)}))
         return 0
     wl, ms, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
+    headline_rel_l2 = None if args.no_cpu else oracle_check(wl, y, True)     # outside the timed region
+    assert headline_rel_l2 is None or headline_rel_l2 <= 1e-2, headline_rel_l2
     us = ms * 1e3 / args.steps
     gbs = wl.algorithmic_bytes / us / 1e3
     kern, grid, block = K.plan(wl.M, wl.N, wl.K, wl.group_size, wl.bits, wl.mode)
@@ -243,7 +297,10 @@ def main():
                    "kernel": "decode (M<=16)" if kern == 1 else "prefill", "grid": grid, "block": block},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": committed_traffic()},
+                     "traffic": committed_traffic(),
+                     "traffic_source": "profiles/decode_qmm_C2_int4_g64_hbm_traffic.txt (two rocprofv3 --pmc "
+                                       "runs of this leg; a counter run cannot happen inside this program)"},
+        "rel_l2_vs_oracle": None if headline_rel_l2 is None else float(f"{headline_rel_l2:.3e}"),
         "TFLOP/s": round(wl.flops / us / 1e6, 2),
     }
     if args.m16_only:
@@ -262,7 +319,10 @@ def main():
         out["other_shapes"] = {"C1": {"workload": wlc1.name, "us": round(usc1, 2),
                                       "GB/s": round(wlc1.algorithmic_bytes / usc1 / 1e3, 1),
                                       "frac_of_hbm_peak": round(wlc1.algorithmic_bytes / usc1 / 1e3 / HBM_PEAK_GBS, 4)}}
-        out["other_shapes"].update({f"C{c}": bench_once(c) for c in (3, 4, 5)})
+        out["other_shapes"].update({f"C{c}": bench_once(c, check=not args.no_cpu) for c in (3, 4, 5)})
+        # the library's bf16 matmul on the same shapes (no dequantization)
+        out["dense_bf16"] = {"C3 [2048,4096]x[4096,4096]": bench_dense_bf16(2048, 4096, 4096),
+                             "C5 8 x [128,4096]x[14336,4096]": bench_dense_bf16(128, 14336, 4096, experts=8)}
         # decode shapes outside the named configurations (random codes, timing only)
         out["other_decode_shapes"] = {
             "int4 g64 [28672,4096] M=4": bench_decode_random(4, 28672, 4096),

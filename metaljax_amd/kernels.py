@@ -271,3 +271,36 @@ class BoundQmm:
         if rc:
             _lib.check(rc)
         return self.y
+
+
+class BoundGrouped:
+    """A grouped_qmm call with every argument resolved once (see BoundQmm):
+    rows of `x` sorted by expert, `row_offsets` int32 [E+1] on the device,
+    results into the preallocated `y` (rows outside the offsets are left as
+    they are)."""
+
+    def __init__(self, x, w, scales, biases, row_offsets, y, group_size=64, bits=4, mode="affine"):
+        _need_cuda(x, w, scales, biases, row_offsets, y)
+        (e,), n, k = _weight_dims(w, bits, mode)
+        for t in (x, w, scales, biases, row_offsets, y):
+            if t is not None and not t.is_contiguous():
+                raise _lib.QmmError(1, "BoundGrouped needs contiguous tensors")
+        if row_offsets.dtype != torch.int32 or tuple(y.shape) != (x.shape[0], n):
+            raise _lib.QmmError(1, "row_offsets must be int32 and y [rows, N]")
+        self._lib = _lib.load()
+        tab = _dt(scales.dtype) if mode == "affine" else BF16
+        r = x.shape[0]
+        need = int(self._lib.qmm_workspace_bytes(1, r, n, k, group_size, bits, _MODE[mode], _dt(x.dtype)))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+        self._keep = (x, w, scales, biases, row_offsets, y, ws)
+        self._args = (_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y),
+                      _dt(y.dtype), _ptr(row_offsets), r, e, n, k, group_size, bits, _MODE[mode],
+                      _ptr(ws), need)
+        self.y = y
+
+    def launch(self, stream=None):
+        st = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        rc = self._lib.qmm_grouped_qmm(*self._args, st)
+        if rc:
+            _lib.check(rc)
+        return self.y
