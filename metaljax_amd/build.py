@@ -25,6 +25,8 @@ def _compile(src: str) -> str:
     # QMM_EXPERIMENTS=1: a measuring build whose kernel choice can be overridden
     # through QMM_* environment switches; the normal build reads no environment
     extra = ["-DQMM_EXPERIMENTS"] if os.environ.get("QMM_EXPERIMENTS") == "1" else []
+    if os.environ.get("QMM_TIMELINE") == "1":       # clock stamps in the decode kernel (qmm_debug_stamps)
+        extra.append("-DQMM_TIMELINE")
     cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

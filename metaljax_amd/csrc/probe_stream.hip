@@ -6,8 +6,14 @@
 //                workgroup a contiguous share, `unroll` loads in flight a
 //                lane) and keeps an XOR so that nothing is elided
 //   probe_empty  a launch of the same geometry and LDS size that does nothing
+//   probe_loaders  the decode kernel's way of asking: only the first `active`
+//                wavefronts of a workgroup request the workgroup's share, 1 KB
+//                an instruction, everything before the first wait, into
+//                registers or straight into LDS (`dma`)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 namespace {
 
@@ -30,6 +36,87 @@ __global__ void read_kernel(const u32x4* __restrict__ p, int64_t pieces_per_wg, 
   }
   const uint32_t x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
   if (x == 0x9E3779B9u && sink) sink[threadIdx.x] = x + lds[0];    // practically never: keeps the loads alive
+}
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+// U requests a wavefront: chunk (1 KB) c = wave + u * active of the workgroup's share.
+template <int U, bool DMA, int AUX>
+__global__ void loaders_kernel(const unsigned char* __restrict__ p, int chunks_per_wg, int active,
+                               uint32_t* sink) {
+  extern __shared__ unsigned char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave >= active) return;
+  const unsigned char* base = p + (int64_t)blockIdx.x * chunks_per_wg * 1024;
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(base), 0, (uint32_t)chunks_per_wg * 1024u, 0x00020000);
+  uint32_t x = 0;
+  if constexpr (DMA) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = wave + u * active;
+      const uint32_t off = c < chunks_per_wg ? (uint32_t)c * 1024u + lane * 16u : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + (c < chunks_per_wg ? c : 0) * 1024),
+                                               16, off, 0u, 0, AUX);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);     // vmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    x = reinterpret_cast<const uint32_t*>(lds)[wave * 256 + lane];
+  } else {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = wave + u * active;
+      const uint32_t off = c < chunks_per_wg ? (uint32_t)c * 1024u + lane * 16u : 0x80000000u;
+      v[u] = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0u, AUX);
+    }
+    u32x4 acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
+    x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  }
+  if (x == 0x9E3779B9u && sink) sink[threadIdx.x] = x;
+}
+
+// The loaders' request with clock stamps (constant 100 MHz clock, lane 0 of
+// every asking wavefront): start, all 32 requests issued, then a quarter, a
+// half, three quarters and all of them landed.  pattern 0: 1 KB runs as above;
+// 1: the decode kernel's tiles (a request = 256 bytes of each of four rows
+// 2 KB apart, the 16-byte pieces of a row permuted by its row number; a
+// wavefront's eight consecutive requests walk along its four rows).
+template <int PATTERN>
+__global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint64_t* stamps) {
+  extern __shared__ unsigned char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave >= 4) return;
+  uint64_t t[6];
+  t[0] = __builtin_amdgcn_s_memrealtime();
+  const unsigned char* base = p + (int64_t)blockIdx.x * 131072;
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(base), 0, 131072u, 0x00020000);
+  uint32_t lane_off;
+  if (PATTERN == 0) {
+    lane_off = (uint32_t)wave * 1024u + lane * 16u;
+  } else {
+    const int row = 4 * wave + (lane >> 4);
+    lane_off = (uint32_t)row * 2048u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
+  }
+#pragma unroll
+  for (int u = 0; u < 32; ++u) {
+    const uint32_t so = PATTERN == 0 ? (uint32_t)u * 4096u : (uint32_t)(u >> 3) * 32768u + (uint32_t)(u & 7) * 256u;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + (wave + 4 * u) * 1024), 16, lane_off, so, 0, 2);
+  }
+  t[1] = __builtin_amdgcn_s_memrealtime();
+  __builtin_amdgcn_s_waitcnt(0x4F78);       // vmcnt(24)
+  t[2] = __builtin_amdgcn_s_memrealtime();
+  __builtin_amdgcn_s_waitcnt(0x4F70);       // vmcnt(16)
+  t[3] = __builtin_amdgcn_s_memrealtime();
+  __builtin_amdgcn_s_waitcnt(0x0F78);       // vmcnt(8)
+  t[4] = __builtin_amdgcn_s_memrealtime();
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+  t[5] = __builtin_amdgcn_s_memrealtime();
+  if (lane == 0)
+    for (int i = 0; i < 6; ++i) stamps[((int64_t)blockIdx.x * 4 + wave) * 6 + i] = t[i];
 }
 
 __global__ void empty_kernel(uint32_t* sink) {
@@ -57,6 +144,45 @@ int probe_read(const void* p, int64_t bytes, void* sink, int blocks, int threads
   else if (unroll >= 4) launch(read_kernel<4>);
   else if (unroll >= 2) launch(read_kernel<2>);
   else launch(read_kernel<1>);
+  return (int)hipGetLastError();
+}
+
+// The workgroup's share (bytes / blocks, a multiple of 1 KB, at most 128 KB and, with dma, at most
+// lds_bytes) requested by `active` in {4, 8, 12} wavefronts.  nt = the loads carry the non-temporal hint.
+int probe_loaders(const void* p, int64_t bytes, void* sink, int blocks, int threads, int active, int dma,
+                  int nt, int lds_bytes, void* stream) {
+  const int chunks = (int)(bytes / blocks / 1024);
+  if (chunks > 128 || (dma && chunks * 1024 > lds_bytes) || active * 64 > threads) return -1;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kern) {
+    if (lds_bytes > 65536)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(threads), lds_bytes, st,
+                       static_cast<const unsigned char*>(p), chunks, active, static_cast<uint32_t*>(sink));
+  };
+  auto pick = [&](auto u) {
+    constexpr int U = decltype(u)::value;
+    if (dma) { if (nt) launch(loaders_kernel<U, true, 2>); else launch(loaders_kernel<U, true, 0>); }
+    else     { if (nt) launch(loaders_kernel<U, false, 2>); else launch(loaders_kernel<U, false, 0>); }
+  };
+  if (active == 4) pick(std::integral_constant<int, 32>());
+  else if (active == 8) pick(std::integral_constant<int, 16>());
+  else if (active == 12) pick(std::integral_constant<int, 11>());
+  else return -1;
+  return (int)hipGetLastError();
+}
+
+// 256 workgroups of 768 threads over 32 MiB at p; stamps: uint64 [256][4][6].
+int probe_stamped_loaders(const void* p, void* stamps, int pattern, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kern) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              147456);
+    hipLaunchKernelGGL(kern, dim3(256), dim3(768), 147456, st, static_cast<const unsigned char*>(p),
+                       static_cast<uint64_t*>(stamps));
+  };
+  if (pattern) launch(stamped_loaders_kernel<1>); else launch(stamped_loaders_kernel<0>);
   return (int)hipGetLastError();
 }
 

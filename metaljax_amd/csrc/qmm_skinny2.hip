@@ -92,10 +92,31 @@ __device__ __forceinline__ void wait_vmcnt() {    // s_waitcnt vmcnt(N) only; al
   asm volatile("" ::: "memory");
 }
 
+// Direct-to-LDS load, 16 bytes a lane.  AUX = 2 marks the lines non-temporal:
+// weights and their tables are read once per launch (a read-only launch over
+// 32 MiB measures 6.5 us with the hint against 7.5 us without).
+constexpr int kStream = 2;
+template <int AUX = 0>
 __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, unsigned char* dst, uint32_t voff,
                                       uint32_t soff) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, voff, soff, 0, 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, voff, soff, 0, AUX);
 }
+
+// Clock stamps (builds with -DQMM_TIMELINE only): lane 0 of every wavefront
+// writes the constant 100 MHz clock into g_stamps[workgroup][wavefront][i];
+// qmm_debug_stamps copies the array out.
+#ifdef QMM_TIMELINE
+constexpr int kStampWgs = 256, kStampWaves = 12, kStampSlots = 16;
+__device__ uint64_t g_stamps[kStampWgs * kStampWaves * kStampSlots];
+#define QMM_STAMP(i)                                                                              \
+  do {                                                                                            \
+    if ((threadIdx.x & 63) == 0 && blockIdx.x < kStampWgs && blockIdx.y == 0)                     \
+      g_stamps[(blockIdx.x * kStampWaves + wave) * kStampSlots + (i)] =                           \
+          __builtin_amdgcn_s_memrealtime();                                                       \
+  } while (0)
+#else
+#define QMM_STAMP(i) do {} while (0)
+#endif
 
 // all LDS traffic of this wavefront done, then the workgroup barrier
 __device__ __forceinline__ void item_barrier() {
@@ -175,8 +196,17 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* ring = smem;
   unsigned char* tabs = smem + S::B * kItem;
+  // One-pass direct variant: behind the ring and the tables, a 1 KB patch a
+  // compute wavefront (staging of more than eight rows of activations).
+  unsigned char* patches = smem + 4 * (kItem + kTab);
 
   const int lane = threadIdx.x & 63;
+  // (Wavefronts start in the order of their hardware index, a whole workgroup
+  // over about 0.4 us.  The compute wavefronts come first on purpose: data
+  // returns in the order of the requests, and their activations -- cache hits
+  // -- must not queue behind the first weight tile; with the loaders first
+  // 4096 x 14336 measured 10.6 against 9.9 us at one row, 13.3 against 11.4 us
+  // at sixteen.)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t bz = blockIdx.y;
   const int64_t n_begin = (int64_t)blockIdx.x * rows_per_wg;
@@ -255,15 +285,24 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // weight tile t of pass `p`, and its table rows, into ring slot `slot`
     auto issue_tile = [&](int p, int t, int slot) __attribute__((always_inline)) {
       unsigned char* base = ring + slot * kItem;
+      // (The wavefront-uniform offset must depend on uniform values only, or
+      // every load turns into a loop over its distinct values: a row past the
+      // end is a lane offset out of range, a slice past the end both.)
+      const bool full = n_begin + t * 16 + 16 <= n_end;                // uniform
+      uint32_t vt[4];
+#pragma unroll
+      for (int o = 0; o < 4; ++o)
+        vt[o] = full || n_begin + t * 16 + wrow[o] < n_end ? wv[o] : kOutOfRange;
+      const uint32_t tile_off = (uint32_t)(t * 16 * wpr);
       static_for<QI>([&](auto qc) __attribute__((always_inline)) {
         constexpr int q = decltype(qc)::value;
         constexpr int o = (q * NL) & 3;
         const int j = lw + q * NL;                // uniform
         const int sloc = j >> 2, rq = j & 3;
         const int sl = p * CW + sloc;
-        const bool rok = sl < slices && n_begin + t * 16 + wrow[o] < n_end;   // false for passes past the last
-        const uint32_t so = rok ? (uint32_t)sl * 256u + (uint32_t)(t * 16 * wpr) : 0u;
-        dma16(rw, base + sloc * 4096 + rq * 1024, rok ? wv[o] : kOutOfRange, so);
+        const bool sok = sl < slices;             // uniform; false for passes past the last
+        const uint32_t so = sok ? (uint32_t)sl * 256u + tile_off : 0u;
+        dma16<kStream>(rw, base + sloc * 4096 + rq * 1024, sok ? vt[o] : kOutOfRange, so);
       });
       unsigned char* tb = tabs + slot * kTab;
 #pragma unroll
@@ -281,8 +320,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // (MXFP4 has no second table: the load still goes out, fetching nothing,
         // so that every loader wavefront issues the same number per tile -- the
         // waits count loads)
-        if constexpr (MX) dma16(rs, tdst, kind == 0 ? vo : kOutOfRange, 0u);
-        else dma16(kind ? rb : rs, tdst, vo, 0u);
+        if constexpr (MX) dma16<kStream>(rs, tdst, kind == 0 ? vo : kOutOfRange, 0u);
+        else dma16<kStream>(kind ? rb : rs, tdst, vo, 0u);
       }
     };
     // item `i` (compile-time kind) of pass `p` into ring slot `slot`
@@ -347,19 +386,26 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const int p = g / ntiles;
         issue_tile(p, g - p * ntiles, g & 3);
       };
+      QMM_STAMP(0);
       issue(0);
+      QMM_STAMP(1);
       if (G > 1) issue(1);
+      QMM_STAMP(2);
 #pragma nounroll
       for (int g = 0; g < G; ++g) {
         // item g has landed: only item g+1 may still be out (a store in
         // between only tightens the wait)
         if (g + 1 < G) wait_vmcnt<LT>(); else wait_vmcnt<0>();
+        if (g < 4) QMM_STAMP(3 + 3 * g);
         item_barrier();                           // item g published; item g-1 consumed
+        if (g < 4) QMM_STAMP(4 + 3 * g);
         if (g + 2 < G) issue(g + 2);              // that slot's last tile was consumed (and, in the last pass, reduced) a step ago
         if (g >= 1 && g - 1 >= G - ntiles) reduce_tile(passes - 1, g - 1 - (G - ntiles), (g - 1) & 3);
+        if (g < 4) QMM_STAMP(5 + 3 * g);
       }
       item_barrier();                             // everything consumed
       reduce_tile(passes - 1, ntiles - 1, (G - 1) & 3);
+      QMM_STAMP(15);
       return;
     }
     // Slot of every item of the current pass (by order of use) and of the next
@@ -640,12 +686,13 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // per instruction), which at sixteen rows costs more than it saves.
       // Here the slice comes in with whole-line loads instead -- instruction
       // (c, h) fetches the 128 bytes of chunk c of rows 8h .. 8h+7 -- all of
-      // them requested at once, and each chunk takes a round trip through a
-      // 2 KB wave-private LDS patch into operand order (piece p of row r at
-      // position p ^ ((r >> 1) & 7): both the 16-lane write and read passes
-      // touch every bank once).
+      // them requested at once, and each takes a round trip through a 1 KB
+      // wave-private LDS patch into operand order (piece p of row r at
+      // position p ^ ((r >> 1) & 3): both the 16-lane write and read passes
+      // touch every bank once; the lanes whose operand row is in the other
+      // half read along and keep what they had).
       auto fetch_x_staged = [&](int p, bool active) __attribute__((always_inline)) {
-        unsigned char* stg = smem + 4 * (kItem + kTab) + wave * 2048;
+        unsigned char* stg = patches + wave * 1024;
         const int srow = lane >> 3, sp = lane & 7;
         u32x4 raw[CPS][2];
         uint32_t lo[2];
@@ -660,27 +707,30 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
           for (int h = 0; h < 2; ++h)
             raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo[h], so + (uint32_t)(c * 128), 0);
-        const uint32_t wr0 = (uint32_t)(srow * 128 + ((sp ^ ((srow >> 1) & 7)) << 4));          // rows 0-7
-        const uint32_t wr1 = (uint32_t)((srow + 8) * 128 + ((sp ^ (((srow + 8) >> 1) & 7)) << 4));
-        const uint32_t rkey = (uint32_t)((r >> 1) & 7);
+        const uint32_t wr = (uint32_t)(srow * 128 + ((sp ^ ((srow >> 1) & 3)) << 4));
+        const uint32_t rkey = (uint32_t)((r >> 1) & 3);
+        const bool upper = r >= 8;
 #pragma unroll
-        for (int c = 0; c < CPS; ++c) {
-          *reinterpret_cast<u32x4*>(stg + wr0) = raw[c][0];
-          *reinterpret_cast<u32x4*>(stg + wr1) = raw[c][1];
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (int c = 0; c < CPS; ++c)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const uint32_t pc = (uint32_t)(kg * 2 + j);
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + r * 128 + ((pc ^ rkey) << 4));
-            if constexpr (BITS == 4 && !MX) xa[c][j] = pair_stride4(v);
-            else xa[c][j] = __builtin_bit_cast(bf16x8, v);
+          for (int h = 0; h < 2; ++h) {                          // rows 8h .. 8h+7 of chunk c
+            *reinterpret_cast<u32x4*>(stg + wr) = raw[c][h];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const uint32_t pc = (uint32_t)(kg * 2 + j);
+              const u32x4 v = *reinterpret_cast<const u32x4*>(stg + (r & 7) * 128 + ((pc ^ rkey) << 4));
+              bf16x8 o;
+              if constexpr (BITS == 4 && !MX) o = pair_stride4(v);
+              else o = __builtin_bit_cast(bf16x8, v);
+              if (upper == (h == 1)) xa[c][j] = o;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
         if constexpr (!MX) {
           if (active) chunk_sums();
         }
@@ -689,21 +739,25 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
         const bool active = wave < slices;        // uniform
+        QMM_STAMP(0);
         if constexpr (!WIDE) {                    // (wide table rows leave no LDS for the staging patches)
           if (M > 8) fetch_x_staged(0, active);
           else fetch_x(0, active, xlane);
         } else {
           fetch_x(0, active, xlane);
         }
+        QMM_STAMP(2);
 #pragma nounroll
         for (int g = 0; g < ntiles; ++g) {
           item_barrier();
+          if (g < 4) QMM_STAMP(3 + 2 * g);
           const int slot = g & 3;
           f32x4 at = zero;
           if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + tab_row, zero);
           float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
 #pragma unroll
           for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
+          if (g < 4) QMM_STAMP(4 + 2 * g);
         }
       } else {
         // Several passes: the tiles' sums stay in registers from pass to pass
@@ -805,9 +859,9 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
   constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (GSHIFT == 5 ? 2 : 1);
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
-  // (one-pass direct variant: plus a 2 KB patch a compute wavefront for staging activations)
+  // (one-pass direct variant: plus a 1 KB patch a compute wavefront for staging activations)
   const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind) +
-                     (XD == 1 && GSHIFT != 5 ? (size_t)CW * 2048 : 0);
+                     (XD == 1 && GSHIFT != 5 ? (size_t)CW * 1024 : 0);
   constexpr auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);
@@ -1011,3 +1065,11 @@ void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st) {
 }
 
 }  // namespace qmm
+
+#ifdef QMM_TIMELINE
+extern "C" int qmm_debug_stamps(void* out, size_t bytes) {
+  if (bytes > sizeof(qmm::g_stamps)) bytes = sizeof(qmm::g_stamps);
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(qmm::g_stamps), bytes);
+}
+#endif
+

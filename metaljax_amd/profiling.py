@@ -64,6 +64,7 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
     vp, ci, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
     lib.probe_read.argtypes = [vp, i64, vp, ci, ci, ci, ci, vp]
     lib.probe_empty.argtypes = [vp, ci, ci, ci, vp]
+    lib.probe_loaders.argtypes = [vp, i64, vp, ci, ci, ci, ci, ci, ci, vp]
     n_sets = (2 * (256 << 20)) // nbytes + 1
     bufs = [torch.randint(-2**31, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda")
             for _ in range(n_sets)]
@@ -91,7 +92,7 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
             torch.cuda.synchronize()
             return a.elapsed_time(b) * 1e3 / (n * n_sets)
 
-    out = {"bytes": nbytes, "buffers": n_sets, "read": {}, "empty": {}}
+    out = {"bytes": nbytes, "buffers": n_sets, "read": {}, "loaders": {}, "empty": {}}
     for blocks, threads, unroll, lds in ((256, 1024, 8, 0), (256, 768, 8, 0), (256, 768, 8, 147456),
                                          (512, 512, 8, 0), (1024, 256, 8, 0), (2048, 256, 4, 0),
                                          (4096, 256, 2, 0), (8192, 256, 1, 0)):
@@ -101,6 +102,18 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
         us = timed(launch)
         out["read"][f"{blocks}x{threads} unroll {unroll} lds {lds}"] = {
             "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1)}
+    if nbytes // 256 <= 128 << 10:
+        for active in (4, 8, 12):
+            for dma in (0, 1):
+                for nt in (0, 1):
+                    def launch(i, st, a=active, d=dma, h=nt):
+                        rc = lib.probe_loaders(bufs[i].data_ptr(), nbytes, sink.data_ptr(), 256, 768, a, d, h,
+                                               147456, st)
+                        assert rc == 0, rc
+                    us = timed(launch)
+                    out["loaders"][f"256x768, {active} wavefronts ask, {'into LDS' if dma else 'into registers'}"
+                                   f"{', non-temporal' if nt else ''}"] = {
+                        "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1)}
     for blocks, threads, lds in ((256, 768, 147456), (256, 768, 0), (256, 256, 0)):
         def launch(i, st, b=blocks, t=threads, l=lds):
             rc = lib.probe_empty(sink.data_ptr(), b, t, l, st)
