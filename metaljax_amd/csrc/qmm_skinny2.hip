@@ -294,16 +294,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       for (int o = 0; o < 4; ++o)
         vt[o] = full || n_begin + t * 16 + wrow[o] < n_end ? wv[o] : kOutOfRange;
       const uint32_t tile_off = (uint32_t)(t * 16 * wpr);
-      static_for<QI>([&](auto qc) __attribute__((always_inline)) {
-        constexpr int q = decltype(qc)::value;
-        constexpr int o = (q * NL) & 3;
-        const int j = lw + q * NL;                // uniform
-        const int sloc = j >> 2, rq = j & 3;
-        const int sl = p * CW + sloc;
-        const bool sok = sl < slices;             // uniform; false for passes past the last
-        const uint32_t so = sok ? (uint32_t)sl * 256u + tile_off : 0u;
-        dma16<kStream>(rw, base + sloc * 4096 + rq * 1024, sok ? vt[o] : kOutOfRange, so);
-      });
+      // The table rows go first (their sixteen quarter lines are the slow part
+      // of a tile's requests; ahead of the codes they measured 0.1-0.2 us a
+      // launch better than behind them).
       unsigned char* tb = tabs + slot * kTab;
 #pragma unroll
       for (int q = 0; q < QT; ++q) {
@@ -323,6 +316,16 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if constexpr (MX) dma16<kStream>(rs, tdst, kind == 0 ? vo : kOutOfRange, 0u);
         else dma16<kStream>(kind ? rb : rs, tdst, vo, 0u);
       }
+      static_for<QI>([&](auto qc) __attribute__((always_inline)) {
+        constexpr int q = decltype(qc)::value;
+        constexpr int o = (q * NL) & 3;
+        const int j = lw + q * NL;                // uniform
+        const int sloc = j >> 2, rq = j & 3;
+        const int sl = p * CW + sloc;
+        const bool sok = sl < slices;             // uniform; false for passes past the last
+        const uint32_t so = sok ? (uint32_t)sl * 256u + tile_off : 0u;
+        dma16<kStream>(rw, base + sloc * 4096 + rq * 1024, sok ? vt[o] : kOutOfRange, so);
+      });
     };
     // item `i` (compile-time kind) of pass `p` into ring slot `slot`
     auto issue_item = [&](int p, auto ic, int slot) __attribute__((always_inline)) {
@@ -503,24 +506,48 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       sl_cur[S::item_at(j)] = j;
     });
     bf16x8 xa[CPS][2];
-    bf16x8 axh, axm, axo;
-    // xs_c = sum_k x over chunk c, in operand layout, split into three bf16
-    // terms and packed as MFMA A operands over the chunk index (kg == 0 lanes)
+    // The code-independent part of a tile's sums is sum_c t_c * xs_c over the
+    // chunks c of the slice, xs_c = sum_k x over chunk c, for every table entry
+    // t that multiplies a constant: the bias, and for four-bit codes (widened
+    // as 128 + q) the scale times -128.  It runs on the matrix cores with the
+    // chunk index as the K dimension: xs_c is split into three bf16 terms
+    // (24 bits, exact), a float16 / float32 table entry into two / three.  A
+    // slice has eight chunks and the instruction's K is 32, so four (x term,
+    // table term) pairs share one MFMA, one per lane quarter kg: pair g =
+    // (kind, table term, x term) sits in MFMA g / 4, quarter g % 4.  The A
+    // operands depend on the activations only and are built once; bf16 tables
+    // with four-bit codes take two MFMAs a tile this way instead of six.
+    constexpr int NT = F32T ? 3 : F16T ? 2 : 1;     // bf16 terms per table entry
+    constexpr int NG = (BITS == 4 ? 2 : 1) * NT * 3;
+    constexpr int NA = (NG + 3) / 4;
+    bf16x8 ax[NA];
     auto chunk_sums = [&]() __attribute__((always_inline)) {
-      float xh[8], xm[8], xo[8];
+      float xt[3][8];
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         float xs = 0.f;
         if (c < CPS) {
           f32x4 t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][0], zero, 0, 0, 0);
           t4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xa[c][1], t4, 0, 0, 0);
-          xs = kg == 0 ? t4[0] : 0.f;
+          xs = t4[0];                               // every row of the product holds the column's sum
         }
-        split3(xs, xh[c], xm[c], xo[c]);
+        split3(xs, xt[0][c], xt[1][c], xt[2][c]);
       }
-      axh = as_bf16x8(hi16_pair(xh[0], xh[1]), hi16_pair(xh[2], xh[3]), hi16_pair(xh[4], xh[5]), hi16_pair(xh[6], xh[7]));
-      axm = as_bf16x8(hi16_pair(xm[0], xm[1]), hi16_pair(xm[2], xm[3]), hi16_pair(xm[4], xm[5]), hi16_pair(xm[6], xm[7]));
-      axo = as_bf16x8(hi16_pair(xo[0], xo[1]), hi16_pair(xo[2], xo[3]), hi16_pair(xo[4], xo[5]), hi16_pair(xo[6], xo[7]));
+      static_for<NA>([&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        float v[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) v[c] = 0.f;
+        static_for<4>([&](auto qc) __attribute__((always_inline)) {
+          constexpr int g = 4 * i + decltype(qc)::value;
+          if constexpr (g < NG) {
+            constexpr float f = g / (3 * NT) ? -128.f : 1.f;      // exact: a power of two
+#pragma unroll
+            for (int c = 0; c < 8; ++c) v[c] = kg == (g & 3) ? f * xt[g % 3][c] : v[c];
+          }
+        });
+        ax[i] = as_bf16x8(hi16_pair(v[0], v[1]), hi16_pair(v[2], v[3]), hi16_pair(v[4], v[5]), hi16_pair(v[6], v[7]));
+      });
     };
     // acc + this wavefront's K-slice of one tile: `base` is the lane's row in
     // the slice's 4 KB of codes, `tb` its table row
@@ -565,23 +592,6 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         hi = as_bf16x8(h[0], h[1], h[2], h[3]);
         lo = as_bf16x8(l[0], l[1], l[2], l[3]);
       };
-      auto xs_times = [&](const u32x4& t, f32x4 in) __attribute__((always_inline)) {
-        if constexpr (F16T) {
-          bf16x8 hi, lo;
-          split_f16(t, hi, lo);
-          f32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, hi, in, 0, 0, 0);
-          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, hi, r, 0, 0, 0);
-          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, hi, r, 0, 0, 0);
-          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, lo, r, 0, 0, 0);
-          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, lo, r, 0, 0, 0);
-          return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, lo, r, 0, 0, 0);
-        } else {
-          const bf16x8 op = __builtin_bit_cast(bf16x8, t);
-          f32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, op, in, 0, 0, 0);
-          r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, op, r, 0, 0, 0);
-          return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, op, r, 0, 0, 0);
-        }
-      };
       // float32 tables: the entries of the eight chunks as floats (group 128: one
       // entry serves two chunks), and as matrix operands three bf16 terms each
       float sf[8], bfv[8];
@@ -602,33 +612,40 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           }
         }
       }
-      auto xs_times_f32 = [&](const float (&v)[8], f32x4 in) __attribute__((always_inline)) {
-        float h[8], m[8], l[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) split3(v[i], h[i], m[i], l[i]);
-        const bf16x8 oh = as_bf16x8(hi16_pair(h[0], h[1]), hi16_pair(h[2], h[3]), hi16_pair(h[4], h[5]), hi16_pair(h[6], h[7]));
-        const bf16x8 om = as_bf16x8(hi16_pair(m[0], m[1]), hi16_pair(m[2], m[3]), hi16_pair(m[4], m[5]), hi16_pair(m[6], m[7]));
-        const bf16x8 ol = as_bf16x8(hi16_pair(l[0], l[1]), hi16_pair(l[2], l[3]), hi16_pair(l[4], l[5]), hi16_pair(l[6], l[7]));
-        f32x4 r = in;
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, oh, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, oh, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, oh, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, om, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, om, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, om, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axh, ol, r, 0, 0, 0);
-        r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(axm, ol, r, 0, 0, 0);
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(axo, ol, r, 0, 0, 0);
-      };
-      f32x4 accb, accs = zero;
+      // the bf16 terms of the table entries as matrix operands over the chunk
+      // index: tt[kind * NT + term], kind 0 = bias, 1 = scale
+      bf16x8 tt[2 * NT];
       if constexpr (F32T) {
-        accb = xs_times_f32(bfv, acc_in);
-        if constexpr (BITS == 4) accs = xs_times_f32(sf, zero);
+        auto terms = [&](const float (&v)[8], bf16x8* out) __attribute__((always_inline)) {
+          float h[8], m[8], l[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) split3(v[i], h[i], m[i], l[i]);
+          out[0] = as_bf16x8(hi16_pair(h[0], h[1]), hi16_pair(h[2], h[3]), hi16_pair(h[4], h[5]), hi16_pair(h[6], h[7]));
+          out[1] = as_bf16x8(hi16_pair(m[0], m[1]), hi16_pair(m[2], m[3]), hi16_pair(m[4], m[5]), hi16_pair(m[6], m[7]));
+          out[2] = as_bf16x8(hi16_pair(l[0], l[1]), hi16_pair(l[2], l[3]), hi16_pair(l[4], l[5]), hi16_pair(l[6], l[7]));
+        };
+        terms(bfv, tt);
+        if constexpr (BITS == 4) terms(sf, tt + NT);
+      } else if constexpr (F16T) {
+        split_f16(bvt, tt[0], tt[1]);
+        if constexpr (BITS == 4) split_f16(svt, tt[2], tt[3]);
       } else {
-        accb = xs_times(bvt, acc_in);
-        if constexpr (BITS == 4) accs = xs_times(svt, zero);
+        tt[0] = __builtin_bit_cast(bf16x8, bvt);
+        if constexpr (BITS == 4) tt[1] = __builtin_bit_cast(bf16x8, svt);
       }
-      f32x4 at = accb;
+      f32x4 at = acc_in;
+      static_for<NA>([&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        bf16x8 op = tt[(4 * i) / 3];
+        static_for<3>([&](auto qc) __attribute__((always_inline)) {
+          constexpr int g = 4 * i + 1 + decltype(qc)::value;
+          if constexpr (g < NG && g / 3 != (g - 1) / 3) {        // the table term changes at this quarter
+            const bf16x8 nx = tt[g / 3];
+            op = kg >= (g & 3) ? nx : op;
+          }
+        });
+        at = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[i], op, at, 0, 0, 0);
+      });
 #pragma unroll
       for (int c = 0; c < CPS; ++c) {
         f32x4 d;
@@ -650,10 +667,6 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         else sc = __uint_as_float((c & 1) ? (sw & 0xFFFF0000u) : (sw << 16));
 #pragma unroll
         for (int e = 0; e < 4; ++e) at[e] = fmaf(sc, d[e], at[e]);
-      }
-      if constexpr (BITS == 4) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) at[e] = fmaf(-128.f, accs[e], at[e]);
       }
       return at;
     };
