@@ -101,10 +101,15 @@ __global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint
     const int row = 4 * wave + (lane >> 4);
     lane_off = (uint32_t)row * 2048u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
   }
+  uint64_t ti[4];
 #pragma unroll
   for (int u = 0; u < 32; ++u) {
     const uint32_t so = PATTERN == 0 ? (uint32_t)u * 4096u : (uint32_t)(u >> 3) * 32768u + (uint32_t)(u & 7) * 256u;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + (wave + 4 * u) * 1024), 16, lane_off, so, 0, 2);
+    if (u == 0) ti[0] = __builtin_amdgcn_s_memrealtime();
+    if (u == 1) ti[1] = __builtin_amdgcn_s_memrealtime();
+    if (u == 7) ti[2] = __builtin_amdgcn_s_memrealtime();
+    if (u == 15) ti[3] = __builtin_amdgcn_s_memrealtime();
   }
   t[1] = __builtin_amdgcn_s_memrealtime();
   __builtin_amdgcn_s_waitcnt(0x4F78);       // vmcnt(24)
@@ -115,8 +120,10 @@ __global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint
   t[4] = __builtin_amdgcn_s_memrealtime();
   __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
   t[5] = __builtin_amdgcn_s_memrealtime();
-  if (lane == 0)
-    for (int i = 0; i < 6; ++i) stamps[((int64_t)blockIdx.x * 4 + wave) * 6 + i] = t[i];
+  if (lane == 0) {
+    for (int i = 0; i < 6; ++i) stamps[((int64_t)blockIdx.x * 4 + wave) * 10 + i] = t[i];
+    for (int i = 0; i < 4; ++i) stamps[((int64_t)blockIdx.x * 4 + wave) * 10 + 6 + i] = ti[i];
+  }
 }
 
 __global__ void empty_kernel(uint32_t* sink) {
@@ -173,7 +180,8 @@ int probe_loaders(const void* p, int64_t bytes, void* sink, int blocks, int thre
   return (int)hipGetLastError();
 }
 
-// 256 workgroups of 768 threads over 32 MiB at p; stamps: uint64 [256][4][6].
+// 256 workgroups of 768 threads over 32 MiB at p; stamps: uint64 [256][4][10] (the six above, then after the
+// 1st, 2nd, 8th and 16th request was issued).
 int probe_stamped_loaders(const void* p, void* stamps, int pattern, void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   auto launch = [&](auto kern) {

@@ -748,6 +748,62 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           if (active) chunk_sums();
         }
       };
+      // Five to eight rows, through the same patch with whole-line loads.  The
+      // direct fetch above makes every live lane a cache-line request of its
+      // own: at eight rows 512 requests a wavefront for 64 lines of data, all
+      // in front of the loaders' first tile in a vector-memory path that serves
+      // a compute unit's requests in order.  Here an instruction covers R rows
+      // with 1024 / R consecutive bytes each, so a slice takes R of them, every
+      // instruction's 1 KB goes through the patch (piece p of row r at position
+      // p ^ key(r): conflict-free both ways) and comes back in operand order.
+      // 4096 x 14336, four-bit, same box: eight rows 9.8 against 10.7 us a
+      // launch; up to four rows the direct fetch stays ahead (R = 4: 10.2
+      // against 10.0 us, R = 1: 10.0-10.5 against 9.8 us: few lanes are live
+      // and the round trip through LDS is the longer way).
+      auto fetch_x_lines = [&](auto rc, bool active) __attribute__((always_inline)) {
+        constexpr int SB = CPS * 128;                             // bytes of a row's slice
+        constexpr int R = decltype(rc)::value * SB < 1024 ? 1024 / SB : decltype(rc)::value;
+        constexpr int W = 1024 / R;                               // bytes a row and instruction
+        constexpr int NI = SB / W;                                // instructions a slice
+        constexpr int CPI = W / 128;                              // chunks an instruction
+        constexpr int LPR = W / 16;                               // lanes a row
+        unsigned char* stg = patches + wave * 1024;
+        const int srow = lane / LPR, sp = lane % LPR;
+        auto key = [](int row) { return R == 8 ? (row >> 1) & 3 : row; };
+        const int64_t xr = active ? xrow(srow) : -1;
+        const uint32_t lo = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)sp * 16u : kOutOfRange;
+        const uint32_t so = active ? (uint32_t)(wave * KS) * 2u : 0u;
+        u32x4 raw[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo, so + (uint32_t)(i * W), 0);
+        const uint32_t wr = (uint32_t)(srow * W + ((sp ^ key(srow)) << 4));
+        const int rr = r % R;
+        const uint32_t rd = (uint32_t)(rr * W), rkey = (uint32_t)key(rr);
+        const bool live = r < R;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          *reinterpret_cast<u32x4*>(stg + wr) = raw[i];
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int cc = 0; cc < CPI; ++cc)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const uint32_t pc = (uint32_t)(cc * 8 + kg * 2 + j);
+              u32x4 v = *reinterpret_cast<const u32x4*>(stg + rd + ((pc ^ rkey) << 4));
+              if (!live) v = u32x4{0u, 0u, 0u, 0u};
+              if constexpr (BITS == 4 && !MX) xa[i * CPI + cc][j] = pair_stride4(v);
+              else xa[i * CPI + cc][j] = __builtin_bit_cast(bf16x8, v);
+            }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        if constexpr (!MX) {
+          if (active) chunk_sums();
+        }
+      };
       if constexpr (XD == 1) {
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
@@ -755,6 +811,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         QMM_STAMP(0);
         if constexpr (!WIDE) {                    // (wide table rows leave no LDS for the staging patches)
           if (M > 8) fetch_x_staged(0, active);
+          else if (M > 4) fetch_x_lines(std::integral_constant<int, 8>{}, active);
           else fetch_x(0, active, xlane);
         } else {
           fetch_x(0, active, xlane);
