@@ -84,11 +84,66 @@ __global__ void loaders_kernel(const unsigned char* __restrict__ p, int chunks_p
 // 1: the decode kernel's tiles (a request = 256 bytes of each of four rows
 // 2 KB apart, the 16-byte pieces of a row permuted by its row number; a
 // wavefront's eight consecutive requests walk along its four rows).
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+// What the other eight wavefronts of the workgroup do meanwhile (`busy`): 0 nothing, 1 sleep in a loop, 2 matrix
+// instructions, 3 vector ALU work, 4 LDS reads, 5 all three, 6 / 7 an activation fetch first (below); about `iters` rounds of 16 instructions of each kind.
+__device__ __forceinline__ void bystander(int busy, int iters, unsigned char* lds, int lane, uint32_t* sink) {
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  bf16x8_t a, b;
+  for (int i = 0; i < 8; ++i) { a[i] = (__bf16)(float)(lane + i); b[i] = (__bf16)1.0f; }
+  float v = (float)lane;
+  uint32_t x = 0;
+  for (int it = 0; it < iters; ++it) {
+    if (busy == 1) __builtin_amdgcn_s_sleep(8);
+    if (busy == 2 || busy == 5) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+    if (busy == 3 || busy == 5) {
+#pragma unroll
+      for (int k = 0; k < 64; ++k) v = __builtin_fmaf(v, 1.0001f, 0.5f);
+    }
+    if (busy == 4 || busy == 5) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        x ^= *reinterpret_cast<volatile uint32_t*>(lds + 135168 + ((lane * 8 + k * 512 + it * 64) & 8191));
+    }
+  }
+  if (acc[0] + v == 12345.678f && x == 77u) sink[0] = 1u;
+}
+
 template <int PATTERN>
-__global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint64_t* stamps) {
+__global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint64_t* stamps, int busy, int iters) {
   extern __shared__ unsigned char lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (wave >= 4) return;
+  if (wave >= 4) {
+    if (busy >= 6) {
+      // the decode kernel's activation fetch ahead of the stream: sixteen loads a wavefront from one 128 KB array
+      // that every workgroup reads (busy 6: one live row, i.e. four live lanes an instruction; 7: sixteen rows,
+      // whole lines), then `iters` rounds of arithmetic
+      const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(p), 0, 131072u, 0x00020000);
+      u32x4 v[16];
+      const int w8 = wave - 4;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        uint32_t off;
+        if (busy == 6) off = (lane & 15) == 0 ? (uint32_t)(w8 * 1024 + (u >> 1) * 128 + (lane >> 4) * 32 + (u & 1) * 16) : 0x80000000u;
+        else off = (uint32_t)(((u & 1) * 8 + (lane >> 3)) * 8192 + w8 * 1024 + (u >> 1) * 128 + (lane & 7) * 16);
+        v[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0u, 0);
+      }
+      uint32_t x = 0;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) x ^= v[u][0] ^ v[u][3];
+      if (x == 0x12345u) reinterpret_cast<uint32_t*>(stamps)[65536 * 2 + 1] = x;
+      bystander(5, iters, lds, lane, reinterpret_cast<uint32_t*>(stamps) + 65536 * 2);
+      return;
+    }
+    if (busy) bystander(busy, iters, lds, lane, reinterpret_cast<uint32_t*>(stamps) + 65536 * 2);
+    return;
+  }
+  if (busy >= 6) __builtin_amdgcn_s_sleep(32);     // (the loaders start about 0.4 us after the first wavefronts)
   uint64_t t[6];
   t[0] = __builtin_amdgcn_s_memrealtime();
   const unsigned char* base = p + (int64_t)blockIdx.x * 131072;
@@ -181,14 +236,14 @@ int probe_loaders(const void* p, int64_t bytes, void* sink, int blocks, int thre
 }
 
 // 256 workgroups of 768 threads over 32 MiB at p; stamps: uint64 [256][4][10] (the six above, then after the
-// 1st, 2nd, 8th and 16th request was issued).
-int probe_stamped_loaders(const void* p, void* stamps, int pattern, void* stream) {
+// 1st, 2nd, 8th and 16th request was issued); at least 1 MiB, its tail is the bystanders' sink.
+int probe_stamped_loaders(const void* p, void* stamps, int pattern, int busy, int iters, void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   auto launch = [&](auto kern) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               147456);
     hipLaunchKernelGGL(kern, dim3(256), dim3(768), 147456, st, static_cast<const unsigned char*>(p),
-                       static_cast<uint64_t*>(stamps));
+                       static_cast<uint64_t*>(stamps), busy, iters);
   };
   if (pattern) launch(stamped_loaders_kernel<1>); else launch(stamped_loaders_kernel<0>);
   return (int)hipGetLastError();
