@@ -144,6 +144,13 @@ __global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint
     return;
   }
   if (busy >= 6) __builtin_amdgcn_s_sleep(32);     // (the loaders start about 0.4 us after the first wavefronts)
+  if (busy == -1) {
+    // 256 scalar instructions of eight bytes each (2 KB of straight-line code) ahead of the first request: what a
+    // preamble of that length costs when the instructions have to be fetched first
+    uint32_t k = (uint32_t)iters;
+    asm volatile(".rept 256\n\ts_add_u32 %0, %0, 0x12345\n\t.endr" : "+s"(k));
+    if (k == 77u) stamps[1 << 17] = k;
+  }
   uint64_t t[6];
   t[0] = __builtin_amdgcn_s_memrealtime();
   const unsigned char* base = p + (int64_t)blockIdx.x * 131072;

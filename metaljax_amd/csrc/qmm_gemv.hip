@@ -49,6 +49,7 @@ namespace {
 // so their scale and bias are zero.
 template <int BITS, int CH, int T, int WAVES, int TAB, int U, bool VT>
 __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
+  load_args_now(a);
   constexpr int STEPS = CH / 32;                 // MFMA steps per chunk
   constexpr int WPL = CH * BITS / 128;           // packed words per lane per chunk
   constexpr int WPC = CH * BITS / 32;            // packed words per row per chunk
@@ -221,6 +222,7 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
 // no rescaling afterwards.  One macro chunk = 128 k = four MFMA steps.
 template <int T, int WAVES, int U>
 __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
+  load_args_now(a);
   constexpr int ROWS = 16 * T;
   __shared__ float red[WAVES][T][4][kWave];
 

@@ -95,4 +95,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64
 
 constexpr uint32_t kOutOfRange = 0x80000000u;     // lane / uniform offset that always misses
 
+// Every argument into scalar registers at the top of a kernel.  Left to
+// itself the compiler loads an argument where it is first used, i.e. behind
+// each early-exit branch in turn: three or four scalar-load round trips, one
+// after the other, before the first useful instruction of a launch that lasts
+// ten microseconds.  Naming them all here makes the loads go out together.
+__device__ __forceinline__ void load_args_now(const GemvArgs& a) {
+  asm volatile("" ::"s"(a.x), "s"(a.w), "s"(a.s), "s"(a.b), "s"(a.y), "s"(a.M), "s"(a.N), "s"(a.K),
+               "s"(a.gshift), "s"(a.y_dtype), "s"(a.lhs_idx), "s"(a.rhs_idx), "s"(a.n_experts),
+               "s"(a.n_xrows), "s"(a.segments), "s"(a.src_row), "s"(a.out_row), "s"(a.x_rows));
+}
+
 }  // namespace qmm

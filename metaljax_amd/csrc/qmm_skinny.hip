@@ -73,6 +73,7 @@ __device__ __forceinline__ void load_tile(u32x4 (&w)[4], __amdgpu_buffer_rsrc_t 
 
 template <int BITS, int WAVES, int TMAX, int GSHIFT>
 __global__ __launch_bounds__(kWave* WAVES) void skinny_affine_kernel(GemvArgs a, int rows_per_wg) {
+  load_args_now(a);
   constexpr int KS = kSliceBytes * 8 / BITS;      // codes per slice: 512 | 256
   constexpr int CPS = KS / 64;                    // 64-code chunks per slice: 8 | 4
   constexpr int XR = KS / 128;                    // activation staging rounds (128 codes each)

@@ -175,6 +175,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 template <int BITS, int CW, int NL, int TMAX, int GSHIFT, int XD>
 __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, int rows_per_wg) {
+  load_args_now(a);
+  asm volatile("" ::"s"(rows_per_wg));
   constexpr int KS = 2048 / BITS;                 // codes per slice: 512 | 256
   constexpr int CPS = KS / 64;                    // 64-code chunks per slice: 8 | 4
   constexpr int XR = XD ? 0 : KS / 128;           // activation rounds per slice through the ring: 4 | 2, or none
