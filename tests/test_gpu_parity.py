@@ -318,7 +318,9 @@ def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     (4, 64, 4, 9000, 4096),      # one pass, activations fetched directly
     (4, 128, 1, 4096, 4096),     # group 128, one tile a workgroup
     (8, 64, 16, 5000, 2048),     # eight-bit codes, sixteen rows
-    (4, 64, 16, 14336, 4096),    # sixteen rows, 56 rows a workgroup: activations through the ring
+    (4, 64, 16, 14336, 4096),    # sixteen rows, 56 rows a workgroup: activations staged through LDS patches
+    (4, 64, 6, 14336, 4096),     # six rows: whole-line activation loads through the patches
+    (8, 128, 8, 7000, 2048),     # the same with eight-bit codes (half as many bytes a slice)
     (4, 64, 3, 3000, 8192),      # two passes, rows packed
     (4, 128, 12, 2048, 12288),   # three passes, one tile a workgroup, activations fetched per pass
 ])
@@ -345,6 +347,8 @@ def test_decode_big_weights_float16_tables(bits, gs, m, n, k):
     (4, 64, 3, 3000, 8192),      # two passes, rows packed
     (4, 128, 12, 2048, 12288),   # three passes, one tile a workgroup, activations fetched per pass
     (4, 64, 2, 28001, 4096),     # seven tiles a workgroup, the last ragged
+    (4, 128, 7, 9000, 4096),     # seven rows, group 128: whole-line activation loads through the patches
+    (4, 64, 6, 9000, 4096),      # six rows, groups of 64: wide table rows leave no patches, direct fetch
 ])
 def test_decode_big_weights_float32_tables(bits, gs, m, n, k):
     """float32 scales and biases (biases that do not fit 16 bits): an entry is
