@@ -251,6 +251,9 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a 64 MiB read + 64 MiB write elementwise kernel five times, "
                          "for scaling FETCH_SIZE / WRITE_SIZE counter readings")
+    ap.add_argument("--timeline", action="store_true",
+                    help="print the decode kernel's clock-stamp timeline on C2 (needs a library built with "
+                         "QMM_TIMELINE=1)")
     ap.add_argument("--probe", action="store_true",
                     help="time read-only and empty launches instead (what one launch over the "
                          "headline's bytes can reach on this GPU whatever its arithmetic)")
@@ -271,6 +274,10 @@ def main():
         for _ in range(5):
             torch.bitwise_not(src, out=dst)
         torch.cuda.synchronize()
+    if args.timeline:
+        from metaljax_amd import profiling
+        print(json.dumps({"decode_timeline_us": profiling.decode_timeline()}, indent=1))
+        return 0
     if args.probe:
         from metaljax_amd import profiling
         print(json.dumps({"probe": profiling.stream_probe()}))

@@ -122,6 +122,53 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
     return out
 
 
+def decode_timeline(cfg: int = 2, rows=(1, 16)):
+    """Clock stamps of the decode kernel's last launch over 18 rotating weight
+    sets (a library built with QMM_TIMELINE=1 keeps them; `qmm_debug_stamps`
+    copies them out): per wavefront role, the median over the workgroups of
+    each stamp in microseconds after the launch's first wavefront starts.
+    Returns {rows: {"compute first / second of a SIMD" | "loader": {stamp: us}}}."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from . import _lib, kernels, synth
+    lib = _lib.load()
+    if not hasattr(lib, "qmm_debug_stamps"):
+        raise RuntimeError("this library keeps no clock stamps: build it with QMM_TIMELINE=1")
+    compute = ["start", None, "activations in", "tile 0 published", "tile 0 computed", "tile 1 published",
+               "tile 1 computed", "tile 2 published", "tile 2 computed", "tile 3 published", "tile 3 computed"]
+    loader = ["start", "tile 0 requested", "tile 1 requested", "tile 0 landed", "tile 0 published",
+              "tile 2 requested", "tile 1 landed", "tile 1 published", "tile 3 requested, tile 0 summed",
+              "tile 2 landed", "tile 2 published", "tile 1 summed", "tile 3 landed", "tile 3 published",
+              "tile 2 summed", "end"]
+    out = {}
+    for m in rows:
+        wl = synth.make(cfg, M=m)
+        sets = [synth.to_device(wl) for _ in range(18)]
+        for x, w, s, b, _ in sets:
+            kernels.quantized_matmul(x, w, s, b, group_size=64, bits=wl.bits)
+        torch.cuda.synchronize()
+        buf = np.zeros((256, 12, 16), dtype=np.uint64)
+        rc = lib.qmm_debug_stamps(buf.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(buf.nbytes))
+        if rc:
+            raise RuntimeError(f"qmm_debug_stamps: {rc}")
+        st = buf.astype(np.int64)
+        us = (st - st[:, :, 0].min()) / 100.0               # the stamp clock runs at 100 MHz
+        med = np.median(us, axis=0)
+        rows_a_workgroup = -(-wl.N // 256)
+        tiles = min(4, -(-rows_a_workgroup // 16))
+        def pick(names, row, upto):
+            return {n: round(float(row[i]), 2) for i, n in enumerate(names) if n and i < upto}
+        out[f"M={m}"] = {
+            "compute wavefronts 0-3 (first of their SIMD)": pick(compute, med[0:4].mean(axis=0), 3 + 2 * tiles),
+            "compute wavefronts 4-7 (second of their SIMD)": pick(compute, med[4:8].mean(axis=0), 3 + 2 * tiles),
+            "loaders": {**pick(loader, med[8:12].mean(axis=0), 3 + 3 * tiles), "end": round(float(med[8:12, 15].mean()), 2)},
+        }
+    return out
+
+
 def main(argv):
     path = argv[1]
     total = sum(r[7] for r in kernel_stats(path)) or 1
