@@ -731,10 +731,53 @@ def share(leaves, w, scales, biases, perm, gs, bits, mode) -> Pack:
 _BUILT = {}
 
 
-def fingerprint(m):
+def _canon_callee(name, module, stack):
+    """A private function as text that does not depend on names: its body in
+    program order, values by position."""
+    name = str(name).lstrip("@")
+    if module is None or name not in module.funcs:
+        raise Reject("callee not found")
+    if name in stack:
+        raise Reject("recursive callee")
+
+    def closed(v):
+        raise Reject("a function body reads a value from outside")
+    return _canon_block(module.funcs[name].body, module, closed, stack + (name,))
+
+
+def _canon_block(block, module, outer, stack):
+    ids = {a: f"b{i}:{a.type}" for i, a in enumerate(block.args)}
+
+    def look(v):
+        return ids[v] if v in ids else outer(v)
+    lines = []
+    for n, o in enumerate(block.ops):
+        lines.append(_canon_op(o, n, [look(x) for x in o.operands], module, look, stack))
+        for i, r in enumerate(o.results):
+            ids[r] = f"%{n}.{i}"
+    return ";".join(lines)
+
+
+def _canon_op(o, n, opnds, module, look, stack):
+    """One op of a canonical text: name, attributes, what it calls and the
+    regions it holds by *content* (a callee's name is not part of the key, its
+    body is: two programs that differ in the name are the same chain, two that
+    differ in the body are not), operands, result types."""
+    attrs = dict(o.attrs)
+    called = ""
+    for ref in ("callee", "decomposition"):
+        if ref in attrs and (o.name == "func.call" or ref == "decomposition"):
+            called += "{" + _canon_callee(attrs.pop(ref), module, stack) + "}"
+    regions = "".join("{" + _canon_block(r, module, look, stack) + "}" for r in o.regions)
+    return (f"{n}={o.name}{sorted((k, repr(val)) for k, val in attrs.items())}{called}{regions}"
+            f"({','.join(opnds)})->{[str(r.type) for r in o.results]}")
+
+
+def fingerprint(m, module=None):
     """Canonical serialization of the reconstruction subtree: ops in a
-    deterministic post-order, operands by position, leaves by argument slot
-    (reference qmm.py:2022-2268 keeps the same two-part key)."""
+    deterministic post-order, operands by position, leaves by argument slot,
+    callees and regions by their bodies (reference qmm.py:2022-2268 keeps the
+    same two-part key)."""
     if m.fp is not None:
         return m.fp
     ids, lines = {}, []
@@ -752,9 +795,8 @@ def fingerprint(m):
         if o.name in OPAQUE_OPS:
             raise Reject("opaque op in subtree")
         opnds = [visit(x) for x in o.operands]
-        attrs = sorted((k, repr(val)) for k, val in o.attrs.items())
         n = len(lines)
-        lines.append(f"{n}={o.name}{attrs}({','.join(opnds)})->{[str(r.type) for r in o.results]}")
+        lines.append(_canon_op(o, n, opnds, module, visit, ()))
         for i, r in enumerate(o.results):
             ids[r] = f"%{n}.{i}"
         return ids[v]
@@ -771,10 +813,10 @@ def fingerprint(m):
     return m.fp
 
 
-def _build_key(m, args):
+def _build_key(m, args, module=None):
     if not BUILD_CACHE:
         return None, None
-    fp = fingerprint(m)
+    fp = fingerprint(m, module)
     if not fp:
         return None, None
     text, slots = fp
@@ -816,7 +858,7 @@ def pack_for(interp, m, args, check=lambda m: None):
         del m.packs[MAX_PACKS:]
         return pk
 
-    key, keyleaves = _build_key(m, args)
+    key, keyleaves = _build_key(m, args, getattr(interp, "module", None))
     if key is not None:
         elsewhere = _cached_build(key, keyleaves)
         if elsewhere is not None:

@@ -123,6 +123,23 @@ func.func public @main(%packed: {_t((k, n // 2), "i8")}, %scale: {_t((n,), el)},
 """
 
 
+def dense_i4_perchannel(k, n, m, el="bf16"):
+    """x [M,K] @ (convert(w : i4 [K,N]) * scale[N]): weights stored as four-bit
+    integers with one scale per output channel (the chain of reference
+    tests/test_qmm.py:342-358)."""
+    return f"""
+module @jit_i4 {{
+  func.func public @main(%w: {_t((k, n), "i4")}, %s: {_t((n,), el)}, %x: {_t((m, k), el)}) -> {_t((m, n), el)} {{
+    %wf = stablehlo.convert %w : ({_t((k, n), "i4")}) -> {_t((k, n), el)}
+    %sb = stablehlo.broadcast_in_dim %s, dims = [1] : ({_t((n,), el)}) -> {_t((k, n), el)}
+    %wq = stablehlo.multiply %wf, %sb : {_t((k, n), el)}
+    %y = stablehlo.dot_general %x, %wq, contracting_dims = [1] x [0], precision = [DEFAULT, DEFAULT] : ({_t((m, k), el)}, {_t((k, n), el)}) -> {_t((m, n), el)}
+    return %y : {_t((m, n), el)}
+  }}
+}}
+"""
+
+
 def _e8m0_table_hex():
     with np.errstate(over="ignore"):
         t = np.ldexp(np.ones(256), np.arange(256) - 127).astype(np.float32)

@@ -142,6 +142,25 @@ def test_perchannel_divide_form():
     np.testing.assert_allclose(got, (q.astype(np.float32) / scale).T, rtol=2e-7)
 
 
+def test_int4_typed_weights_with_a_per_channel_scale():
+    """Weights stored with the four-bit integer element type and one scale per
+    output channel (reference tests/test_qmm.py:342-358): four-bit codes, one
+    group spanning as much of K as a legal group size allows, exact."""
+    k, n, m = 128, 64, 2
+    rng = np.random.default_rng(50)
+    codes = rng.integers(-8, 8, size=(k, n)).astype(np.int8)
+    scale = T.bf16_round((rng.random(n).astype(np.float32) + 0.5) * 0.02)
+    ex = engine.compile_program(T.dense_i4_perchannel(k, n, m))
+    st = qmm.analyze(ex.interp)
+    assert len(st.matches) == 1
+    args = [I.from_numpy(codes, "i4"), I.from_numpy(scale, "bf16"), I.from_numpy(np.zeros((m, k), np.float32), "bf16")]
+    qmm.prologue(ex.interp, args)
+    assert qmm.stats()["recognized"] == 1 and qmm.stats()["packs"] == 1 and qmm.stats()["fallbacks"] == 0
+    pk = st.matches[0].packs[0]
+    assert pk.bits == 4 and pk.gs == 128
+    np.testing.assert_array_equal(dequant_pack(pk), (codes.astype(np.float32) * scale).T)
+
+
 @pytest.mark.parametrize("el", ["bf16", "f32"])
 def test_mxfp4_chain_packs_bit_exactly(el):
     n, k, t = 48, 128, 5
@@ -207,6 +226,59 @@ def test_interleaved_groups_are_fused_through_a_permutation():
     np.testing.assert_allclose(dequant_pack(pk), wref.T[:, perm], rtol=1e-5, atol=1e-7)
 
 
+def test_identity_permutation_is_the_zero_overhead_path():
+    """Groups that are already contiguous carry no permutation: three packed
+    values, no `take` on the activations (reference tests/test_qmm.py:575-586)."""
+    k, n, m = 256, 128, 4
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, 128, seed=124)
+    x = np.zeros((m, k), np.float32)
+    ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+    st = qmm.analyze(ex.interp)
+    qmm.prologue(ex.interp, host_args_dense(packed, scale, zero, g_idx, x))
+    mt = st.matches[0]
+    assert qmm.stats()["packs"] == 1 and qmm.stats()["perms"] == 0
+    assert not mt.has_perm and mt.nvals == 3 and mt.packs[0].perm is None
+    np.testing.assert_allclose(dequant_pack(mt.packs[0]), wref.T, rtol=1e-5, atol=1e-7)
+
+
+def test_shuffled_g_idx_is_regrouped():
+    """A g_idx that scatters each group's members across K still has equal
+    groups of identical (scale, zero) columns: the permutation recovers them
+    (reference tests/test_qmm.py:606-619)."""
+    k, n, m, block = 256, 64, 2, 128
+    rng = np.random.default_rng(12)
+    g_idx = rng.permutation(np.arange(k) // block).astype(np.float32)
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, block, seed=13, g_idx=g_idx)
+    ex = engine.compile_program(T.dense_sub(k, n, k // block, m))
+    st = qmm.analyze(ex.interp)
+    qmm.prologue(ex.interp, host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32)))
+    assert qmm.stats()["packs"] == 1 and qmm.stats()["perms"] == 1 and qmm.stats()["fallbacks"] == 0
+    pk = st.matches[0].packs[0]
+    perm = np.asarray(pk.perm)
+    assert sorted(perm.tolist()) == list(range(k))
+    np.testing.assert_allclose(dequant_pack(pk), wref.T[:, perm], rtol=1e-5, atol=1e-7)
+
+
+def test_second_weight_set_with_a_different_permutation():
+    """Two weight sets whose groups interleave differently through one
+    executable: the permutation is a packed value of the pack, so the second
+    set must get its own (reference tests/test_qmm.py:472-501)."""
+    k, n, m, ng = 256, 64, 2, 2
+    ex = engine.compile_program(T.dense_sub(k, n, ng, m))
+    st = qmm.analyze(ex.interp)
+    x = np.zeros((m, k), np.float32)
+    perms, wrefs, held = [], [], []
+    for seed, g_idx in ((100, (np.arange(k) % ng)), (110, ((np.arange(k) // 2) % ng))):
+        q, packed, scale, zero, g, wref = T.quantize(k, n, k // ng, seed=seed, g_idx=g_idx.astype(np.float32))
+        held.append(host_args_dense(packed, scale, zero, g, x))
+        qmm.prologue(ex.interp, held[-1])
+        pk = st.matches[0].packs[0]
+        perms.append(np.asarray(pk.perm).copy())
+        np.testing.assert_allclose(dequant_pack(pk), wref.T[:, perms[-1]], rtol=1e-5, atol=1e-7)
+    assert qmm.stats()["packs"] == 2 and qmm.stats()["perms"] == 2
+    assert not np.array_equal(perms[0], perms[1])
+
+
 # --------------------------------------------------------------- fallbacks ---
 
 def _one_fallback(ex, args):
@@ -223,6 +295,16 @@ def test_group_of_16_falls_back():
     x = np.zeros((m, k), np.float32)
     ex = engine.compile_program(T.dense_sub(k, n, k // 16, m))
     _one_fallback(ex, host_args_dense(packed, scale, zero, g_idx, x))
+
+
+def test_uneven_group_sizes_fall_back():
+    """Groups of 129 and 127 columns line up on no legal group boundary: the
+    literal chain runs (reference tests/test_qmm.py:622-634)."""
+    k, n, m = 256, 64, 2
+    g_idx = (np.arange(k) >= 129).astype(np.float32)
+    q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 128, seed=13, g_idx=g_idx)
+    ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+    _one_fallback(ex, host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32)))
 
 
 def test_off_grid_e2m1_value_falls_back():
@@ -325,6 +407,96 @@ def test_build_cache_serves_a_second_executable_over_the_same_buffers():
     ex3 = engine.compile_program(T.dense_sub(k, n, 2, m))
     qmm.prologue(ex3.interp, host_args_dense(packed.copy(), scale, zero, g_idx, np.zeros((m, k), np.float32)))
     assert qmm.stats()["packs"] == 2 and qmm.stats()["build_hits"] == 1
+
+
+def test_different_weight_content_misses_the_build_cache():
+    """Same shapes and types, different bytes in different buffers: the key
+    names buffers by identity, so nothing is reused and each executable's pack
+    holds its own weight (reference tests/test_qmm.py:1213-1243)."""
+    k, n, m = 128, 64, 2
+    packs_seen = []
+    for seed in (42, 43):
+        q, packed, scale, zero, g_idx, wref = T.quantize(k, n, 64, seed=seed, bf16=False)
+        ex = engine.compile_program(T.dense_sub(k, n, 2, m, el="f32"))
+        st = qmm.analyze(ex.interp)
+        args = host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32), el="f32")
+        qmm.prologue(ex.interp, args)
+        packs_seen.append((st.matches[0].packs[0], wref, args))
+    assert qmm.stats()["build_hits"] == 0 and qmm.stats()["packs"] == 2
+    for pk, wref, _ in packs_seen:
+        np.testing.assert_allclose(dequant_pack(pk), wref.T, rtol=1e-5, atol=1e-7)   # f32 scales, nonzero zero points: the exactness matrix of reference tests/test_qmm.py:117-132
+    assert packs_seen[0][0].w is not packs_seen[1][0].w
+
+
+def test_one_different_constant_misses_the_build_cache():
+    """Same buffers, same shapes, one constant of the chain apart (the group
+    count the indices are clamped to): a wrong hit would hand the second
+    executable the first one's weight (reference tests/test_qmm.py:1247-1275)."""
+    k, n, m = 128, 64, 2
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, 64, seed=45)
+    args = host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32))
+    text = T.dense_sub(k, n, 2, m)
+    other = text.replace("%gns = stablehlo.constant dense<2>", "%gns = stablehlo.constant dense<3>")
+    assert other != text
+    ex1, ex2 = engine.compile_program(text), engine.compile_program(other)
+    qmm.prologue(ex1.interp, args)
+    qmm.prologue(ex2.interp, args)
+    assert qmm.stats()["build_hits"] == 0 and qmm.stats()["packs"] == 2
+
+
+def test_the_fused_dot_is_what_the_cost_model_charges():
+    """`emit_reads` names exactly the activation, and `emit_bytes` is the
+    packed operands plus activation and result -- far below the literal chain's
+    traffic (reference tests/test_qmm.py:930-957 through qmm.py:2424-2466)."""
+    k, n, m = 128, 128, 1
+    q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 128, seed=40)
+    ex = engine.compile_program(T.dense_sub(k, n, 1, m))
+    st = qmm.analyze(ex.interp)
+    qmm.prologue(ex.interp, host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32)))
+    mt = st.matches[0]
+    assert tuple(qmm.emit_reads(mt)) == (mt.lhs,)
+    fused = qmm.emit_bytes(mt)
+    literal = 3 * k * n * 2                                   # the dequantized weight written, re-read and multiplied
+    assert 0 < fused < literal // 4, (fused, literal)
+
+
+def test_fingerprint_reads_callee_bodies_not_their_names():
+    """Two programs that differ only in the name of a private callee are the
+    same weight chain (a build hit over the same buffers); one constant inside
+    the callee's body apart, they are not (reference
+    tests/test_qmm_mxfp4.py:895-928)."""
+    n, k, t = 64, 128, 2
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=7)
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(np.zeros((t, k), np.float32), "bf16")]
+    text = T.dense_mxfp4_rows(n, k, t)
+    renamed = text.replace("@_take", "@_take_17")
+    wrap = "%ns = stablehlo.constant dense<16> : tensor<i32>"
+    assert renamed != text and wrap in text
+    other_body = text.replace(wrap, "%ns = stablehlo.constant dense<32> : tensor<i32>")   # what a negative index wraps by
+    ex1, ex2, ex3 = (engine.compile_program(x) for x in (text, renamed, other_body))
+    qmm.prologue(ex1.interp, args)
+    qmm.prologue(ex2.interp, args)
+    assert qmm.stats()["packs"] == 1 and qmm.stats()["build_hits"] == 1
+    qmm.prologue(ex3.interp, args)
+    assert qmm.stats()["packs"] == 2 and qmm.stats()["build_hits"] == 1
+
+
+def test_identical_mxfp4_weights_in_two_buffers_share_one_pack():
+    """Content-addressed sharing: the same bytes arriving in other buffers are
+    packed again (identity misses) but end up aliasing the first pack's arrays;
+    different bytes do not (reference tests/test_qmm_mxfp4.py:423-480)."""
+    n, k, t = 64, 128, 2
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=8)
+    _, blocks2, sb2, _ = T.random_mxfp4((n, k), seed=9)
+    x = I.from_numpy(np.zeros((t, k), np.float32), "bf16")
+    text = T.dense_mxfp4(n, k, t)
+    exs = [engine.compile_program(text) for _ in range(3)]
+    qmm.prologue(exs[0].interp, [I.from_numpy(blocks), I.from_numpy(sb), x])
+    qmm.prologue(exs[1].interp, [I.from_numpy(blocks.copy()), I.from_numpy(sb.copy()), x])
+    qmm.prologue(exs[2].interp, [I.from_numpy(blocks2), I.from_numpy(sb2), x])
+    assert qmm.stats()["packs"] == 3 and qmm.stats()["shared"] == 1
+    p0, p1, p2 = (e.interp._qmm.matches[0].packs[0] for e in exs)
+    assert p1.w is p0.w and p1.scales is p0.scales and p2.w is not p0.w
 
 
 # --------------------------------------------------- decode loop, run path ---
@@ -644,6 +816,47 @@ def test_a_router_that_is_not_a_top_k_scatter_is_refused():
         "return %out : tensor<3x64xf32>", "return %out, %y : tensor<3x64xf32>, tensor<4x3x64xf32>")
     st = qmm.analyze(engine.compile_program(shared).interp)
     assert st.moe == []
+
+
+def test_near_misses_of_the_expert_sum_are_refused():
+    """The root must be a sum over experts of outputs times top-k scores
+    (reference tests/test_moe.py:328-385): a max over experts, and scores that
+    are a dense function of the logits, leave the block dense."""
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    root = "%out = stablehlo.reduce(%ys init: %zero) applies stablehlo.add across dimensions = [0]"
+    assert root in text
+    as_max = text.replace(root, "%out = stablehlo.reduce(%ys init: %ninf) applies stablehlo.maximum across dimensions = [0]")
+    st = qmm.analyze(engine.compile_program(as_max).interp)
+    assert st.moe == [] and len(st.roots) == 2 and not any(m.absorbed for m in st.matches)
+    # every expert really routed: the scores are exp(logits), no selection anywhere near them
+    scores = f"%s = stablehlo.reduce(%hw init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<{Tk}x{K}x{E}xf32>, tensor<f32>) -> tensor<{Tk}x{E}xf32>"
+    assert scores in text
+    dense = text.replace(scores, f"%s = stablehlo.exponential %logits : tensor<{Tk}x{E}xf32>")
+    st = qmm.analyze(engine.compile_program(dense).interp)
+    assert st.moe == [] and len(st.roots) == 2
+
+
+def test_values_around_the_expert_sum_do_not_stop_the_dispatch():
+    """The dense scores also returned (they then stay computed), and a shared
+    branch added outside the sum (reference tests/test_moe.py:157-187): the
+    block is still one dispatch."""
+    from metaljax_amd import moe
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    sig, ret = f"-> tensor<{Tk}x{H}xf32> {{", f"return %out : tensor<{Tk}x{H}xf32>"
+    assert sig in text and ret in text
+    with_scores = text.replace(sig, f"-> (tensor<{Tk}x{H}xf32>, tensor<{Tk}x{E}xf32>) {{", 1).replace(
+        ret, f"return %out, %s : tensor<{Tk}x{H}xf32>, tensor<{Tk}x{E}xf32>")
+    ex = engine.compile_program(with_scores)
+    st = qmm.analyze(ex.interp)
+    assert len(st.moe) == 1
+    by_name = {v.name: v for b in ir.walk_blocks(ex.interp.main.body) for o in b.ops for v in o.results}
+    g = st.moe[0]
+    assert by_name["s"] not in g.skip_keys and by_name["ys"] in g.skip_keys      # the scores live on, the dense product does not
+    shared = text.replace(ret, f"%side = stablehlo.tanh %x : tensor<{Tk}x{H}xf32>\n    %both = stablehlo.add %out, %side : tensor<{Tk}x{H}xf32>\n    return %both : tensor<{Tk}x{H}xf32>")
+    st = qmm.analyze(engine.compile_program(shared).interp)
+    assert len(st.moe) == 1 and st.moe[0].out_shape == [Tk, H]
 
 
 def test_a_dispatch_that_fails_its_check_runs_densely(monkeypatch):
