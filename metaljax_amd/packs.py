@@ -758,19 +758,33 @@ def _canon_block(block, module, outer, stack):
     return ";".join(lines)
 
 
+# A constant of more than this many elements is a weight baked into the
+# program: serializing it costs more than the build the cache would save, so
+# such a chain is built every time (reference qmm.py:1965-1975); the same for
+# any attribute whose printed form is very long.
+FP_DENSE_ELEMS = 1024
+FP_ATTR_CHARS = 1 << 16
+
+
 def _canon_op(o, n, opnds, module, look, stack):
     """One op of a canonical text: name, attributes, what it calls and the
     regions it holds by *content* (a callee's name is not part of the key, its
     body is: two programs that differ in the name are the same chain, two that
     differ in the body are not), operands, result types."""
     attrs = dict(o.attrs)
+    if o.name == "stablehlo.constant" and o.results:
+        shape = getattr(o.results[0].type, "shape", None)
+        if shape is not None and int(np.prod(shape, dtype=np.int64)) > FP_DENSE_ELEMS:
+            raise Reject(f"a constant of {int(np.prod(shape, dtype=np.int64))} elements")
     called = ""
     for ref in ("callee", "decomposition"):
         if ref in attrs and (o.name == "func.call" or ref == "decomposition"):
             called += "{" + _canon_callee(attrs.pop(ref), module, stack) + "}"
     regions = "".join("{" + _canon_block(r, module, look, stack) + "}" for r in o.regions)
-    return (f"{n}={o.name}{sorted((k, repr(val)) for k, val in attrs.items())}{called}{regions}"
-            f"({','.join(opnds)})->{[str(r.type) for r in o.results]}")
+    shown = sorted((k, repr(val)) for k, val in attrs.items())
+    if any(len(text) > FP_ATTR_CHARS for _, text in shown):
+        raise Reject("an attribute too long to serialize")
+    return f"{n}={o.name}{shown}{called}{regions}({','.join(opnds)})->{[str(r.type) for r in o.results]}"
 
 
 def fingerprint(m, module=None):

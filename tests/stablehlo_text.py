@@ -83,6 +83,40 @@ module @jit_dense_sub {{
 """
 
 
+def _dense_sub_with_dot(k, n, ng, el, x_shape, out_shape, dot_lines):
+    """`dense_sub`'s dequantization chain (it defines %wq [K, N]) with another
+    activation shape and another tail: `dot_lines` must define %y."""
+    text = dense_sub(k, n, ng, 1, el)
+    x_old, out_old = _t((1, k), el), _t((1, n), el)
+    head, dot, tail = text.partition("    %y = stablehlo.dot_general")
+    assert dot
+    head = head.replace(f"%x: {x_old}) -> {out_old} {{", f"%x: {_t(x_shape, el)}) -> {_t(out_shape, el)} {{")
+    return head + dot_lines + f"\n    return %y : {_t(out_shape, el)}\n  }}\n}}\n"
+
+
+def einsum_sub(d, heads, head_dim, ng, b, t, el="bf16"):
+    """einsum("btd,dnh->btnh", x, reshape(dequant(W), [d, n, h])): the weight
+    is reshaped after the chain and N has two axes (the EinsumDense chain of
+    reference tests/test_qmm.py:226-236, :329-339)."""
+    n = heads * head_dim
+    w2, w3 = _t((d, n), el), _t((d, heads, head_dim), el)
+    x, out = (b, t, d), (b, t, heads, head_dim)
+    return _dense_sub_with_dot(d, n, ng, el, x, out, f"""    %w3 = stablehlo.reshape %wq : ({w2}) -> {w3}
+    %y = stablehlo.dot_general %x, %w3, contracting_dims = [2] x [0], precision = [DEFAULT, DEFAULT] : ({_t(x, el)}, {w3}) -> {_t(out, el)}""")
+
+
+def einsum_out_proj(nh, h, d, ng, b, t, el="bf16"):
+    """einsum("btnh,nhd->btd", x, reshape(dequant(W), [n, h, d])) as jax lowers
+    it, `contracting_dims = [3, 2] x [1, 0]`: the pairing is reversed, so the
+    canonical K axis runs h-major over a weight stored (and grouped) n-major
+    (reference tests/test_qmm.py:208-223, :409-418)."""
+    rows = nh * h
+    w2, w3 = _t((rows, d), el), _t((nh, h, d), el)
+    x, out = (b, t, nh, h), (b, t, d)
+    return _dense_sub_with_dot(rows, d, ng, el, x, out, f"""    %w3 = stablehlo.reshape %wq : ({w2}) -> {w3}
+    %y = stablehlo.dot_general %x, %w3, contracting_dims = [3, 2] x [1, 0], precision = [DEFAULT, DEFAULT] : ({_t(x, el)}, {w3}) -> {_t(out, el)}""")
+
+
 def dense_i8_codes(k, n, ng, m, el="bf16"):
     """dense_sub with the codes stored as plain i8 [K, N] (no nibble unpack)."""
     text = dense_sub(k, n, ng, m, el)

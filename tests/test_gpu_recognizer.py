@@ -190,6 +190,39 @@ def test_mxfp4_experts_gathered(E, K, Tk):
     assert qmm.stats()["packs"] == 2 and moe.stats()["dispatches"] == 2
 
 
+def test_an_expert_nobody_selects_is_never_evaluated():
+    """The one intended divergence from the dense block (reference
+    tests/test_moe.py:428-458): an expert whose output is not finite and whose
+    router logit keeps every token away from it gives NaN in the dense sum
+    (inf times an exact zero) and nothing at all in the dispatch, which never
+    evaluates it."""
+    import stablehlo_text as S
+    moe.reset_stats()
+    E, K, Tk, H, Ii = 4, 2, 2, 64, 32
+    rng = np.random.default_rng(37)
+    gu_c, gu_s, gu_ref = S.make_mxfp4_experts(2 * Ii, H, E, seed=37)
+    d_c, d_s, d_ref = S.make_mxfp4_experts(H, Ii, E, seed=38)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    wr = (rng.standard_normal((H, E)) / 8).astype(np.float32)
+    br = rng.standard_normal(E).astype(np.float32)
+    bgu = (rng.standard_normal((E, 2 * Ii)) / 8).astype(np.float32)
+    bd = (rng.standard_normal((E, H)) / 8).astype(np.float32)
+    bd[3] = np.inf
+    br[3] = -1e4
+    text = S.moe_block_mxfp4(E, Tk, H, Ii, K)
+    args = [I.from_numpy(a) for a in (x, wr, br, gu_c, gu_s, d_c, d_s, bgu, bd)]
+    (buf,) = engine.execute(engine.compile_program(text), args)
+    assert moe.stats()["recognized"] == 1 and moe.stats()["dispatches"] == 1 and moe.stats()["fallbacks"] == 0
+    got = buf.data.float().cpu().numpy()
+    lit = I.host(I.Interpreter(text).run(args)[0]).a
+    assert np.isnan(lit).any(), "the dense block should carry the NaN"
+    assert np.isfinite(got).all(), "the dispatch should stay finite"
+    bd0 = bd.copy()
+    bd0[3] = 0.0
+    want = S.moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd0, K)
+    np.testing.assert_allclose(got, want, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+
+
 def test_gather_qmm_with_several_rows_per_pair():
     """x [T, M, K]: every pair multiplies M rows (mx.gather_qmm's general
     form, reference src/metaljax/moe.py:1293-1301)."""

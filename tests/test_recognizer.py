@@ -226,6 +226,53 @@ def test_interleaved_groups_are_fused_through_a_permutation():
     np.testing.assert_allclose(dequant_pack(pk), wref.T[:, perm], rtol=1e-5, atol=1e-7)
 
 
+def _fused_and_literal(monkeypatch, text, args):
+    """The program's first result with the recognized dot replaced by the
+    oracle-backed stand-in, and from the literal chain."""
+    literal = I.host(I.Interpreter(text).run(args)[0]).a
+    monkeypatch.setattr(qmm, "emit", oracle_emit)
+    ex = engine.compile_program(text)
+    st = qmm.analyze(ex.interp)
+    qmm.prologue(ex.interp, args)
+    (y,) = ex.interp.run(args)
+    return st, I.host(y).a, literal
+
+
+def test_einsum_with_two_output_axes(monkeypatch):
+    """`btd,dnh->btnh`: the weight is reshaped to [d, n, h] behind the chain
+    and the dot keeps both N axes (reference tests/test_qmm.py:329-339)."""
+    d, heads, hd, b, t = 256, 4, 32, 1, 2
+    q, packed, scale, zero, g_idx, wref = T.quantize(d, heads * hd, 128, seed=7)
+    x = T.bf16_round(np.random.default_rng(8).standard_normal((b, t, d)).astype(np.float32) * 0.3)
+    st, fused, literal = _fused_and_literal(monkeypatch, T.einsum_sub(d, heads, hd, 2, b, t),
+                                            host_args_dense(packed, scale, zero, g_idx, x))
+    assert qmm.stats()["recognized"] == 1 and qmm.stats()["packs"] == 1 and qmm.stats()["perms"] == 0
+    mt = st.matches[0]
+    assert (mt.M, mt.K, mt.N) == (b * t, d, heads * hd) and list(mt.nshape) == [heads, hd]
+    exact = np.einsum("btd,dnh->btnh", x, wref.reshape(d, heads, hd))
+    assert fused.shape == exact.shape
+    assert np.abs(fused - exact).max() <= 1.5 * np.abs(literal - exact).max() + 1e-6
+
+
+@pytest.mark.parametrize("nh,h,block", [(8, 32, 128), (4, 64, 64), (16, 16, 128)])
+def test_einsum_out_projection_interleaved_groups(monkeypatch, nh, h, block):
+    """`btnh,nhd->btd` with the reversed pairing jax emits: the quantization
+    groups of the n-major weight arrive interleaved along the canonical K, and
+    a permutation of K (the same one on the activations) makes them contiguous
+    (reference tests/test_qmm.py:409-426)."""
+    d, b, t = 64, 1, 3
+    rows = nh * h
+    q, packed, scale, zero, g_idx, wref = T.quantize(rows, d, block, seed=100)
+    x = T.bf16_round(np.random.default_rng(9).standard_normal((b, t, nh, h)).astype(np.float32) * 0.3)
+    st, fused, literal = _fused_and_literal(monkeypatch, T.einsum_out_proj(nh, h, d, rows // block, b, t),
+                                            host_args_dense(packed, scale, zero, g_idx, x))
+    stats = qmm.stats()
+    assert stats["recognized"] == 1 and stats["packs"] == 1 and stats["fallbacks"] == 0
+    assert stats["perms"] == 1                              # n-major groups, h-major K: always interleaved
+    exact = np.einsum("btnh,nhd->btd", x, wref.reshape(nh, h, d))
+    assert np.abs(fused - exact).max() <= 1.5 * np.abs(literal - exact).max() + 1e-6
+
+
 def test_identity_permutation_is_the_zero_overhead_path():
     """Groups that are already contiguous carry no permutation: three packed
     values, no `take` on the activations (reference tests/test_qmm.py:575-586)."""
@@ -479,6 +526,22 @@ def test_fingerprint_reads_callee_bodies_not_their_names():
     assert qmm.stats()["packs"] == 1 and qmm.stats()["build_hits"] == 1
     qmm.prologue(ex3.interp, args)
     assert qmm.stats()["packs"] == 2 and qmm.stats()["build_hits"] == 1
+
+
+def test_a_big_constant_declines_the_build_cache(monkeypatch):
+    """A decode table too big to serialize: no cache entry, no wrong reuse,
+    the chain is simply built for every executable (reference
+    tests/test_qmm_mxfp4.py:858-876; here the E2M1 table is put over the limit)."""
+    monkeypatch.setattr(packs, "FP_DENSE_ELEMS", 8)
+    n, k = 64, 128
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=78)
+    args = [I.from_numpy(blocks), I.from_numpy(sb)]
+    for t in (2, 5):
+        ex = engine.compile_program(T.dense_mxfp4(n, k, t))
+        qmm.prologue(ex.interp, args + [I.from_numpy(np.zeros((t, k), np.float32), "bf16")])
+        np.testing.assert_array_equal(np.asarray(ex.interp._qmm.matches[0].packs[0].w), O.pack_codes(codes, 4))
+    st = qmm.stats()
+    assert st["build_declines"] == 2 and st["build_hits"] == 0 and st["packs"] == 2
 
 
 def test_identical_mxfp4_weights_in_two_buffers_share_one_pack():
@@ -857,6 +920,46 @@ def test_values_around_the_expert_sum_do_not_stop_the_dispatch():
     shared = text.replace(ret, f"%side = stablehlo.tanh %x : tensor<{Tk}x{H}xf32>\n    %both = stablehlo.add %out, %side : tensor<{Tk}x{H}xf32>\n    return %both : tensor<{Tk}x{H}xf32>")
     st = qmm.analyze(engine.compile_program(shared).interp)
     assert len(st.moe) == 1 and st.moe[0].out_shape == [Tk, H]
+
+
+def test_the_one_pass_dead_sweep_agrees_with_a_fixpoint(monkeypatch):
+    """`sweep_dead` walks the block once from the last op to the first; the
+    argument for that is that it finds what rescanning to a fixpoint finds
+    (reference tests/test_moe.py:609-636).  Here both run on the real block and
+    must give the same set, and the sweep must add something."""
+    from metaljax_amd import moe
+    seen = []
+    one_pass = moe.sweep_dead
+
+    def both(block, skip, g):
+        before = set(skip)
+        got = set(one_pass(block, set(skip), g))
+        keep, todo = set(), list(g.reads) + [g.router.indices, g.router.weights]
+        while todo:
+            v = todo.pop()
+            if v not in keep:
+                keep.add(v)
+                if moe._producer(v) is not None:
+                    todo.extend(moe._producer(v).operands)
+        ref, changed = set(before), True
+        while changed:
+            changed = False
+            for op in block.ops:
+                key = moe.op_key(op)
+                if (key is None or key in ref or key is g.key or op.name in moe.OPAQUE_OPS
+                        or (op.regions and op.name != "stablehlo.reduce") or any(r in keep for r in op.results)):
+                    continue
+                readers = [u for r in op.results for u in r.uses]
+                if readers and all(moe.op_key(u) is g.key or moe.op_key(u) in ref for u in readers):
+                    ref.add(key)
+                    changed = True
+        assert got == ref, (got - ref, ref - got)
+        seen.append((len(before), len(got)))
+        return one_pass(block, skip, g)
+
+    monkeypatch.setattr(moe, "sweep_dead", both)
+    st = qmm.analyze(engine.compile_program(T.moe_block_mxfp4(4, 5, 64, 32, 2)).interp)
+    assert len(st.moe) == 1 and seen and any(after > before for before, after in seen), seen
 
 
 def test_a_dispatch_that_fails_its_check_runs_densely(monkeypatch):
