@@ -368,19 +368,29 @@ def affine_grouped_data(n, k, gs, seed, interleave=False):
     return q, scale, zero, ref
 
 
-def dense_mxfp4_rows(n, k, t, el="bf16"):
+def dense_mxfp4_rows(n, k, t, el="bf16", e=None):
     """dense_mxfp4 as jax lowers `jnp.take`: the E2M1 decode is a private
     @_take callee (index wrap with full-extent splats, then a gather that
-    batches over the indices), and every op keeps N as the leading axis
-    (reference tests/test_qmm_mxfp4.py:282-298, :908-916)."""
+    batches over the indices), and every op keeps the weight's leading axis
+    leading (reference tests/test_qmm_mxfp4.py:282-298, :908-916).  With `e`
+    the weight is [E, N, K] and the product batches over the experts."""
     h = k // 2
+    L = () if e is None else (e,)
+    r = len(L)                                    # axes in front of N
     vals = ", ".join(("-" if np.signbit(v) else "") + f"{abs(v):.6e}"
                      for v in np.array(list(E2M1) + [-v for v in E2M1], np.float64))
-    bl, sb = _t((n, h), "ui8"), _t((n, k // 32), "ui8")
-    idx, idx3 = _t((n, k), "i32"), _t((n, k, 1), "i32")
+    bl, sb = _t(L + (n, h), "ui8"), _t(L + (n, k // 32), "ui8")
+    idx, idx3 = _t(L + (n, k), "i32"), _t(L + (n, k, 1), "i32")
+    dims = ", ".join(str(i) for i in range(r + 2))
+    if e is None:
+        xs, ys = (t, k), (t, n)
+        dot = f"contracting_dims = [1] x [1]"
+    else:
+        xs, ys = (e, t, k), (e, t, n)
+        dot = f"batching_dims = [0] x [0], contracting_dims = [2] x [2]"
     return f"""
 module @jit_dense_mxfp4_rows {{
-  func.func public @main(%blocks: {bl}, %scales: {sb}, %x: {_t((t, k), el)}) -> {_t((t, n), el)} {{
+  func.func public @main(%blocks: {bl}, %scales: {sb}, %x: {_t(xs, el)}) -> {_t(ys, el)} {{
     %vt = stablehlo.constant dense<[{vals}]> : tensor<16x{el}>
     %stab = stablehlo.constant dense<"{_e8m0_table_hex()}"> : tensor<256xf32>
     %m15s = stablehlo.constant dense<15> : tensor<ui8>
@@ -389,34 +399,34 @@ module @jit_dense_mxfp4_rows {{
     %s4 = stablehlo.broadcast_in_dim %s4s, dims = [] : (tensor<ui8>) -> {bl}
     %lo = stablehlo.and %blocks, %m15 : {bl}
     %hi = stablehlo.shift_right_logical %blocks, %s4 : {bl}
-    %lo3 = stablehlo.reshape %lo : ({bl}) -> {_t((n, h, 1), "ui8")}
-    %hi3 = stablehlo.reshape %hi : ({bl}) -> {_t((n, h, 1), "ui8")}
-    %nb = stablehlo.concatenate %lo3, %hi3, dim = 2 : ({_t((n, h, 1), "ui8")}, {_t((n, h, 1), "ui8")}) -> {_t((n, h, 2), "ui8")}
-    %nib = stablehlo.reshape %nb : ({_t((n, h, 2), "ui8")}) -> {_t((n, k), "ui8")}
-    %ni = stablehlo.convert %nib : ({_t((n, k), "ui8")}) -> {idx}
-    %v = func.call @_take(%vt, %ni) : (tensor<16x{el}>, {idx}) -> {_t((n, k), el)}
-    %sbi0 = stablehlo.convert %scales : ({sb}) -> {_t((n, k // 32), "i32")}
-    %sbi = stablehlo.reshape %sbi0 : ({_t((n, k // 32), "i32")}) -> {_t((n, k // 32, 1), "i32")}
-    %s32 = "stablehlo.gather"(%stab, %sbi) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1>}}> : (tensor<256xf32>, {_t((n, k // 32, 1), "i32")}) -> {_t((n, k // 32), "f32")}
-    %scd = stablehlo.convert %s32 : ({_t((n, k // 32), "f32")}) -> {_t((n, k // 32), el)}
-    %scb = stablehlo.broadcast_in_dim %scd, dims = [0, 1] : ({_t((n, k // 32), el)}) -> {_t((n, k // 32, 32), el)}
-    %v3 = stablehlo.reshape %v : ({_t((n, k), el)}) -> {_t((n, k // 32, 32), el)}
-    %w3 = stablehlo.multiply %v3, %scb : {_t((n, k // 32, 32), el)}
-    %wt = stablehlo.reshape %w3 : ({_t((n, k // 32, 32), el)}) -> {_t((n, k), el)}
-    %y = stablehlo.dot_general %x, %wt, contracting_dims = [1] x [1] : ({_t((t, k), el)}, {_t((n, k), el)}) -> {_t((t, n), el)}
-    return %y : {_t((t, n), el)}
+    %lo3 = stablehlo.reshape %lo : ({bl}) -> {_t(L + (n, h, 1), "ui8")}
+    %hi3 = stablehlo.reshape %hi : ({bl}) -> {_t(L + (n, h, 1), "ui8")}
+    %nb = stablehlo.concatenate %lo3, %hi3, dim = {r + 2} : ({_t(L + (n, h, 1), "ui8")}, {_t(L + (n, h, 1), "ui8")}) -> {_t(L + (n, h, 2), "ui8")}
+    %nib = stablehlo.reshape %nb : ({_t(L + (n, h, 2), "ui8")}) -> {_t(L + (n, k), "ui8")}
+    %ni = stablehlo.convert %nib : ({_t(L + (n, k), "ui8")}) -> {idx}
+    %v = func.call @_take(%vt, %ni) : (tensor<16x{el}>, {idx}) -> {_t(L + (n, k), el)}
+    %sbi0 = stablehlo.convert %scales : ({sb}) -> {_t(L + (n, k // 32), "i32")}
+    %sbi = stablehlo.reshape %sbi0 : ({_t(L + (n, k // 32), "i32")}) -> {_t(L + (n, k // 32, 1), "i32")}
+    %s32 = "stablehlo.gather"(%stab, %sbi) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = {r + 2}>, slice_sizes = array<i64: 1>}}> : (tensor<256xf32>, {_t(L + (n, k // 32, 1), "i32")}) -> {_t(L + (n, k // 32), "f32")}
+    %scd = stablehlo.convert %s32 : ({_t(L + (n, k // 32), "f32")}) -> {_t(L + (n, k // 32), el)}
+    %scb = stablehlo.broadcast_in_dim %scd, dims = [{dims}] : ({_t(L + (n, k // 32), el)}) -> {_t(L + (n, k // 32, 32), el)}
+    %v3 = stablehlo.reshape %v : ({_t(L + (n, k), el)}) -> {_t(L + (n, k // 32, 32), el)}
+    %w3 = stablehlo.multiply %v3, %scb : {_t(L + (n, k // 32, 32), el)}
+    %wt = stablehlo.reshape %w3 : ({_t(L + (n, k // 32, 32), el)}) -> {_t(L + (n, k), el)}
+    %y = stablehlo.dot_general %x, %wt, {dot} : ({_t(xs, el)}, {_t(L + (n, k), el)}) -> {_t(ys, el)}
+    return %y : {_t(ys, el)}
   }}
-  func.func private @_take(%table: tensor<16x{el}>, %i: {idx}) -> {_t((n, k), el)} {{
+  func.func private @_take(%table: tensor<16x{el}>, %i: {idx}) -> {_t(L + (n, k), el)} {{
     %zs = stablehlo.constant dense<0> : tensor<i32>
     %z = stablehlo.broadcast_in_dim %zs, dims = [] : (tensor<i32>) -> {idx}
     %ns = stablehlo.constant dense<16> : tensor<i32>
     %nn = stablehlo.broadcast_in_dim %ns, dims = [] : (tensor<i32>) -> {idx}
-    %neg = stablehlo.compare LT, %i, %z, SIGNED : ({idx}, {idx}) -> {_t((n, k), "i1")}
+    %neg = stablehlo.compare LT, %i, %z, SIGNED : ({idx}, {idx}) -> {_t(L + (n, k), "i1")}
     %wrap = stablehlo.add %i, %nn : {idx}
-    %sel = stablehlo.select %neg, %wrap, %i : {_t((n, k), "i1")}, {idx}
+    %sel = stablehlo.select %neg, %wrap, %i : {_t(L + (n, k), "i1")}, {idx}
     %i3 = stablehlo.reshape %sel : ({idx}) -> {idx3}
-    %r = "stablehlo.gather"(%table, %i3) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 2>, slice_sizes = array<i64: 1>}}> : (tensor<16x{el}>, {idx3}) -> {_t((n, k), el)}
-    return %r : {_t((n, k), el)}
+    %r = "stablehlo.gather"(%table, %i3) <{{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = {r + 2}>, slice_sizes = array<i64: 1>}}> : (tensor<16x{el}>, {idx3}) -> {_t(L + (n, k), el)}
+    return %r : {_t(L + (n, k), el)}
   }}
 }}
 """

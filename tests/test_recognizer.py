@@ -784,6 +784,52 @@ def test_blocked_mxfp4_pack_is_bit_identical_through_a_take_callee(monkeypatch):
     np.testing.assert_allclose(lit, T.bf16_round(x @ w.T), rtol=2e-2, atol=1e-2 * np.abs(x @ w.T).max())
 
 
+def test_blocked_pack_bounds_the_transient(monkeypatch):
+    """The point of blocking: the pack costs a block, not a weight.  The MXFP4
+    chain is several times wider than the weight it reconstructs (index
+    tensors, gathered values, broadcast scales), so the peak of live host
+    memory during a whole evaluation is many times the packed result; by
+    blocks it must be well under half of that (reference
+    tests/test_qmm_mxfp4.py:745-777)."""
+    import tracemalloc
+    e, n, k, t = 4, 512, 512, 2
+    codes, blocks, sb, _ = T.random_mxfp4((e, n, k), seed=12)
+    x = np.zeros((e, t, k), np.float32)
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")]
+    text = T.dense_mxfp4_rows(n, k, t, e=e)                 # every op keeps the expert axis leading: one expert a block
+
+    def peak(block_elems):
+        tracemalloc.start()
+        try:
+            built, st, _ = _packs_built(monkeypatch, text, args, block_elems)
+            return built, st, tracemalloc.get_traced_memory()[1]
+        finally:
+            tracemalloc.stop()
+    whole, st_w, peak_whole = peak(1 << 40)
+    small, st_b, peak_blocked = peak(1 << 14)
+    assert st_w["blocked"] == 0 and st_b["blocked"] == 1
+    _same_packs(whole, small)
+    assert peak_blocked < peak_whole / 2, (peak_blocked, peak_whole)
+
+
+def test_blocked_pack_reads_a_decode_table_whole(monkeypatch):
+    """Sixteen experts and a sixteen-entry E2M1 table: whether a value is cut
+    into blocks is decided by the demand coming down from the weight, not by
+    its shape -- the gather's indices are blocked, the table it gathers
+    through is read whole (reference tests/test_qmm_mxfp4.py:782-806)."""
+    e, n, k, t = 16, 64, 128, 2
+    codes, blocks, sb, w = T.random_mxfp4((e, n, k), seed=13)
+    args = [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(np.zeros((e, t, k), np.float32), "bf16")]
+    text = T.dense_mxfp4_rows(n, k, t, e=e)
+    whole, st_w, _ = _packs_built(monkeypatch, text, args, 1 << 40)
+    small, st_b, state = _packs_built(monkeypatch, text, args, 1 << 10)
+    assert st_b["blocked"] == 1 and st_b["fallbacks"] == 0
+    _same_packs(whole, small)
+    pk = state.matches[0].packs[0]
+    np.testing.assert_array_equal(np.asarray(pk.w), O.pack_codes(codes, 4))
+    np.testing.assert_array_equal(dequant_pack(pk), w)
+
+
 def test_a_chain_that_is_not_row_local_packs_whole(monkeypatch):
     """A reshape that folds N into other axes (the decode over a flat index
     list) is not row-local: blocks are refused and the pack is the whole
