@@ -354,6 +354,30 @@ def test_uneven_group_sizes_fall_back():
     _one_fallback(ex, host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32)))
 
 
+def test_mxfp4_scales_over_blocks_of_sixteen_are_turned_down_at_analysis():
+    """The block-scaled form has exactly one legal block: a scale that
+    broadcasts one value per 16 elements is no MXFP4 weight, and no affine one
+    either (its values are not integer codes); nothing is ever evaluated
+    (reference tests/test_qmm_mxfp4.py:643-668)."""
+    n, k, t = 48, 128, 2                                      # (N * K / 32 must not be the 256 of the scale table)
+    text = T.dense_mxfp4(n, k, t)
+    # the same chain with sixteen-wide blocks: [N, K/16] scale bytes, [N, K/16, 16] products
+    narrow = (text.replace(f"tensor<{n}x{k // 32}x32x", f"tensor<{n}x{k // 16}x16x")
+                  .replace(f"tensor<{n}x{k // 32}x", f"tensor<{n}x{k // 16}x")
+                  .replace(f"tensor<{n * k // 32}x", f"tensor<{n * k // 16}x"))
+    assert narrow != text
+    ex = engine.compile_program(narrow)
+    st = qmm.analyze(ex.interp)
+    assert st.matches == [] and qmm.stats()["recognized"] == 0
+    # ... and the program still runs literally
+    codes, blocks, sb, w = T.random_mxfp4((n, k), seed=8)
+    sb16 = np.repeat(sb, 2, axis=1)
+    x = T.bf16_round(np.random.default_rng(8).standard_normal((t, k)).astype(np.float32) * 0.4)
+    (y,) = ex.interp.run([I.from_numpy(blocks), I.from_numpy(sb16), I.from_numpy(x, "bf16")])
+    exact = x @ w.T
+    np.testing.assert_allclose(I.host(y).a, exact, rtol=2e-2, atol=2e-2 * np.abs(exact).max())
+
+
 def test_off_grid_e2m1_value_falls_back():
     n, k, t = 16, 64, 2
     vt = list(T.E2M1) + [-v for v in T.E2M1]
@@ -576,6 +600,27 @@ def test_decode_loop_weights_are_hoisted_out_of_the_carry():
     qmm.prologue(ex.interp, args)
     qmm.prologue(ex.interp, args)
     assert qmm.stats()["packs"] == 1 and qmm.stats()["fallbacks"] == 0
+
+
+def test_interleaved_groups_in_a_decode_loop(monkeypatch):
+    """The permutation of K travels into the loop with the other packed values:
+    packed once, applied to the activations in every step, and the loop's
+    result follows the literal chain (reference tests/test_qmm.py:429-469)."""
+    k, m, steps, ng = 128, 2, 3, 2
+    g_idx = (np.arange(k) % ng).astype(np.float32)
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, k, k // ng, seed=21, g_idx=g_idx)
+    x = T.bf16_round(np.random.default_rng(2).standard_normal((m, k)).astype(np.float32))
+    args = host_args_dense(packed, scale * 0.2, zero, g_idx, x)
+    args[1] = I.from_numpy(T.bf16_round(scale * 0.2), "bf16")
+    st, fused, literal = _fused_and_literal(monkeypatch, T.decode_loop(k, ng, m, steps), args)
+    assert qmm.stats()["packs"] == 1 and qmm.stats()["perms"] == 1 and qmm.stats()["fallbacks"] == 0
+    assert st.matches[0].has_perm and st.matches[0].nvals == 4
+    w = T.bf16_round(scale * 0.2)[g_idx.astype(np.int32)] * (q.astype(np.float32) - zero[g_idx.astype(np.int32)])
+    exact = x
+    for _ in range(steps):
+        exact = T.bf16_round(exact @ w)
+    np.testing.assert_allclose(fused, literal, rtol=3e-2, atol=3e-2 * np.abs(exact).max())
+    np.testing.assert_allclose(fused, exact, rtol=3e-2, atol=3e-2 * np.abs(exact).max())
 
 
 def test_rewritten_program_runs_the_root_and_never_the_absorbed_ops(monkeypatch):
