@@ -17,24 +17,28 @@
 // Two variants (template flag XD):
 //
 // * ring variant (XD = 0; more than eight rows of activations on a weight of
-//   at most 64 rows per compute unit): activations and weight tiles both
-//   travel through the ring, as described below;
-// * direct variant (M <= 8, or any M where the weight is wide enough for the
-//   ring variant to need a second round of workgroups): each compute wavefront
-//   fetches its own K-slice of the activations straight into MFMA operand
-//   registers when a pass begins, every ring slot holds a weight tile, and the
-//   loaders' tile loop is a real loop.  XD = 1, K exactly one pass: the compute
-//   wavefronts' tile loop is a real loop too, any number of tiles, a tile's
-//   sums leave for LDS at once; XD = 2, several passes: the tiles' sums stay in
-//   registers from pass to pass (at most eight tiles, unrolled).  The host
-//   deals up to 128 rows a workgroup, so that a 28672-row weight is still one
-//   workgroup per compute unit.  The loaders keep two tiles requested: tile
-//   g+1 before tile g is published, tile g+2 right after -- issuing a tile
-//   takes about as long as receiving one, and a wavefront stuck in issue
-//   cannot publish.  Measured on 4096 x 14336 four-bit weights: 10.3 us at
-//   M = 1 against 11.9 us for the ring variant; at M = 16 the 128 KB of
-//   activations in front of the first tile cost more than the ring's
-//   interleaving (13.3 against 12.8 us).
+//   at most 64 rows per compute unit, where the direct variant has no room
+//   for its staging patches or K takes several passes): activations and
+//   weight tiles both travel through the ring, as described below;
+// * direct variant (every one-pass shape, and several passes with few rows or
+//   wide weights): each compute wavefront fetches its own K-slice of the
+//   activations when a pass begins -- straight into MFMA operand registers up
+//   to four rows, with whole-line loads through a wave-private LDS patch from
+//   five rows on -- every ring slot holds a weight tile, and the loaders' tile
+//   loop is a real loop.  XD = 1, K exactly one pass: the compute wavefronts'
+//   tile loop is a real loop too, any number of tiles, a tile's sums leave for
+//   LDS at once; XD = 2, several passes: the tiles' sums stay in registers
+//   from pass to pass (at most eight tiles, unrolled).  The host deals up to
+//   128 rows a workgroup, so that a 28672-row weight is still one workgroup
+//   per compute unit.  The loaders keep two tiles requested: tile g+1 before
+//   tile g is published, tile g+2 right after.  A wavefront holds about
+//   sixteen loads in flight, so two tiles are all four loaders can have out,
+//   and a wavefront blocked in issue cannot publish; more in flight (every
+//   tile up front with flags in LDS, eight loaders with three tiles out) was
+//   built and measured slower every time: what ends the launch early is the
+//   next needed tile landing early, and more requests share the bandwidth
+//   among later tiles.  Measured on 4096 x 14336 four-bit weights: 9.6 us a
+//   launch at one row, 10.4-10.7 us at sixteen (ring variant: 11.2 / 12.0 us).
 //
 // The direct variants also serve MXFP4 weights (template value GSHIFT = 2): the
 // hardware converter widens two E2M1 codes at a time with the 32-block's
