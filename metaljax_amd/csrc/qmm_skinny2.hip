@@ -491,9 +491,19 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const uint32_t one = pin_vgpr(kOnesBf16x2);
     const bf16x8 ones = as_bf16x8(one, one, one, one);
     const uint32_t nib = pin_vgpr(0x000F000Fu), magic = pin_vgpr(0x43004300u);
-    const uint32_t rowb = (uint32_t)(wave * 4096 + r * 256);    // this lane's row inside its slice's 4 KB
+    // The K-slice this wavefront works on.  In the one-pass variant the
+    // assignment rotates with the workgroup (and so does the order in which a
+    // wavefront asks for its slice's chunks, below): every workgroup reads all
+    // of the activations, and 256 of them walking through the same lines in
+    // the same order at the same time wait on one another's misses -- 128 KB
+    // that are not in L2 take a compute unit 2.6 us in lockstep, 1.85 us
+    // rotated (measured with a fetch-only kernel).  The slices' sums are added
+    // in slice order whoever computed them, so the results do not change.
+    static_assert((CW & (CW - 1)) == 0, "slice rotation");
+    const int sw = XD == 1 ? (wave + (int)(blockIdx.x >> 3)) & (CW - 1) : wave;
+    const uint32_t rowb = (uint32_t)(sw * 4096 + r * 256);      // this lane's row inside its slice's 4 KB
     // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
-    const int tab_row = (wave >> 2) * (WIDE ? 2048 : 1024) + (wave & 3) * 256 + r * 16;   // this lane's table row inside a kind
+    const int tab_row = (sw >> 2) * (WIDE ? 2048 : 1024) + (sw & 3) * 256 + r * 16;   // this lane's table row inside a kind
     const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
     const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? xrows * a.K * 2 : 0);
     auto xrow = [&](int m) -> int64_t {
@@ -682,7 +692,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // (r, kg) takes pieces 2*kg and 2*kg + 1 of every chunk of row r.
       auto fetch_x = [&](int p, bool active, uint32_t lane_off) __attribute__((always_inline)) {
         u32x4 raw[CPS][2];
-        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
+        const uint32_t so = active ? (uint32_t)((p * CW + sw) * KS) * 2u : 0u;
 #pragma unroll
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
@@ -710,7 +720,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // position p ^ ((r >> 1) & 3): both the 16-lane write and read passes
       // touch every bank once; the lanes whose operand row is in the other
       // half read along and keep what they had).
-      auto fetch_x_staged = [&](int p, bool active) __attribute__((always_inline)) {
+      auto fetch_x_staged = [&](auto rotc, int p, bool active) __attribute__((always_inline)) {
+        constexpr int ROT = decltype(rotc)::value % CPS;          // chunk asked for first
         unsigned char* stg = patches + wave * 1024;
         const int srow = lane >> 3, sp = lane & 7;
         u32x4 raw[CPS][2];
@@ -720,12 +731,12 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           const int64_t xr = active ? xrow(8 * h + srow) : -1;
           lo[h] = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)sp * 16u : kOutOfRange;
         }
-        const uint32_t so = active ? (uint32_t)((p * CW + wave) * KS) * 2u : 0u;
+        const uint32_t so = active ? (uint32_t)((p * CW + sw) * KS) * 2u : 0u;
 #pragma unroll
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
           for (int h = 0; h < 2; ++h)
-            raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo[h], so + (uint32_t)(c * 128), 0);
+            raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo[h], so + (uint32_t)(((c + ROT) % CPS) * 128), 0);
         const uint32_t wr = (uint32_t)(srow * 128 + ((sp ^ ((srow >> 1) & 3)) << 4));
         const uint32_t rkey = (uint32_t)((r >> 1) & 3);
         const bool upper = r >= 8;
@@ -744,7 +755,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
               bf16x8 o;
               if constexpr (BITS == 4 && !MX) o = pair_stride4(v);
               else o = __builtin_bit_cast(bf16x8, v);
-              if (upper == (h == 1)) xa[c][j] = o;
+              if (upper == (h == 1)) xa[(c + ROT) % CPS][j] = o;
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -778,7 +789,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         auto key = [](int row) { return R == 8 ? (row >> 1) & 3 : row; };
         const int64_t xr = active ? xrow(srow) : -1;
         const uint32_t lo = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)sp * 16u : kOutOfRange;
-        const uint32_t so = active ? (uint32_t)(wave * KS) * 2u : 0u;
+        const uint32_t so = active ? (uint32_t)(sw * KS) * 2u : 0u;
         u32x4 raw[NI];
 #pragma unroll
         for (int i = 0; i < NI; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo, so + (uint32_t)(i * W), 0);
@@ -813,10 +824,17 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       if constexpr (XD == 1) {
         // One pass (the host sees to it).  The tiles as a real loop (any number of them): a tile's sums leave
         // for its slot at once, where the loaders add up the slices.
-        const bool active = wave < slices;        // uniform
+        const bool active = sw < slices;          // uniform
         QMM_STAMP(0);
         if constexpr (!WIDE) {                    // (wide table rows leave no LDS for the staging patches)
-          if (M > 8) fetch_x_staged(0, active);
+          if (M > 8) {
+            switch ((blockIdx.x >> 6) & 3) {
+              case 0: fetch_x_staged(std::integral_constant<int, 0>{}, 0, active); break;
+              case 1: fetch_x_staged(std::integral_constant<int, 2>{}, 0, active); break;
+              case 2: fetch_x_staged(std::integral_constant<int, 4>{}, 0, active); break;
+              default: fetch_x_staged(std::integral_constant<int, 6>{}, 0, active); break;
+            }
+          }
           else if (M > 4) fetch_x_lines(std::integral_constant<int, 8>{}, active);
           else fetch_x(0, active, xlane);
         } else {
@@ -830,7 +848,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           const int slot = g & 3;
           f32x4 at = zero;
           if (active) at = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + tab_row, zero);
-          float* part = reinterpret_cast<float*>(ring + slot * kItem + wave * 4096);
+          float* part = reinterpret_cast<float*>(ring + slot * kItem + sw * 4096);
 #pragma unroll
           for (int e = 0; e < 4; ++e) part[e * kWave + lane] = at[e];
           if (g < 4) QMM_STAMP(4 + 2 * g);
