@@ -202,8 +202,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* ring = smem;
   unsigned char* tabs = smem + S::B * kItem;
-  // One-pass direct variant: behind the ring and the tables, a 1 KB patch a
-  // compute wavefront (staging of more than eight rows of activations).
+  // Direct variants: behind the ring and the tables, a 1 KB patch a compute
+  // wavefront (staging of activations that come in with whole-line loads).
   unsigned char* patches = smem + 4 * (kItem + kTab);
 
   const int lane = threadIdx.x & 63;
@@ -720,7 +720,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // position p ^ ((r >> 1) & 3): both the 16-lane write and read passes
       // touch every bank once; the lanes whose operand row is in the other
       // half read along and keep what they had).
-      auto fetch_x_staged = [&](auto rotc, int p, bool active) __attribute__((always_inline)) {
+      // (pk != 0, the row packing of the several-pass variant: operand row
+      // q*pk + m is row m of x over the K-slice of pass q.)
+      auto fetch_x_staged = [&](auto rotc, int p, bool active, int pk) __attribute__((always_inline)) {
         constexpr int ROT = decltype(rotc)::value % CPS;          // chunk asked for first
         unsigned char* stg = patches + wave * 1024;
         const int srow = lane >> 3, sp = lane & 7;
@@ -728,8 +730,17 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         uint32_t lo[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const int64_t xr = active ? xrow(8 * h + srow) : -1;
-          lo[h] = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)sp * 16u : kOutOfRange;
+          const int rr = 8 * h + srow;
+          int64_t xr;
+          uint32_t pass_off = 0u;
+          if (pk == 0) {
+            xr = active ? xrow(rr) : -1;
+          } else {
+            const int q = pk == 8 ? rr >> 3 : rr >> 2, m = rr - q * pk;
+            xr = active && q * CW + wave < slices ? xrow(m) : -1;
+            pass_off = (uint32_t)(q * CW * KS) * 2u;
+          }
+          lo[h] = xr >= 0 ? (uint32_t)(xr * a.K * 2) + pass_off + (uint32_t)sp * 16u : kOutOfRange;
         }
         const uint32_t so = active ? (uint32_t)((p * CW + sw) * KS) * 2u : 0u;
 #pragma unroll
@@ -829,10 +840,10 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         if constexpr (!WIDE) {                    // (wide table rows leave no LDS for the staging patches)
           if (M > 8) {
             switch ((blockIdx.x >> 6) & 3) {
-              case 0: fetch_x_staged(std::integral_constant<int, 0>{}, 0, active); break;
-              case 1: fetch_x_staged(std::integral_constant<int, 2>{}, 0, active); break;
-              case 2: fetch_x_staged(std::integral_constant<int, 4>{}, 0, active); break;
-              default: fetch_x_staged(std::integral_constant<int, 6>{}, 0, active); break;
+              case 0: fetch_x_staged(std::integral_constant<int, 0>{}, 0, active, 0); break;
+              case 1: fetch_x_staged(std::integral_constant<int, 2>{}, 0, active, 0); break;
+              case 2: fetch_x_staged(std::integral_constant<int, 4>{}, 0, active, 0); break;
+              default: fetch_x_staged(std::integral_constant<int, 6>{}, 0, active, 0); break;
             }
           }
           else if (M > 4) fetch_x_lines(std::integral_constant<int, 8>{}, active);
@@ -857,6 +868,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // Several passes: the tiles' sums stay in registers from pass to pass
         // (at most TMAX tiles, unrolled); the next pass's activations are
         // fetched when the pass begins.
+        QMM_STAMP(0);
         if (PK != 0) {
           // every pass's activations at once: lane row r = q*PK + m reads row m
           // over the K-slice of pass q (lanes past M, past the passes or past
@@ -865,9 +877,20 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
           const int64_t xr = q * CW + wave < slices ? xrow(m) : -1;
           const uint32_t off = xr >= 0 ? (uint32_t)(xr * a.K * 2) + (uint32_t)kg * 32u + (uint32_t)(q * CW * KS) * 2u
                                        : kOutOfRange;
-          fetch_x(0, wave < slices, off);
+          // more than eight live operand rows: whole-line loads through the
+          // patch, as in the one-pass variant (the direct fetch asks for a
+          // quarter line a lane: sixteen live rows are sixteen line requests
+          // an instruction).  Same box, direct against staged: 8192 x 8192
+          // at eight rows 13.3 / 11.7 us, 4096 x 14336 at four rows 11.4 /
+          // 11.0; with eight live rows it goes either way (8192 x 8192 at
+          // four rows 11.35 / 10.9, 4096 x 14336 at two rows 9.7 / 10.2).
+          bool staged = false;
+          if constexpr (!WIDE) staged = M * passes > 8;
+          if (staged) fetch_x_staged(std::integral_constant<int, 0>{}, 0, wave < slices, PK);
+          else fetch_x(0, wave < slices, off);
         }
         const int my_pass = PK == 8 ? kg >> 1 : kg;   // the pass whose sums this lane's accumulator rows hold
+        QMM_STAMP(2);
         for (int p = 0; p < passes; ++p) {
           const bool active = p * CW + wave < slices;   // uniform
           if (PK == 0) fetch_x(p, active, xlane);
@@ -875,6 +898,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
             constexpr int t = decltype(tc)::value;
             if (t < ntiles) {
               item_barrier();
+              if (p * ntiles + t < 4) QMM_STAMP(3 + 2 * (p * ntiles + t));
               const int slot = (p * ntiles + t) & 3;
               if (active) {
                 const f32x4 d = tile_math(ring + slot * kItem + rowb, tabs + slot * kTab + tab_row, zero);
@@ -887,6 +911,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
                 for (int e = 0; e < 4; ++e) part[e * kWave + lane] = acc[t][e];
               }
+              if (p * ntiles + t < 4) QMM_STAMP(4 + 2 * (p * ntiles + t));
             }
           });
         }
@@ -953,9 +978,9 @@ void launch_one(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t s
   dim3 grid((unsigned)ceil_div(a.N, rows_per_wg), (unsigned)batch, (unsigned)chunks);
   constexpr int kTabKind = (CW >= 4 ? CW * 256 : 1024) * (GSHIFT == 5 ? 2 : 1);
   constexpr int XR = XD ? 0 : 2048 / BITS / 128;
-  // (one-pass direct variant: plus a 1 KB patch a compute wavefront for staging activations)
+  // (direct variants: plus a 1 KB patch a compute wavefront for staging activations)
   const size_t lds = (size_t)(XD || XR + TMAX >= 4 ? 4 : XR + TMAX) * (CW * 4096 + 2 * kTabKind) +
-                     (XD == 1 && GSHIFT != 5 ? (size_t)CW * 1024 : 0);
+                     (XD != 0 && GSHIFT != 5 ? (size_t)CW * 1024 : 0);
   constexpr auto kern = skinny2_kernel<BITS, CW, NL, TMAX, GSHIFT, XD>;
   if (!lds_limit<kern>(lds)) return;
   hipLaunchKernelGGL(kern, grid, dim3(kWave * (CW + NL)), lds, st, a, rows_per_wg);

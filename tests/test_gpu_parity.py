@@ -230,6 +230,8 @@ def test_gemv_mxfp4(m):
     (3, 4100, 12288),     # three passes packed by four rows
     (12, 2048, 8192),     # two passes, activations fetched per pass
     (2, 640, 16384),      # four passes packed by four, fewer workgroups than compute units
+    (7, 4096, 8192),      # two passes packed by eight, fourteen live operand rows: whole-line loads through the patches
+    (4, 2048, 16384),     # four passes packed by four, sixteen live operand rows
 ])
 def test_decode_mxfp4_big_weights_on_the_loader_wavefront_kernel(m, n, k):
     """MXFP4 decode with K a multiple of 512 and at least eight 256-byte slices:
@@ -322,6 +324,7 @@ def test_decode_big_weights_on_the_loader_wavefront_kernel(bits, gs, m, n, k):
     (4, 64, 6, 14336, 4096),     # six rows: whole-line activation loads through the patches
     (8, 128, 8, 7000, 2048),     # the same with eight-bit codes (half as many bytes a slice)
     (4, 64, 3, 3000, 8192),      # two passes, rows packed
+    (4, 64, 7, 3000, 8192),      # two passes, rows packed, more than eight live operand rows (staged through the patches)
     (4, 128, 12, 2048, 12288),   # three passes, one tile a workgroup, activations fetched per pass
 ])
 def test_decode_big_weights_float16_tables(bits, gs, m, n, k):
@@ -349,6 +352,8 @@ def test_decode_big_weights_float16_tables(bits, gs, m, n, k):
     (4, 64, 2, 28001, 4096),     # seven tiles a workgroup, the last ragged
     (4, 128, 7, 9000, 4096),     # seven rows, group 128: whole-line activation loads through the patches
     (4, 64, 6, 9000, 4096),      # six rows, groups of 64: wide table rows leave no patches, direct fetch
+    (4, 128, 4, 4096, 14336),    # 3.5 passes packed by four, group 128: sixteen live operand rows through the patches
+    (4, 64, 8, 3000, 8192),      # two passes packed by eight, groups of 64: no patches, direct fetch
 ])
 def test_decode_big_weights_float32_tables(bits, gs, m, n, k):
     """float32 scales and biases (biases that do not fit 16 bits): an entry is
