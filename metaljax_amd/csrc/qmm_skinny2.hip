@@ -785,9 +785,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // instruction's 1 KB goes through the patch (piece p of row r at position
       // p ^ key(r): conflict-free both ways) and comes back in operand order.
       // 4096 x 14336, four-bit, same box: eight rows 9.8 against 10.7 us a
-      // launch; up to four rows the direct fetch stays ahead (R = 4: 10.2
-      // against 10.0 us, R = 1: 10.0-10.5 against 9.8 us: few lanes are live
-      // and the round trip through LDS is the longer way).
+      // launch, four rows (R = 4) 10.1 against 10.35 and 5.5 against 5.8 on
+      // 4096 x 4096; with one or two rows it is a wash (R = 1: 9.93 against
+      // 9.93, 5.72 against 5.56) and the direct fetch stays.
       auto fetch_x_lines = [&](auto rc, bool active) __attribute__((always_inline)) {
         constexpr int SB = CPS * 128;                             // bytes of a row's slice
         constexpr int R = decltype(rc)::value * SB < 1024 ? 1024 / SB : decltype(rc)::value;
@@ -847,6 +847,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
             }
           }
           else if (M > 4) fetch_x_lines(std::integral_constant<int, 8>{}, active);
+          else if (M > 2) fetch_x_lines(std::integral_constant<int, 4>{}, active);
           else fetch_x(0, active, xlane);
         } else {
           fetch_x(0, active, xlane);
