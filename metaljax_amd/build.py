@@ -68,5 +68,45 @@ def build_probe(verbose: bool = False) -> str:
     return PROBE_LIB
 
 
+PJRT_LIB = os.path.join(LIBDIR, "libqmm_pjrt.so")
+PJRT_HARNESS = os.path.join(LIBDIR, "libqmm_pjrt_harness.so")
+
+
+def pjrt_header_dir():
+    """The directory holding OpenXLA's `pjrt_c_api.h`: $PJRT_C_API_INCLUDE, or
+    the reference checkout's vendored copy; None when there is none."""
+    for d in (os.environ.get("PJRT_C_API_INCLUDE"), "/root/reference/plugin/vendor"):
+        if d and os.path.exists(os.path.join(d, "pjrt_c_api.h")):
+            return d
+    return None
+
+
+def build_pjrt(verbose: bool = False):
+    """The PJRT plugin (`GetPjrtApi` over `metaljax_amd.engine`) and the C++
+    harness the tests drive it with.  Host code only.  Both are compiled against
+    the header where it lies (it is not part of this tree); without the header
+    the step is skipped and what is already built stays."""
+    inc = pjrt_header_dir()
+    if inc is None:
+        if verbose:
+            print("pjrt_c_api.h not found (PJRT_C_API_INCLUDE): PJRT plugin not rebuilt")
+        return None
+    import sysconfig
+    os.makedirs(LIBDIR, exist_ok=True)
+    base = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wno-unused-function", "-I", inc]
+    # the Python symbols resolve against the process that loads the plugin
+    # (a Python interpreter), so it is not linked against libpython
+    jobs = [(base + ["-I", sysconfig.get_paths()["include"], os.path.join(CSRC, "pjrt_plugin.cc"), "-o", PJRT_LIB], PJRT_LIB),
+            (base + [os.path.join(os.path.dirname(HERE), "tests", "pjrt_harness.cc"), "-ldl", "-o", PJRT_HARNESS], PJRT_HARNESS)]
+    for cmd, out in jobs:
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode:
+            raise RuntimeError(f"g++ failed on {out}:\n{r.stderr}")
+        if verbose:
+            print(f"built {out}")
+    return PJRT_LIB
+
+
 if __name__ == "__main__":
     build(verbose=True)
+    build_pjrt(verbose=True)

@@ -3,8 +3,9 @@ execute it on buffers (reference src/metaljax/engine.py:325, :385).
 
 Only what the quantized-matmul path needs is here: `compile_program` parses
 the module text, `execute` runs the packing prologue and then the program.
-The PJRT plugin, buffer donation/aliasing and the trace cache of the reference
-engine are outside this package.  What the plugin calls by name keeps its name,
+Buffer donation/aliasing and the trace cache of the reference engine are
+outside this package.  What a PJRT plugin calls by name (csrc/pjrt_plugin.cc
+is one) keeps its name,
 argument meaning and result type (reference plugin/metal_pjrt.cc):
 
     compile_program(code, fmt, options) -> object with name, fingerprint,
@@ -81,10 +82,12 @@ def buffer_from_host(data, type_enum: int, dims, byte_strides=None, offset: int 
     if data is None:
         arr = np.zeros(dims, dt)
     elif byte_strides is None:
-        arr = np.frombuffer(data, dt).reshape(dims)
+        arr = np.frombuffer(data, dt).reshape(dims).copy()
     else:
         arr = np.ndarray(shape=dims, dtype=dt, buffer=data, offset=offset, strides=list(byte_strides))
-        arr = np.ascontiguousarray(arr).reshape(dims)
+        arr = np.array(arr, order="C", copy=True).reshape(dims)
+    # (the bytes are copied either way: the caller's memory is free again when
+    # this returns, which is what the plugin tells PJRT, pjrt_plugin.cc)
     if el == "bf16":
         arr = (arr.astype(np.uint32) << 16).view(np.float32)      # held as float32 values
     return Buffer(from_numpy(arr, el), type_enum, dims)
