@@ -466,6 +466,225 @@ int pjrt_harness_topology() {
   return taken(g_api->PJRT_Client_TopologyDescription(&t));
 }
 
+namespace {
+int g_called = 0;
+int g_called_code = -1;
+void on_ready(PJRT_Error* e, void* arg) {
+  ++g_called;
+  g_called_code = e ? taken(e) : 0;
+  *static_cast<int*>(arg) += 1;
+}
+}  // namespace
+
+// A scripted walk over the smaller entry points (events a caller creates and
+// sets, buffer copies / layout / reference counts, memories and their user
+// data, device assignment, look-ups).  0, or the number of the first step whose
+// answer was not the expected one (the message says what the plugin answered).
+#define STEP(n, cond)                 \
+  do {                                \
+    if (!(cond)) return (n);          \
+  } while (0)
+#define ARGS(T, v)                    \
+  T v;                                \
+  memset(&v, 0, sizeof(v));           \
+  v.struct_size = T##_STRUCT_SIZE
+
+int pjrt_harness_walk(int buffer, int exe) {
+  NEED_OPEN();
+  if (buffer < 0 || buffer >= (int)g_bufs.size() || !g_bufs[buffer]) return harness_failure("no such buffer");
+  if (exe < 0 || exe >= (int)g_exes.size() || !g_exes[exe]) return harness_failure("no such executable");
+  PJRT_Buffer* b = g_bufs[buffer];
+  PJRT_LoadedExecutable* le = g_exes[exe];
+  g_error.clear();
+  // -- an event the caller creates: not ready, callback deferred, then set
+  ARGS(PJRT_Event_Create_Args, ec);
+  STEP(1, taken(g_api->PJRT_Event_Create(&ec)) == 0 && ec.event);
+  ARGS(PJRT_Event_IsReady_Args, ir);
+  ir.event = ec.event;
+  STEP(2, taken(g_api->PJRT_Event_IsReady(&ir)) == 0 && !ir.is_ready);
+  int hits = 0;
+  g_called = 0;
+  ARGS(PJRT_Event_OnReady_Args, orr);
+  orr.event = ec.event;
+  orr.callback = on_ready;
+  orr.user_arg = &hits;
+  STEP(3, taken(g_api->PJRT_Event_OnReady(&orr)) == 0 && hits == 0);
+  ARGS(PJRT_Event_Await_Args, aw);
+  aw.event = ec.event;
+  STEP(4, taken(g_api->PJRT_Event_Await(&aw)) == (int)PJRT_Error_Code_INVALID_ARGUMENT);   // nobody has set it: no wait for ever
+  ARGS(PJRT_Event_Set_Args, es);
+  es.event = ec.event;
+  es.error_code = PJRT_Error_Code_OK;
+  STEP(5, taken(g_api->PJRT_Event_Set(&es)) == 0 && hits == 1 && g_called_code == 0);
+  STEP(6, taken(g_api->PJRT_Event_IsReady(&ir)) == 0 && ir.is_ready);
+  STEP(7, taken(g_api->PJRT_Event_Await(&aw)) == 0);
+  STEP(8, taken(g_api->PJRT_Event_OnReady(&orr)) == 0 && hits == 2);       // already ready: called at once
+  ARGS(PJRT_Event_Destroy_Args, ed);
+  ed.event = ec.event;
+  STEP(9, taken(g_api->PJRT_Event_Destroy(&ed)) == 0);
+  // -- an event set with an error hands that error to whoever asks
+  ARGS(PJRT_Event_Create_Args, ec2);
+  STEP(10, taken(g_api->PJRT_Event_Create(&ec2)) == 0);
+  ARGS(PJRT_Event_Set_Args, es2);
+  es2.event = ec2.event;
+  es2.error_code = PJRT_Error_Code_ABORTED;
+  es2.error_message = "stopped by the caller";
+  es2.error_message_size = strlen(es2.error_message);
+  STEP(11, taken(g_api->PJRT_Event_Set(&es2)) == 0);
+  ARGS(PJRT_Event_Error_Args, ee);
+  ee.event = ec2.event;
+  STEP(12, taken(g_api->PJRT_Event_Error(&ee)) == (int)PJRT_Error_Code_ABORTED && g_error == "stopped by the caller");
+  ed.event = ec2.event;
+  STEP(13, taken(g_api->PJRT_Event_Destroy(&ed)) == 0);
+  // -- a buffer's own event is ready
+  ARGS(PJRT_Buffer_ReadyEvent_Args, re);
+  re.buffer = b;
+  STEP(14, taken(g_api->PJRT_Buffer_ReadyEvent(&re)) == 0 && re.event);
+  ir.event = re.event;
+  STEP(15, taken(g_api->PJRT_Event_IsReady(&ir)) == 0 && ir.is_ready && settle(re.event) == 0);
+  // -- layout: dense, minor to major = last dimension first
+  ARGS(PJRT_Buffer_Dimensions_Args, bd);
+  bd.buffer = b;
+  STEP(16, taken(g_api->PJRT_Buffer_Dimensions(&bd)) == 0);
+  ARGS(PJRT_Buffer_GetMemoryLayout_Args, ml);
+  ml.buffer = b;
+  STEP(17, taken(g_api->PJRT_Buffer_GetMemoryLayout(&ml)) == 0 && ml.layout.type == PJRT_Buffer_MemoryLayout_Type_Tiled &&
+               ml.layout.tiled.minor_to_major_size == bd.num_dims && ml.layout.tiled.num_tiles == 0);
+  for (size_t i = 0; i < bd.num_dims; ++i) STEP(18, ml.layout.tiled.minor_to_major[i] == (int64_t)(bd.num_dims - 1 - i));
+  ARGS(PJRT_Buffer_UnpaddedDimensions_Args, ud);
+  ud.buffer = b;
+  STEP(19, taken(g_api->PJRT_Buffer_UnpaddedDimensions(&ud)) == 0 && ud.num_dims == bd.num_dims);
+  ARGS(PJRT_Buffer_DynamicDimensionIndices_Args, dd);
+  dd.buffer = b;
+  STEP(20, taken(g_api->PJRT_Buffer_DynamicDimensionIndices(&dd)) == 0 && dd.num_dynamic_dims == 0);
+  // -- a copy to the (only) device is another buffer with the same bytes
+  ARGS(PJRT_Buffer_CopyToDevice_Args, cd);
+  cd.buffer = b;
+  cd.dst_device = g_device;
+  STEP(21, taken(g_api->PJRT_Buffer_CopyToDevice(&cd)) == 0 && cd.dst_buffer && cd.dst_buffer != b);
+  {
+    ARGS(PJRT_Buffer_ToHostBuffer_Args, q1);
+    q1.src = b;
+    ARGS(PJRT_Buffer_ToHostBuffer_Args, q2);
+    q2.src = cd.dst_buffer;
+    STEP(22, taken(g_api->PJRT_Buffer_ToHostBuffer(&q1)) == 0 && taken(g_api->PJRT_Buffer_ToHostBuffer(&q2)) == 0 &&
+                 q1.dst_size == q2.dst_size);
+    std::vector<char> h1(q1.dst_size + 1), h2(q2.dst_size + 1);
+    q1.dst = h1.data();
+    q2.dst = h2.data();
+    STEP(23, taken(g_api->PJRT_Buffer_ToHostBuffer(&q1)) == 0 && settle(q1.event) == 0 &&
+                 taken(g_api->PJRT_Buffer_ToHostBuffer(&q2)) == 0 && settle(q2.event) == 0 && h1 == h2);
+    q1.dst_size = q1.dst_size ? q1.dst_size - 1 : 0;              // too small a destination is refused
+    if (q2.dst_size) STEP(24, taken(g_api->PJRT_Buffer_ToHostBuffer(&q1)) == (int)PJRT_Error_Code_INVALID_ARGUMENT);
+  }
+  ARGS(PJRT_Buffer_Destroy_Args, bdel);
+  bdel.buffer = cd.dst_buffer;
+  STEP(25, taken(g_api->PJRT_Buffer_Destroy(&bdel)) == 0);
+  // -- external reference counts go up and down, never below zero
+  ARGS(PJRT_Buffer_IncreaseExternalReferenceCount_Args, inc);
+  inc.buffer = b;
+  ARGS(PJRT_Buffer_DecreaseExternalReferenceCount_Args, dec);
+  dec.buffer = b;
+  STEP(26, taken(g_api->PJRT_Buffer_IncreaseExternalReferenceCount(&inc)) == 0 &&
+               taken(g_api->PJRT_Buffer_DecreaseExternalReferenceCount(&dec)) == 0);
+  STEP(27, taken(g_api->PJRT_Buffer_DecreaseExternalReferenceCount(&dec)) == (int)PJRT_Error_Code_INVALID_ARGUMENT);
+  ARGS(PJRT_Buffer_OpaqueDeviceMemoryDataPointer_Args, op);
+  op.buffer = b;
+  ARGS(PJRT_Buffer_UnsafePointer_Args, up);
+  up.buffer = b;
+  STEP(28, taken(g_api->PJRT_Buffer_OpaqueDeviceMemoryDataPointer(&op)) == 0 && taken(g_api->PJRT_Buffer_UnsafePointer(&up)) == 0 &&
+               (uintptr_t)op.device_memory_ptr == up.buffer_pointer && up.buffer_pointer != 0);
+  // -- the buffer's memory is the device's default memory, kind "device", with user data
+  ARGS(PJRT_Buffer_Memory_Args, bm);
+  bm.buffer = b;
+  STEP(29, taken(g_api->PJRT_Buffer_Memory(&bm)) == 0 && bm.memory && bm.memory->vtable);
+  ARGS(PJRT_Device_DefaultMemory_Args, dm);
+  dm.device = g_device;
+  STEP(30, taken(g_api->PJRT_Device_DefaultMemory(&dm)) == 0 && dm.memory == bm.memory);
+  ARGS(PJRT_Memory_Kind_Args, mk);
+  mk.memory = bm.memory;
+  STEP(31, taken(g_api->PJRT_Memory_Kind(&mk)) == 0 && std::string(mk.kind, mk.kind_size) == "device");
+  static int key = 0, payload = 42;
+  STEP(32, bm.memory->vtable->get_user_data(bm.memory, &key) == nullptr);
+  bm.memory->vtable->set_user_data(bm.memory, &key, &payload, nullptr);
+  STEP(33, bm.memory->vtable->get_user_data(bm.memory, &key) == &payload);
+  ARGS(PJRT_Memory_AddressableByDevices_Args, mad);
+  mad.memory = bm.memory;
+  STEP(34, taken(g_api->PJRT_Memory_AddressableByDevices(&mad)) == 0 && mad.num_devices == 1 && mad.devices[0] == g_device);
+  ARGS(PJRT_Buffer_Device_Args, bdev);
+  bdev.buffer = b;
+  STEP(35, taken(g_api->PJRT_Buffer_Device(&bdev)) == 0 && bdev.device == g_device);
+  // -- look-ups and the default assignment of one replica on one partition
+  ARGS(PJRT_Client_LookupDevice_Args, ld);
+  ld.client = g_client;
+  ld.id = 0;
+  STEP(36, taken(g_api->PJRT_Client_LookupDevice(&ld)) == 0 && ld.device == g_device);
+  ld.id = 1;
+  STEP(37, taken(g_api->PJRT_Client_LookupDevice(&ld)) == (int)PJRT_Error_Code_INVALID_ARGUMENT);
+  int assignment[2] = {-1, -1};
+  ARGS(PJRT_Client_DefaultDeviceAssignment_Args, da);
+  da.client = g_client;
+  da.num_replicas = 1;
+  da.num_partitions = 1;
+  da.default_assignment_size = 1;
+  da.default_assignment = assignment;
+  STEP(38, taken(g_api->PJRT_Client_DefaultDeviceAssignment(&da)) == 0 && assignment[0] == 0);
+  da.num_replicas = 2;
+  da.default_assignment_size = 2;
+  STEP(39, taken(g_api->PJRT_Client_DefaultDeviceAssignment(&da)) == (int)PJRT_Error_Code_INVALID_ARGUMENT);
+  // -- the loaded executable: its device, its fingerprint, memory kinds, delete
+  ARGS(PJRT_LoadedExecutable_AddressableDevices_Args, lad);
+  lad.executable = le;
+  STEP(40, taken(g_api->PJRT_LoadedExecutable_AddressableDevices(&lad)) == 0 && lad.num_addressable_devices == 1 &&
+               lad.addressable_devices[0] == g_device);
+  ARGS(PJRT_LoadedExecutable_GetExecutable_Args, ge);
+  ge.loaded_executable = le;
+  STEP(41, taken(g_api->PJRT_LoadedExecutable_GetExecutable(&ge)) == 0 && ge.executable);
+  ARGS(PJRT_Executable_Fingerprint_Args, f1);
+  f1.executable = ge.executable;
+  ARGS(PJRT_LoadedExecutable_Fingerprint_Args, f2);
+  f2.executable = le;
+  STEP(42, taken(g_api->PJRT_Executable_Fingerprint(&f1)) == 0 && taken(g_api->PJRT_LoadedExecutable_Fingerprint(&f2)) == 0 &&
+               std::string(f1.executable_fingerprint, f1.executable_fingerprint_size) ==
+                   std::string(f2.executable_fingerprint, f2.executable_fingerprint_size));
+  ARGS(PJRT_Executable_OutputMemoryKinds_Args, omk);
+  omk.executable = ge.executable;
+  STEP(43, taken(g_api->PJRT_Executable_OutputMemoryKinds(&omk)) == 0 && omk.num_outputs >= 1 &&
+               std::string(omk.memory_kinds[0], omk.memory_kind_sizes[0]) == "device");
+  ARGS(PJRT_Executable_GetCostAnalysis_Args, ca);
+  ca.executable = ge.executable;
+  STEP(44, taken(g_api->PJRT_Executable_GetCostAnalysis(&ca)) == 0 && ca.num_properties == 0);
+  ARGS(PJRT_Executable_Serialize_Args, ser);
+  ser.executable = ge.executable;
+  STEP(45, taken(g_api->PJRT_Executable_Serialize(&ser)) == (int)PJRT_Error_Code_UNIMPLEMENTED);
+  ARGS(PJRT_Executable_Destroy_Args, xd);
+  xd.executable = ge.executable;
+  STEP(46, taken(g_api->PJRT_Executable_Destroy(&xd)) == 0);
+  ARGS(PJRT_ExecuteContext_Create_Args, cc);
+  STEP(47, taken(g_api->PJRT_ExecuteContext_Create(&cc)) == 0 && cc.context);
+  ARGS(PJRT_ExecuteContext_Destroy_Args, cdx);
+  cdx.context = cc.context;
+  STEP(48, taken(g_api->PJRT_ExecuteContext_Destroy(&cdx)) == 0);
+  ARGS(PJRT_Device_MemoryStats_Args, ms);
+  ms.device = g_device;
+  STEP(49, taken(g_api->PJRT_Device_MemoryStats(&ms)) == 0 && !ms.bytes_limit_is_set);
+  g_error.clear();
+  return 0;
+}
+
+// Marks the executable deleted (it stays a valid handle that refuses to run).
+int pjrt_harness_executable_delete(int exe) {
+  NEED_OPEN();
+  if (exe < 0 || exe >= (int)g_exes.size() || !g_exes[exe]) return harness_failure("no such executable");
+  ARGS(PJRT_LoadedExecutable_Delete_Args, d);
+  d.executable = g_exes[exe];
+  if (int rc = taken(g_api->PJRT_LoadedExecutable_Delete(&d))) return rc;
+  ARGS(PJRT_LoadedExecutable_IsDeleted_Args, q);
+  q.executable = g_exes[exe];
+  if (int rc = taken(g_api->PJRT_LoadedExecutable_IsDeleted(&q))) return rc;
+  return q.is_deleted ? 0 : harness_failure("still reported alive");
+}
+
 // How many members of PJRT_Api (function pointers) the plugin left null.
 int pjrt_harness_null_entries() {
   if (!g_api) return harness_failure("no plugin is open");

@@ -177,6 +177,25 @@ def test_compile_execute_and_copy_back_equal_the_engine(plugin):
     assert plugin.to_host(outs2[0])[1] == want
 
 
+def test_the_smaller_entry_points_answer_as_the_c_api_says(plugin):
+    """Events a caller creates and sets (deferred and immediate callbacks, an
+    error handed on), a buffer's ready event, dense layout, copies, external
+    reference counts, the memory's kind and user data, look-ups, the default
+    device assignment, the loaded executable's device / fingerprint / memory
+    kinds, and deletion: a scripted walk in the harness that reports the first
+    step whose answer was not the C API's."""
+    text = T.float_dot(8, 16, 4, el="f32")
+    rc, exe = plugin.compile(text)
+    plugin.ok(rc)
+    rc, b = plugin.buffer(np.arange(24, dtype=np.float32).reshape(2, 3, 4), F32)
+    plugin.ok(rc)
+    step = plugin.h.pjrt_harness_walk(b, exe)
+    assert step == 0, (step, plugin.error())
+    plugin.ok(plugin.h.pjrt_harness_executable_delete(exe))
+    rc, _ = plugin.execute(exe, [b, b, b])
+    assert rc == INVALID_ARGUMENT and "deleted" in plugin.error()
+
+
 def test_bf16_bytes_round_trip(plugin):
     bits = np.array([0x3F80, 0xC000, 0x0000, 0x7F7F], np.uint16)
     rc, b = plugin.buffer(bits, BF16)
