@@ -157,12 +157,44 @@ class Executable:
         self.interp.invalidate_plans()
 
 
+class UnsupportedProgram(ValueError):
+    """A program this engine cannot read ("Unsupported" in the class name: a
+    PJRT plugin reports it as UNIMPLEMENTED, reference metal_pjrt.cc:185-226)."""
+
+
+_BYTECODE_MAGIC = b"ML\xefR"
+
+
+def _module_text(raw: bytes) -> str:
+    """Module text of what a client handed over.  A JAX client serialises the
+    module as a StableHLO portable artifact (MLIR bytecode); this package reads
+    text only, so the bytecode is printed back to text by the MLIR bindings
+    that ship with jaxlib -- present wherever such a client runs, absent where
+    this package was built (then: UnsupportedProgram)."""
+    if not raw.startswith(_BYTECODE_MAGIC):
+        return raw.decode("utf-8")
+    try:
+        from jaxlib.mlir import ir as mlir
+        from jaxlib.mlir.dialects import stablehlo
+    except Exception as e:
+        raise UnsupportedProgram("MLIR bytecode needs jaxlib's MLIR bindings to be printed as text "
+                                 f"(import failed: {e})") from None
+    with mlir.Context() as ctx:
+        stablehlo.register_dialect(ctx)
+        try:
+            module = stablehlo.deserialize_portable_artifact(ctx, raw)
+        except Exception:
+            module = mlir.Module.parse(raw, ctx)
+        return module.operation.get_asm(enable_debug_info=False)
+
+
 def compile_program(code, fmt="mlir", options=None) -> Executable:
-    """`code`: StableHLO module text (str or UTF-8 bytes)."""
+    """`code`: a StableHLO module, as text (str or UTF-8 bytes) or as the MLIR
+    bytecode a JAX client sends (see `_module_text`)."""
     if fmt not in ("mlir", "stablehlo"):
-        raise ValueError(f"Unsupported program format {fmt!r}: module text only")
-    raw = bytes(code) if isinstance(code, (bytes, bytearray)) else code.encode("utf-8")
-    return Executable(Interpreter(raw.decode("utf-8")), fingerprint=hashlib.sha256(raw).hexdigest())
+        raise UnsupportedProgram(f"Unsupported program format {fmt!r}: StableHLO modules only")
+    raw = bytes(code) if isinstance(code, (bytes, bytearray, memoryview)) else code.encode("utf-8")
+    return Executable(Interpreter(_module_text(raw)), fingerprint=hashlib.sha256(raw).hexdigest())
 
 
 def execute(ex: Executable, buffers):

@@ -63,7 +63,7 @@ class Harness:
         return list(ver), plat.value.decode(), kind.value.decode(), list(counts), list(shlo)
 
     def compile(self, text, fmt="mlir"):
-        raw = text.encode()
+        raw = text if isinstance(text, bytes) else text.encode()
         out = ctypes.c_int(-1)
         rc = self.h.pjrt_harness_compile(raw, len(raw), fmt.encode(), ctypes.byref(out))
         return rc, out.value
@@ -212,6 +212,10 @@ def test_failures_come_back_as_errors_with_the_reference_codes(plugin):
     INTERNAL (reference metal_pjrt.cc:185-226); bad calls are INVALID_ARGUMENT."""
     rc, _ = plugin.compile("this is not a module")
     assert rc == INTERNAL and "compile_program" in plugin.error() and "Traceback" in plugin.error()
+    rc, _ = plugin.compile(b"ML\xefR\x01StableHLO_v1.0.0")          # MLIR bytecode, and no jaxlib here to print it
+    assert rc == UNIMPLEMENTED and "UnsupportedProgram" in plugin.error() and "jaxlib" in plugin.error()
+    rc, _ = plugin.compile(T.float_dot(8, 16, 4, el="f32"), fmt="hlo")
+    assert rc == UNIMPLEMENTED and "program format" in plugin.error()
     rc, _ = plugin.buffer(np.zeros(2, np.complex64), engine.PJRT_TYPES.index("C64"))
     assert rc == INTERNAL and "Unsupported PJRT buffer type" in plugin.error()     # a TypeError: the class decides
     rc, _ = plugin.buffer(np.zeros(2, np.uint8), engine.PJRT_TYPES.index("F8E5M2"))
