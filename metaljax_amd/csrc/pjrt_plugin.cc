@@ -677,6 +677,15 @@ PJRT_Error* DeviceMemoryStats(PJRT_Device_MemoryStats_Args* a) {
   return nullptr;
 }
 
+void no_attributes_to_free(PJRT_Device_Attributes*) {}
+PJRT_Error* DeviceGetAttributes(PJRT_Device_GetAttributes_Args* a) {
+  a->attributes = nullptr;
+  a->num_attributes = 0;
+  a->device_attributes = nullptr;
+  a->attributes_deleter = no_attributes_to_free;
+  return nullptr;
+}
+
 // ----------------------------------------------------------------- memories --
 PJRT_Error* MemoryId(PJRT_Memory_Id_Args* a) {
   a->id = 0;
@@ -1074,7 +1083,7 @@ extern "C" __attribute__((visibility("default"))) const PJRT_Api* GetPjrtApi() {
   LACK(PJRT_Device_PoisonExecution);
   LACK(PJRT_Device_CreateAsyncTrackingEvent);
   LACK(PJRT_Device_ClearMemoryStats);
-  LACK(PJRT_Device_GetAttributes);
+  HAVE(PJRT_Device_GetAttributes, DeviceGetAttributes);
   LACK(PJRT_AsyncTrackingEvent_Destroy);
   HAVE(PJRT_Memory_Id, MemoryId);
   HAVE(PJRT_Memory_Kind, MemoryKind);
