@@ -257,6 +257,9 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="time read-only and empty launches instead (what one launch over the "
                          "headline's bytes can reach on this GPU whatever its arithmetic)")
+    ap.add_argument("--probe-mfma", action="store_true",
+                    help="time a stream of matrix instructions with and without operand loads beside it "
+                         "(what bounds the prefill kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU; --gpus {args.gpus} is not supported "
@@ -281,6 +284,10 @@ def main():
     if args.probe:
         from metaljax_amd import profiling
         print(json.dumps({"probe": profiling.stream_probe()}))
+        return 0
+    if args.probe_mfma:
+        from metaljax_amd import profiling
+        print(json.dumps({"mfma_feed": profiling.mfma_feed_probe()}))
         return 0
     if args.shape:
         print(json.dumps({args.shape: bench_once(int(args.shape[1]), check=not args.no_cpu)}))

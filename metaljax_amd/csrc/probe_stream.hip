@@ -6,6 +6,8 @@
 //                workgroup a contiguous share, `unroll` loads in flight a
 //                lane) and keeps an XOR so that nothing is elided
 //   probe_empty  a launch of the same geometry and LDS size that does nothing
+//   probe_mfma_feed  a stream of matrix instructions with and without operand
+//                loads beside it (what bounds the prefill kernels)
 //   probe_loaders  the decode kernel's way of asking: only the first `active`
 //                wavefronts of a workgroup request the workgroup's share, 1 KB
 //                an instruction, everything before the first wait, into
@@ -188,6 +190,80 @@ __global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint
   }
 }
 
+// What feeding the matrix cores costs (the prefill kernels' bound): a
+// wavefront runs `iters` groups of eight MFMAs; per group it also issues LOADS
+// 1 KB loads into registers (16 bytes a lane, from a window that stays in L2)
+// and LDSR 1 KB LDS reads.  The loaded registers are the A operands of the
+// group after next, as in a kernel that prefetches.  KIND 0: bf16 32x32x16;
+// 1: the block-scaled 32x32x64 FP6 x FP4 form.  Lane 0 of every wavefront
+// reports the constant-clock (100 MHz) and shader-clock time of the loop.
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
+template <int LOADS, int LDSR, int KIND, int DMA = 0>
+__global__ void mfma_feed_kernel(const unsigned char* __restrict__ p, uint64_t* out, int iters, uint32_t* sink) {
+  extern __shared__ unsigned char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(p) + (int64_t)(blockIdx.x & 63) * 262144, 0, 262144u, 0x00020000);
+  constexpr int NB = LOADS > 0 ? LOADS : 1;
+  u32x4 cur[NB], nxt[NB], nxt2[NB];
+  for (int j = 0; j < NB; ++j) cur[j] = nxt[j] = nxt2[j] = u32x4{0x3f803f80u + (uint32_t)lane, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  u32x4 lv = {0u, 0u, 0u, 0u};
+  f32x16_t acc[2];
+  for (int t = 0; t < 2; ++t)
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  bf16x8_t bop;
+  for (int i = 0; i < 8; ++i) bop[i] = (__bf16)1.0f;
+  const uint32_t lane_off = (uint32_t)wave * 65536u + (uint32_t)lane * 16u;
+  const uint64_t c0 = __builtin_amdgcn_s_memtime(), t0 = __builtin_amdgcn_s_memrealtime();
+  // (the loop has no side effects of its own: tie it between the two clock reads)
+  asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]) : "s"(c0), "s"(t0));
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j)
+      nxt2[j] = __builtin_amdgcn_raw_buffer_load_b128(r, lane_off + (uint32_t)(j * 1024), (uint32_t)((it & 7) * 8192), 0);
+    // (DMA: as many 1 KB loads straight into LDS instead, four groups ahead of
+    // the LDS reads that would use them)
+#pragma unroll
+    for (int j = 0; j < DMA; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + ((wave * 16 + (it & 3) * 4 + (j & 3)) * 1024) % 65536), 16,
+                                               lane_off + (uint32_t)(j * 1024), (uint32_t)((it & 7) * 8192), 0, 0);
+    if (DMA) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * DMA) & 0xF) | (((3 * DMA) >> 4) << 14));   // at most three groups' loads out
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const u32x4 a = cur[m % NB];
+      if constexpr (KIND == 0) {
+        acc[m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), bop, acc[m & 1], 0, 0, 0);
+      } else {
+        const i32x8_t a8 = {(int)a[0], (int)a[1], (int)a[2], (int)a[3], (int)a[0], (int)a[1], 0, 0};
+        const i32x8_t b8 = {(int)a[1], (int)a[2], (int)a[3], (int)a[0], 0, 0, 0, 0};
+        acc[m & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[m & 1], 2, 4, 0, 127, 0, 127);
+      }
+      if (m < LDSR / 2) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+          lv ^= *reinterpret_cast<const u32x4*>(lds + ((wave * 16 + m * 2 + q) * 1024 + lane * 16) % 65536);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      cur[j] = nxt[j];
+      nxt[j] = nxt2[j];
+    }
+  }
+  asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(cur[0][0]), "+v"(nxt[0][0]));
+  const uint64_t c1 = __builtin_amdgcn_s_memtime(), t1 = __builtin_amdgcn_s_memrealtime();
+  float v = 0.f;
+  for (int t = 0; t < 2; ++t)
+    for (int i = 0; i < 16; ++i) v += acc[t][i];
+  if (v == 12345.678f && (lv[0] ^ lv[3]) == 77u) sink[0] = 1u;
+  if (lane == 0) {
+    out[((int64_t)blockIdx.x * (blockDim.x >> 6) + wave) * 2] = t1 - t0;
+    out[((int64_t)blockIdx.x * (blockDim.x >> 6) + wave) * 2 + 1] = c1 - c0;
+  }
+}
+
 __global__ void empty_kernel(uint32_t* sink) {
   extern __shared__ unsigned char lds[];
   if (sink && threadIdx.x == 0xFFFFFF) sink[0] = lds[0];
@@ -253,6 +329,43 @@ int probe_stamped_loaders(const void* p, void* stamps, int pattern, int busy, in
                        static_cast<uint64_t*>(stamps), busy, iters);
   };
   if (pattern) launch(stamped_loaders_kernel<1>); else launch(stamped_loaders_kernel<0>);
+  return (int)hipGetLastError();
+}
+
+// 256 workgroups of `waves` wavefronts (4: one a SIMD, 8: two); `loads` in {0, 2, 4, 8} register loads and
+// `lds_reads` in {0, 8, 16} LDS reads of 1 KB per group of eight MFMAs of `kind` (0 bf16, 1 block-scaled FP6 x FP4;
+// + 100: the loads go straight into LDS, with 8 LDS reads);
+// p: at least 16 MiB; out: uint64 [256 * waves][2] = (10 ns ticks, shader clocks) of the loop.
+int probe_mfma_feed(const void* p, void* out, void* sink, int waves, int loads, int lds_reads, int kind, int iters,
+                    void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (waves != 4 && waves != 8) return -1;
+  auto launch = [&](auto kern) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    hipLaunchKernelGGL(kern, dim3(256), dim3(64 * waves), 65536, st, static_cast<const unsigned char*>(p),
+                       static_cast<uint64_t*>(out), iters, static_cast<uint32_t*>(sink));
+  };
+  const int key = (kind >= 100 ? 1000000 : 0) + (kind % 100) * 10000 + loads * 100 + lds_reads;
+  switch (key) {
+    case 0: launch(mfma_feed_kernel<0, 0, 0>); break;
+    case 200: launch(mfma_feed_kernel<2, 0, 0>); break;
+    case 400: launch(mfma_feed_kernel<4, 0, 0>); break;
+    case 800: launch(mfma_feed_kernel<8, 0, 0>); break;
+    case 8: launch(mfma_feed_kernel<0, 8, 0>); break;
+    case 16: launch(mfma_feed_kernel<0, 16, 0>); break;
+    case 816: launch(mfma_feed_kernel<8, 16, 0>); break;
+    case 10000: launch(mfma_feed_kernel<0, 0, 1>); break;
+    case 10200: launch(mfma_feed_kernel<2, 0, 1>); break;
+    case 10400: launch(mfma_feed_kernel<4, 0, 1>); break;
+    case 10800: launch(mfma_feed_kernel<8, 0, 1>); break;
+    case 10008: launch(mfma_feed_kernel<0, 8, 1>); break;
+    case 1000208: launch(mfma_feed_kernel<0, 8, 0, 2>); break;      // + 1000000: the loads go straight into LDS
+    case 1000408: launch(mfma_feed_kernel<0, 8, 0, 4>); break;
+    case 1000808: launch(mfma_feed_kernel<0, 8, 0, 8>); break;
+    case 1010208: launch(mfma_feed_kernel<0, 8, 1, 2>); break;
+    case 1010408: launch(mfma_feed_kernel<0, 8, 1, 4>); break;
+    default: return -1;
+  }
   return (int)hipGetLastError();
 }
 

@@ -122,6 +122,43 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
     return out
 
 
+def mfma_feed_probe(iters: int = 2000):
+    """What feeding the matrix cores costs: per group of eight MFMAs, the
+    median over all wavefronts of the loop time in shader clocks (and ns), for
+    a pure MFMA stream and with 1 KB register loads / LDS reads beside it, one
+    and two wavefronts a SIMD, bf16 32x32x16 and block-scaled FP6 x FP4
+    32x32x64.  Returns a dict of results."""
+    import ctypes
+    import os
+
+    import numpy as np
+    import torch
+    here = os.path.dirname(os.path.abspath(__file__))
+    lib = ctypes.CDLL(os.path.join(here, "lib", "libqmm_probe.so"))
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.probe_mfma_feed.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    data = torch.randint(-2**31, 2**31 - 1, ((16 << 20) // 4,), dtype=torch.int32, device="cuda")
+    out = torch.zeros(256 * 8 * 2, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+    res = {}
+    cases = [(0, 0, 0), (0, 2, 0), (0, 4, 0), (0, 8, 0), (0, 0, 8), (0, 0, 16), (0, 8, 16),
+             (1, 0, 0), (1, 2, 0), (1, 4, 0), (1, 8, 0), (1, 0, 8),
+             (100, 2, 8), (100, 4, 8), (100, 8, 8), (101, 2, 8), (101, 4, 8)]
+    for kind, loads, reads in cases:
+        for waves in (4, 8):
+            for _ in range(2):                      # the second run is the measured one
+                rc = lib.probe_mfma_feed(data.data_ptr(), out.data_ptr(), sink.data_ptr(), waves, loads, reads, kind,
+                                         iters, None)
+                assert rc == 0, rc
+                torch.cuda.synchronize()
+            t = out.cpu().numpy()[:256 * waves * 2].reshape(-1, 2)
+            name = (f"{'bf16 32x32x16' if kind % 100 == 0 else 'fp6 x fp4 32x32x64'}, {waves // 4} wavefront(s) a SIMD, "
+                    f"{loads} KB {'loads into LDS' if kind >= 100 else 'register loads'} + {reads} KB LDS reads a group")
+            res[name] = {"clocks_per_group": round(float(np.median(t[:, 1])) / iters, 1),
+                         "ns_per_group": round(float(np.median(t[:, 0])) * 10.0 / iters, 1)}
+    return res
+
+
 def decode_timeline(cfg: int = 2, rows=(1, 16)):
     """Clock stamps of the decode kernel's last launch over 18 rotating weight
     sets (a library built with QMM_TIMELINE=1 keeps them; `qmm_debug_stamps`
