@@ -193,8 +193,8 @@ __global__ void stamped_loaders_kernel(const unsigned char* __restrict__ p, uint
 // What feeding the matrix cores costs (the prefill kernels' bound): a
 // wavefront runs `iters` groups of eight MFMAs; per group it also issues LOADS
 // 1 KB loads into registers (16 bytes a lane, from a window that stays in L2)
-// and LDSR 1 KB LDS reads.  The loaded registers are the A operands of the
-// group after next, as in a kernel that prefetches.  KIND 0: bf16 32x32x16;
+// and LDSR 1 KB LDS reads.  The loaded registers are the A operands of a group
+// five groups later, as in a kernel that prefetches.  KIND 0: bf16 32x32x16;
 // 1: the block-scaled 32x32x64 FP6 x FP4 form.  Lane 0 of every wavefront
 // reports the constant-clock (100 MHz) and shader-clock time of the loop.
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -207,8 +207,13 @@ __global__ void mfma_feed_kernel(const unsigned char* __restrict__ p, uint64_t* 
   const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<unsigned char*>(p) + (int64_t)(blockIdx.x & 63) * 262144, 0, 262144u, 0x00020000);
   constexpr int NB = LOADS > 0 ? LOADS : 1;
-  u32x4 cur[NB], nxt[NB], nxt2[NB];
-  for (int j = 0; j < NB; ++j) cur[j] = nxt[j] = nxt2[j] = u32x4{0x3f803f80u + (uint32_t)lane, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  // The loaded registers are used DEPTH - 1 groups after they were asked for
+  // (about 1300 clocks of matrix work: more than L2's latency), in a loop
+  // unrolled DEPTH times so that the buffers keep static names.
+  constexpr int DEPTH = 6;
+  u32x4 buf[DEPTH][NB];
+  for (int d = 0; d < DEPTH; ++d)
+    for (int j = 0; j < NB; ++j) buf[d][j] = u32x4{0x3f803f80u + (uint32_t)lane, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
   u32x4 lv = {0u, 0u, 0u, 0u};
   f32x16_t acc[2];
   for (int t = 0; t < 2; ++t)
@@ -219,40 +224,38 @@ __global__ void mfma_feed_kernel(const unsigned char* __restrict__ p, uint64_t* 
   const uint64_t c0 = __builtin_amdgcn_s_memtime(), t0 = __builtin_amdgcn_s_memrealtime();
   // (the loop has no side effects of its own: tie it between the two clock reads)
   asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]) : "s"(c0), "s"(t0));
-  for (int it = 0; it < iters; ++it) {
+  for (int it = 0; it < iters; it += DEPTH) {
 #pragma unroll
-    for (int j = 0; j < LOADS; ++j)
-      nxt2[j] = __builtin_amdgcn_raw_buffer_load_b128(r, lane_off + (uint32_t)(j * 1024), (uint32_t)((it & 7) * 8192), 0);
-    // (DMA: as many 1 KB loads straight into LDS instead, four groups ahead of
-    // the LDS reads that would use them)
+    for (int d = 0; d < DEPTH; ++d) {
 #pragma unroll
-    for (int j = 0; j < DMA; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + ((wave * 16 + (it & 3) * 4 + (j & 3)) * 1024) % 65536), 16,
-                                               lane_off + (uint32_t)(j * 1024), (uint32_t)((it & 7) * 8192), 0, 0);
-    if (DMA) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * DMA) & 0xF) | (((3 * DMA) >> 4) << 14));   // at most three groups' loads out
+      for (int j = 0; j < LOADS; ++j)
+        buf[d][j] = __builtin_amdgcn_raw_buffer_load_b128(r, lane_off + (uint32_t)(j * 1024), (uint32_t)(((it + d) & 7) * 8192), 0);
+      // (DMA: as many 1 KB loads straight into LDS instead, at most three
+      // groups' worth outstanding)
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-      const u32x4 a = cur[m % NB];
-      if constexpr (KIND == 0) {
-        acc[m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), bop, acc[m & 1], 0, 0, 0);
-      } else {
-        const i32x8_t a8 = {(int)a[0], (int)a[1], (int)a[2], (int)a[3], (int)a[0], (int)a[1], 0, 0};
-        const i32x8_t b8 = {(int)a[1], (int)a[2], (int)a[3], (int)a[0], 0, 0, 0, 0};
-        acc[m & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[m & 1], 2, 4, 0, 127, 0, 127);
+      for (int j = 0; j < DMA; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(lds + ((wave * 16 + (d & 3) * 4 + (j & 3)) * 1024) % 65536), 16,
+                                                 lane_off + (uint32_t)(j * 1024), (uint32_t)(((it + d) & 7) * 8192), 0, 0);
+      if (DMA) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * DMA) & 0xF) | (((3 * DMA) >> 4) << 14));
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        const u32x4 a = buf[(d + 1) % DEPTH][m % NB];             // the oldest buffer
+        if constexpr (KIND == 0) {
+          acc[m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), bop, acc[m & 1], 0, 0, 0);
+        } else {
+          const i32x8_t a8 = {(int)a[0], (int)a[1], (int)a[2], (int)a[3], (int)a[0], (int)a[1], 0, 0};
+          const i32x8_t b8 = {(int)a[1], (int)a[2], (int)a[3], (int)a[0], 0, 0, 0, 0};
+          acc[m & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[m & 1], 2, 4, 0, 127, 0, 127);
+        }
+        if (m < LDSR / 2) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+            lv ^= *reinterpret_cast<const u32x4*>(lds + ((wave * 16 + m * 2 + q) * 1024 + lane * 16) % 65536);
+        }
       }
-      if (m < LDSR / 2) {
-#pragma unroll
-        for (int q = 0; q < 2; ++q)
-          lv ^= *reinterpret_cast<const u32x4*>(lds + ((wave * 16 + m * 2 + q) * 1024 + lane * 16) % 65536);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < NB; ++j) {
-      cur[j] = nxt[j];
-      nxt[j] = nxt2[j];
     }
   }
-  asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(cur[0][0]), "+v"(nxt[0][0]));
+  asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(buf[0][0][0]), "+v"(buf[DEPTH - 1][0][0]));
   const uint64_t c1 = __builtin_amdgcn_s_memtime(), t1 = __builtin_amdgcn_s_memrealtime();
   float v = 0.f;
   for (int t = 0; t < 2; ++t)

@@ -122,7 +122,7 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
     return out
 
 
-def mfma_feed_probe(iters: int = 2000):
+def mfma_feed_probe(iters: int = 1998):
     """What feeding the matrix cores costs: per group of eight MFMAs, the
     median over all wavefronts of the loop time in shader clocks (and ns), for
     a pure MFMA stream and with 1 KB register loads / LDS reads beside it, one
