@@ -220,6 +220,7 @@ __global__ void mfma_feed_kernel(const unsigned char* __restrict__ p, uint64_t* 
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
   bf16x8_t bop;
   for (int i = 0; i < 8; ++i) bop[i] = (__bf16)1.0f;
+  const i32x8_t b8 = {0x22222222 + lane, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};
   const uint32_t lane_off = (uint32_t)wave * 65536u + (uint32_t)lane * 16u;
   const uint64_t c0 = __builtin_amdgcn_s_memtime(), t0 = __builtin_amdgcn_s_memrealtime();
   // (the loop has no side effects of its own: tie it between the two clock reads)
@@ -243,8 +244,9 @@ __global__ void mfma_feed_kernel(const unsigned char* __restrict__ p, uint64_t* 
         if constexpr (KIND == 0) {
           acc[m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), bop, acc[m & 1], 0, 0, 0);
         } else {
-          const i32x8_t a8 = {(int)a[0], (int)a[1], (int)a[2], (int)a[3], (int)a[0], (int)a[1], 0, 0};
-          const i32x8_t b8 = {(int)a[1], (int)a[2], (int)a[3], (int)a[0], 0, 0, 0, 0};
+          // (the eight-register operand is two loads' registers side by side: no copies)
+          const u32x4 a2 = buf[(d + 1) % DEPTH][(m + 1) % NB];
+          const i32x8_t a8 = {(int)a[0], (int)a[1], (int)a[2], (int)a[3], (int)a2[0], (int)a2[1], (int)a2[2], (int)a2[3]};
           acc[m & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[m & 1], 2, 4, 0, 127, 0, 127);
         }
         if (m < LDSR / 2) {
