@@ -363,8 +363,7 @@ PJRT_Error* PluginAttributes(PJRT_Plugin_Attributes_Args* a) {
   // asks for it before serialising a module
   static int64_t current[3] = {1, 0, 0}, minimum[3] = {0, 9, 0};
   static PJRT_NamedValue attrs[2];
-  static bool made = false;
-  if (!made) {
+  static const bool made = [] {               // once, whichever thread asks first
     ensure_python();
     Gil g;
     if (PyObject* mod = PyImport_ImportModule("metaljax_amd.engine")) {
@@ -388,8 +387,9 @@ PJRT_Error* PluginAttributes(PJRT_Plugin_Attributes_Args* a) {
       attrs[i].int64_array_value = values[i];
       attrs[i].value_size = 3;
     }
-    made = true;
-  }
+    return true;
+  }();
+  (void)made;
   a->attributes = attrs;
   a->num_attributes = 2;
   return nullptr;
@@ -1017,10 +1017,8 @@ PJRT_Error* ContextDestroy(PJRT_ExecuteContext_Destroy_Args* a) {
 
 }  // namespace
 
-extern "C" __attribute__((visibility("default"))) const PJRT_Api* GetPjrtApi() {
-  static PJRT_Api api;
-  static bool made = false;
-  if (made) return &api;
+namespace {
+void fill_api(PJRT_Api& api) {
   memset(&api, 0, sizeof(api));
   api.struct_size = PJRT_Api_STRUCT_SIZE;
   api.pjrt_api_version.struct_size = PJRT_Api_Version_STRUCT_SIZE;
@@ -1174,6 +1172,14 @@ extern "C" __attribute__((visibility("default"))) const PJRT_Api* GetPjrtApi() {
   HAVE(PJRT_ExecuteContext_Destroy, ContextDestroy);
 #undef HAVE
 #undef LACK
-  made = true;
-  return &api;
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) const PJRT_Api* GetPjrtApi() {
+  static const PJRT_Api* const table = [] {   // filled once, whichever thread asks first
+    static PJRT_Api api;
+    fill_api(api);
+    return &api;
+  }();
+  return table;
 }
