@@ -36,7 +36,7 @@
 //   * weight scales: 16 bytes a row per K-quad, direct-to-LDS, double buffered;
 //     the lane shifts its block's byte to bits 0-7.
 //   * activation terms: straight from global (L2-resident) into operand
-//     registers, two K-steps ahead.
+//     registers, one K-step ahead.
 // Per K-step a wavefront issues 32 MFMAs of 32x32x64 (2 K-halves x 2 terms x 2
 // row tiles x 4 column tiles) against 24 + 8 loads.  (The 16x16x128 form of
 // the instruction sustains well under half the rate of the 32x32x64 form.)
@@ -316,13 +316,15 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
 
   // Loads retire in order, so a wait can only say "all but the newest n have
   // landed": the order of issue has to be the order of use.  A K-step i uses
-  // its activation terms A(i) and its weight codes W(i); step i issues A(i+2)
-  // during its first two MFMA groups and W(i+3) during its last two, and
+  // its activation terms A(i) and its weight codes W(i); step i issues A(i+1)
+  // during its first two MFMA groups and W(i+2) during its last two, and
   // before its last group waits for W(i+1) and reads its fragments, so that a
   // step starts with its weight operands already in registers.  The prologue issues in the same
-  // order (W0 A0 W1 A1 W2), which keeps every count in the loop valid on its
+  // order (W0 A0 W1), which keeps every count in the loop valid on its
   // first pass.  A step issues 20 loads, the first of a quad 10 more (its
-  // activation scales and the next quad's weight scales).
+  // activation scales and the next quad's weight scales).  (Asking further
+  // ahead -- A(i+2), W(i+3) -- measured 2 % slower on C4: a wavefront keeps
+  // about sixteen loads in flight and sits in issue beyond that.)
   i32x8 bfq[2][2][4];                             // [step parity][u][nt] weight fragments
   auto read_bf = [&](int stage, i32x8 (&dst)[2][4]) {
     const unsigned char* st = wbase + stage * kStageBytes;
@@ -343,17 +345,15 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
     dma_w(kstep_of(0), 0);
     issue_a(kstep_of(0), areg[0]);
     dma_w(kstep_of(1), 1);
-    issue_a(kstep_of(1), areg[1]);
-    dma_w(kstep_of(2), 2);
-    wait_vmcnt<40>();                              // W0 and the first scales
+    wait_vmcnt<20>();                              // W0 and the first scales
     read_bf(0, bfq[0]);
     read_sbq(0);
     auto step = [&](int qi, auto tc) __attribute__((always_inline)) {
       constexpr int t = decltype(tc)::value;
       const int i = 4 * qi + t;
-      // A(i) has landed once at most W(i+1) and the previous step's loads are out
-      wait_vmcnt<(t == 1 ? 38 : 28)>();
-      const int ks_a = kstep_of(i + 2), ks_w = kstep_of(i + 3);
+      // A(i) has landed once at most W(i+1), the loads issued after it, are out
+      wait_vmcnt<8>();
+      const int ks_a = kstep_of(i + 1), ks_w = kstep_of(i + 2);
       int sb[2][4];
 #pragma unroll
       for (int u = 0; u < 2; ++u)
@@ -375,20 +375,20 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);
         if (g < 2) {
-          issue_a_part(ks_a, areg[(t + 2) & 3], 2 * g);
-          issue_a_part(ks_a, areg[(t + 2) & 3], 2 * g + 1);
+          issue_a_part(ks_a, areg[(t + 1) & 3], 2 * g);
+          issue_a_part(ks_a, areg[(t + 1) & 3], 2 * g + 1);
           if (t == 0 && g == 0) {
             issue_sa(quad_of(qi + 1), sa_nxt);
             dma_s(quad_of(qi + 1), (qi + 1) & 1);
           }
         } else {
-          dma_w_part(ks_w, (t + 3) & 3, 2 * (g - 2));
-          dma_w_part(ks_w, (t + 3) & 3, 2 * (g - 2) + 1);
+          dma_w_part(ks_w, (t + 2) & 3, 2 * (g - 2));
+          dma_w_part(ks_w, (t + 2) & 3, 2 * (g - 2) + 1);
         }
         if (g == 2) {
           // W(i+1): everything but the previous step's loads and this step's so far;
           // the fragment reads then run under the last MFMA group
-          wait_vmcnt<(t <= 1 ? 46 : 36)>();
+          wait_vmcnt<(t == 0 ? 26 : 16)>();
           read_bf((t + 1) & 3, bfq[(t + 1) & 1]);
           if (t == 3) read_sbq((qi + 1) & 1);
         }
