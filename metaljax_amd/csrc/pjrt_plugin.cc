@@ -209,7 +209,7 @@ namespace {
 struct Program {
   std::atomic<int> refs{1};
   PyObject* ex = nullptr;
-  std::string name, fingerprint;
+  std::string name, fingerprint, code;    // code: the module as it was handed to Compile
   size_t num_params = 0;
   std::vector<PJRT_Buffer_Type> out_types;
   std::vector<int64_t> out_dims;          // every output's dimensions, back to back
@@ -533,6 +533,7 @@ PJRT_Error* ClientCompile(PJRT_Client_Compile_Args* a) {
   if (!ex) return python_failure("compile_program");
   auto* p = new Program;
   p->ex = ex;
+  p->code.assign(a->program->code, a->program->code_size);
   std::vector<int64_t> types;
   size_t outputs = 0;
   bool ok = read_attr_text(ex, "name", &p->name) && read_attr_text(ex, "fingerprint", &p->fingerprint) &&
@@ -784,6 +785,31 @@ PJRT_Error* ExecutableOutputDimensions(PJRT_Executable_OutputDimensions_Args* a)
 PJRT_Error* ExecutableFingerprint(PJRT_Executable_Fingerprint_Args* a) {
   a->executable_fingerprint = a->executable->program->fingerprint.data();
   a->executable_fingerprint_size = a->executable->program->fingerprint.size();
+  return nullptr;
+}
+
+// The program an executable was made from: nothing is optimised, so it is the
+// module the caller compiled, in the format it came in ("mlir").
+PJRT_Error* ExecutableOptimizedProgram(PJRT_Executable_OptimizedProgram_Args* a) {
+  REQUIRE(a->program, "no program to fill");
+  static const char format[] = "mlir";
+  const std::string& code = a->executable->program->code;
+  a->program->format = format;
+  a->program->format_size = sizeof(format) - 1;
+  if (!a->program->code) {                    // a query for the size
+    a->program->code_size = code.size();
+    return nullptr;
+  }
+  REQUIRE(a->program->code_size >= code.size(), "the program buffer is too small");
+  memcpy(a->program->code, code.data(), code.size());
+  a->program->code_size = code.size();
+  return nullptr;
+}
+
+PJRT_Error* LoadedLogicalIds(PJRT_LoadedExecutable_AddressableDeviceLogicalIds_Args* a) {
+  static PJRT_LogicalDeviceIds ids[1] = {{0, 0}};   // replica 0, partition 0 on the one device
+  a->addressable_device_logical_ids = ids;
+  a->num_addressable_device_logical_ids = 1;
   return nullptr;
 }
 
@@ -1102,7 +1128,7 @@ void fill_api(PJRT_Api& api) {
   HAVE(PJRT_Executable_OutputElementTypes, ExecutableOutputElementTypes);
   HAVE(PJRT_Executable_OutputDimensions, ExecutableOutputDimensions);
   HAVE(PJRT_Executable_Fingerprint, ExecutableFingerprint);
-  LACK(PJRT_Executable_OptimizedProgram);
+  HAVE(PJRT_Executable_OptimizedProgram, ExecutableOptimizedProgram);
   LACK(PJRT_Executable_Serialize);
   LACK(PJRT_Executable_GetCompiledMemoryStats);
   LACK(PJRT_Executable_GetCompileOptions);
@@ -1115,7 +1141,7 @@ void fill_api(PJRT_Api& api) {
   HAVE(PJRT_LoadedExecutable_Execute, LoadedExecute);
   HAVE(PJRT_LoadedExecutable_Fingerprint, LoadedFingerprint);
   LACK(PJRT_LoadedExecutable_GetDeviceAssignment);
-  LACK(PJRT_LoadedExecutable_AddressableDeviceLogicalIds);
+  HAVE(PJRT_LoadedExecutable_AddressableDeviceLogicalIds, LoadedLogicalIds);
 
   HAVE(PJRT_Buffer_Destroy, BufferDestroy);
   HAVE(PJRT_Buffer_ElementType, BufferElementType);

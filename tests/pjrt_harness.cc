@@ -657,6 +657,25 @@ int pjrt_harness_walk(int buffer, int exe) {
   ARGS(PJRT_Executable_Serialize_Args, ser);
   ser.executable = ge.executable;
   STEP(45, taken(g_api->PJRT_Executable_Serialize(&ser)) == (int)PJRT_Error_Code_UNIMPLEMENTED);
+  {   // the program comes back as it went in: size query first, then the bytes
+    PJRT_Program prog;
+    memset(&prog, 0, sizeof(prog));
+    prog.struct_size = PJRT_Program_STRUCT_SIZE;
+    ARGS(PJRT_Executable_OptimizedProgram_Args, opg);
+    opg.executable = ge.executable;
+    opg.program = &prog;
+    STEP(50, taken(g_api->PJRT_Executable_OptimizedProgram(&opg)) == 0 && prog.code_size > 0 &&
+                 std::string(prog.format, prog.format_size) == "mlir");
+    std::vector<char> text(prog.code_size);
+    prog.code = text.data();
+    STEP(51, taken(g_api->PJRT_Executable_OptimizedProgram(&opg)) == 0 &&
+                 std::string(text.data(), text.size()).find("func.func") != std::string::npos);
+    ARGS(PJRT_LoadedExecutable_AddressableDeviceLogicalIds_Args, lids);
+    lids.executable = le;
+    STEP(52, taken(g_api->PJRT_LoadedExecutable_AddressableDeviceLogicalIds(&lids)) == 0 &&
+                 lids.num_addressable_device_logical_ids == 1 && lids.addressable_device_logical_ids[0].replica == 0 &&
+                 lids.addressable_device_logical_ids[0].partition == 0);
+  }
   ARGS(PJRT_Executable_Destroy_Args, xd);
   xd.executable = ge.executable;
   STEP(46, taken(g_api->PJRT_Executable_Destroy(&xd)) == 0);
