@@ -214,6 +214,7 @@ struct Program {
   std::vector<PJRT_Buffer_Type> out_types;
   std::vector<int64_t> out_dims;          // every output's dimensions, back to back
   std::vector<size_t> out_ranks;
+  std::vector<int64_t> donated;           // parameters whose buffers the program consumes
   std::vector<const char*> out_kinds, param_kinds;
   std::vector<size_t> out_kind_sizes, param_kind_sizes;
 };
@@ -538,7 +539,7 @@ PJRT_Error* ClientCompile(PJRT_Client_Compile_Args* a) {
   size_t outputs = 0;
   bool ok = read_attr_text(ex, "name", &p->name) && read_attr_text(ex, "fingerprint", &p->fingerprint) &&
             read_attr_size(ex, "num_outputs", &outputs) && read_attr_size(ex, "num_params", &p->num_params) &&
-            read_attr_ints(ex, "out_types", &types);
+            read_attr_ints(ex, "out_types", &types) && read_attr_ints(ex, "donated_params", &p->donated);
   if (ok) {
     PyObject* dims = PyObject_GetAttrString(ex, "out_dims");
     PyObject* fast = dims ? PySequence_Fast(dims, "out_dims: expected a sequence") : nullptr;
@@ -892,6 +893,22 @@ PJRT_Error* LoadedExecute(PJRT_LoadedExecutable_Execute_Args* a) {
   }
   Py_DECREF(fast);
   for (size_t i = 0; i < n; ++i) a->output_lists[0][i] = made[i];
+  // A donated parameter's buffer is consumed by the call (reference
+  // metal_pjrt.cc:1032-1036) unless the caller lists it as not donatable: its
+  // value is dropped and the handle reports deleted.  (The engine writes fresh
+  // outputs, so nothing aliases the dropped value.)
+  for (int64_t d : p->donated) {
+    if (d < 0 || (size_t)d >= a->num_args) continue;
+    bool keep = false;
+    if (a->options)
+      for (size_t k = 0; k < a->options->num_non_donatable_input_indices; ++k)
+        keep = keep || a->options->non_donatable_input_indices[k] == d;
+    if (keep) continue;
+    PJRT_Buffer* b = a->argument_lists[0][d];
+    if (b->external_refs > 0) continue;     // someone outside still reads it
+    Py_CLEAR(b->value);
+    b->deleted = true;
+  }
   if (a->device_complete_events) a->device_complete_events[0] = ready_event();
   return nullptr;
 }

@@ -20,8 +20,9 @@ argument meaning and result type (reference plugin/metal_pjrt.cc):
     device_kind() -> str, stablehlo_version() -> [int] metal_pjrt.cc:382, :440
 
 The reference's executables also carry `forwarded_outputs`-style donation
-plumbing inside `execute`; here `donated_params` is reported and donation is
-not acted on (every output is a fresh buffer).
+plumbing inside `execute`; here `donated_params` is reported, every output is
+a fresh buffer, and the plugin drops a donated argument's buffer after the
+call (csrc/pjrt_plugin.cc).
 """
 
 from __future__ import annotations

@@ -381,6 +381,18 @@ int pjrt_harness_to_host(int handle, void* dst, int64_t* size) {
   return settle(a.event);
 }
 
+namespace {
+int64_t g_keep[16];
+int g_num_keep = 0;
+}  // namespace
+
+// Parameters the next execute lists as not donatable (at most 16).
+int pjrt_harness_keep_inputs(const int64_t* indices, int n) {
+  g_num_keep = n < 16 ? n : 16;
+  for (int i = 0; i < g_num_keep; ++i) g_keep[i] = indices[i];
+  return 0;
+}
+
 int pjrt_harness_execute(int exe, const int* args, int num_args, int* outs, int out_cap, int* num_outs) {
   NEED_OPEN();
   if (exe < 0 || exe >= (int)g_exes.size() || !g_exes[exe]) return harness_failure("no such executable");
@@ -414,6 +426,9 @@ int pjrt_harness_execute(int exe, const int* args, int num_args, int* outs, int 
   PJRT_ExecuteOptions opts;
   memset(&opts, 0, sizeof(opts));
   opts.struct_size = PJRT_ExecuteOptions_STRUCT_SIZE;
+  opts.non_donatable_input_indices = g_keep;
+  opts.num_non_donatable_input_indices = (size_t)g_num_keep;
+  g_num_keep = 0;
   PJRT_LoadedExecutable_Execute_Args a;
   memset(&a, 0, sizeof(a));
   a.struct_size = PJRT_LoadedExecutable_Execute_Args_STRUCT_SIZE;

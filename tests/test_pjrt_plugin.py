@@ -196,6 +196,32 @@ def test_the_smaller_entry_points_answer_as_the_c_api_says(plugin):
     assert rc == INVALID_ARGUMENT and "deleted" in plugin.error()
 
 
+def test_a_donated_parameter_is_consumed_unless_the_caller_keeps_it(plugin):
+    """`jax.buffer_donor` / `tf.aliasing_output` on a parameter: the call
+    consumes that buffer (reference metal_pjrt.cc:1032-1036, :1109-1116) unless
+    the execute options list it as not donatable."""
+    text = T.float_dot(8, 16, 4, el="f32").replace("%x: tensor<4x8xf32>", "%x: tensor<4x8xf32> {jax.buffer_donor = true}")
+    assert engine.compile_program(text).donated_params == [2]
+    rc, exe = plugin.compile(text)
+    plugin.ok(rc)
+    rng = np.random.default_rng(1)
+    w, r, x = (rng.standard_normal(s).astype(np.float32) for s in ((8, 16), (8,), (4, 8)))
+    (_, bw), (_, br), (_, bx) = plugin.buffer(w, F32), plugin.buffer(r, F32), plugin.buffer(x, F32)
+    plugin.h.pjrt_harness_keep_inputs.argtypes = [ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
+    plugin.ok(plugin.h.pjrt_harness_keep_inputs((ctypes.c_int64 * 1)(2), 1))
+    rc, outs = plugin.execute(exe, [bw, br, bx])
+    plugin.ok(rc)
+    assert not plugin.buffer_info(bx)["deleted"]          # kept
+    rc, outs = plugin.execute(exe, [bw, br, bx])
+    plugin.ok(rc)
+    assert plugin.buffer_info(bx)["deleted"] and not plugin.buffer_info(bw)["deleted"]
+    rc, raw = plugin.to_host(outs[0])
+    plugin.ok(rc)
+    np.testing.assert_allclose(np.frombuffer(raw, np.float32).reshape(4, 16), x @ (w * r[:, None]), rtol=1e-5, atol=1e-5)
+    rc, _ = plugin.execute(exe, [bw, br, bx])              # a consumed buffer is not an argument any more
+    assert rc == INVALID_ARGUMENT and "deleted" in plugin.error()
+
+
 def test_bf16_bytes_round_trip(plugin):
     bits = np.array([0x3F80, 0xC000, 0x0000, 0x7F7F], np.uint16)
     rc, b = plugin.buffer(bits, BF16)
