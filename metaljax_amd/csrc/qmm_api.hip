@@ -321,6 +321,12 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
     if (kernel) *kernel = QMM_KERNEL_GEMV;
     if (grid) *grid = (int)ceil_div(N, 16 * t);
     if (block) *block = 64 * waves;
+  } else if (K % 256 == 0 && (mode == QMM_MODE_MXFP4 || bits == 4 || bits == 8)) {
+    // the split-role kernel (bf16 tables assumed): 256-row tiles, four
+    // multiplying and four dequantizing wavefronts
+    if (kernel) *kernel = QMM_KERNEL_GEMM;
+    if (grid) *grid = (int)(ceil_div(N, 128) * ceil_div(M, 256));
+    if (block) *block = 512;
   } else {
     const int64_t bm = gemm_row_tile(M, 1);
     if (kernel) *kernel = QMM_KERNEL_GEMM;

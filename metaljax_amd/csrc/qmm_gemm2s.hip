@@ -1,16 +1,17 @@
-// Grouped (per-expert) prefill-regime quantized matmul for short row groups on
-// gfx950: experts of up to about 160 rows, the MoE prefill case.  It serves the
-// expert-indexed product that the reference hands to mx.gather_qmm
-// (src/metaljax/moe.py:1283-1340) with the dequantization semantics of
-// src/metaljax/qmm.py:71-79 (w = scale * q + bias as one fma).
+// Prefill-regime quantized matmul on gfx950 with the wavefronts' roles split:
+// the grouped (per-expert) product that the reference hands to mx.gather_qmm
+// (src/metaljax/moe.py:1283-1340) and the dense product of
+// mx.quantized_matmul (src/metaljax/qmm.py:2491) at M > 16, with the
+// dequantization semantics of src/metaljax/qmm.py:71-79 (w = scale * q + bias
+// as one fma).
 //
-// Why a second kernel.  With row groups this short a 128-column weight tile is
-// dequantized for very little matrix work: in the general kernel, where every
-// wavefront both dequantizes and multiplies, a K-tile of a 128-row tile takes
-// 0.78 us of which the MFMAs are a third; the dequantization (about 100 vector
-// ALU instructions per thread, the LDS writes, the loads that feed them) is
-// the largest part, and a single wavefront a SIMD cannot run it beside its own
-// MFMAs: it issues one instruction per four clocks, of any kind.
+// Why a second kernel.  In the general kernel every wavefront both
+// dequantizes and multiplies, and a single wavefront a SIMD issues one
+// instruction per four clocks, of any kind: the dequantization of a K-tile
+// (about 100 vector ALU instructions per thread, the LDS writes, the loads
+// that feed them) stands in the way of its own MFMAs.  With short row groups
+// that is most of the time (a K-tile of a 128-row tile took 0.78 us of which
+// the MFMAs were a third).
 //
 // So the roles are split, as in the decode kernel.  A workgroup is eight
 // wavefronts, two a SIMD:
@@ -21,14 +22,15 @@
 //   * consumers (wavefronts 0-3) load their activation fragments (the re-laid
 //     ax[k/8][row] form of the general kernel), read the weight fragments of
 //     K-tile t from LDS and issue the MFMAs.
-// The vector ALU and the matrix core of a SIMD are then driven by different
-// wavefronts and overlap; one workgroup barrier per K-tile publishes tile t+1
-// and frees the stage of tile t-1 (three stages).
+// One workgroup barrier per K-tile publishes tile t+1 and frees the stage of
+// tile t-1 (three stages).
 //
-// Tile: up to 160 rows x 128 columns.  Consumer w multiplies row block w
-// (32 rows) with the whole weight tile; rows 128..159, when the tile has them,
-// are a fifth block split by columns: consumer w multiplies it with column
-// block w.  Longer experts take several tiles.
+// Tile: up to 256 rows x 128 columns, and the rows a tile really holds pick
+// one of three loops.  Up to 128 rows: consumer w multiplies row block w
+// (32 rows) with the whole weight tile.  Up to 160: rows 128..159 are a fifth
+// block split by columns, consumer w multiplies it with column block w.  More:
+// consumer w multiplies row blocks w and w + 4 (every weight fragment read
+// from LDS then feeds two MFMAs).  Longer experts take several tiles.
 #include <type_traits>
 
 #include "qmm_gemm2_common.hpp"
@@ -40,8 +42,18 @@ namespace {
 using namespace g2;
 
 constexpr int kS = 3;                 // LDS stages: K-tile t lives in stage t % 3
-constexpr int kTileRows = 160;        // four row blocks + the fifth
-constexpr int kAR = 3;                // activation fragments: K-tile t lives in ring slot t % 3
+constexpr int kTileRows = 256;        // eight row blocks, two a consumer
+constexpr int kAR = 3;                // activation fragments: K-tile t lives in ring slot t % 3 (t % 2 on full tiles)
+
+// Rows [lo, hi) of expert i; a product without row offsets is one expert of all rows.
+__device__ __forceinline__ void expert_rows(const Gemm2Args& a, int i, int& lo, int& hi) {
+  if (a.row_offsets) {
+    group_rows(a, i, lo, hi);
+  } else {
+    lo = 0;
+    hi = a.R;
+  }
+}
 // Table rows staged in LDS (a row's scales / biases of the whole K when they
 // fit 128 bytes): 128 + 16 bytes a row, so that eight rows fall on different banks.
 constexpr int kTabRow = 144;
@@ -67,13 +79,22 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
   int m_tiles = 0;
   for (int i = 0; i < a.E; ++i) {
     int lo, hi;
-    group_rows(a, i, lo, hi);
+    expert_rows(a, i, lo, hi);
     m_tiles += (hi - lo + kTileRows - 1) / kTileRows;
   }
   const int band = (n_tiles + 7) / 8;
-  const int l = blockIdx.x >> 3;
-  const int tile_m = l / band;
-  const int tile_n = (blockIdx.x & 7) * band + l % band;
+  const int xcd = blockIdx.x & 7, l = blockIdx.x >> 3;
+  int tile_m = l / band;
+  int tile_n = xcd * band + l % band;
+  if (!a.row_offsets) {
+    // one expert of all rows: an eighth of the grid takes a contiguous run of
+    // tiles, column tile fastest, so its workgroups share few activation rows
+    const int total = n_tiles * m_tiles, per = (total + 7) / 8;
+    const int t = xcd * per + l;
+    if (l >= per || t >= total) return;
+    tile_m = t / n_tiles;
+    tile_n = t % n_tiles;
+  }
   if (tile_m >= m_tiles || tile_n >= n_tiles) return;
   int e = 0, row_lo = 0, row_hi = 0, mt_idx = 0;
   {
@@ -81,7 +102,7 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     bool found = false;
     for (int i = 0; i < a.E; ++i) {
       int lo, hi;
-      group_rows(a, i, lo, hi);
+      expert_rows(a, i, lo, hi);
       const int tiles = (hi - lo + kTileRows - 1) / kTileRows;
       if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
       t -= tiles;
@@ -238,12 +259,12 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       }
       float sc, bi;
       entry(clampk(kt + 2), std::integral_constant<int, (t + 2) & 3>{}, t >= 2 ? tw_nxt : tw_cur, sc, bi);
+      // the step's barrier as soon as the write has landed (the consumers reach
+      // theirs before their last k-step); the next tile's arithmetic after it
+      lds_barrier();
+      __builtin_amdgcn_sched_barrier(0);
       dequant_tile(pend, wr[(t12 + 2) % 12], sc, bi);
       if (t == 3) tw_cur = tw_nxt;
-      lds_barrier();
-      // every step does its own tile's arithmetic: work moved across the
-      // barrier would make the consumers wait for a long step and the
-      // producers idle in the short ones
       __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
@@ -278,11 +299,17 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
   // ========================= consumers: the MFMAs ==========================
   const int wm = wave;                             // row block, and column block of the fifth
   const int li = lane & 31, kh = lane >> 5;
-  const bool five = m0 + 128 < m_end;              // uniform over the workgroup
+  // How many rows the tile holds decides the loop, for the whole workgroup:
+  //   0: up to 128, one row block a consumer;
+  //   1: up to 160, plus a fifth block split by columns;
+  //   2: up to 256, two row blocks a consumer (w and w + 4).
+  const int path = m_end - m0 <= 128 ? 0 : (m_end - m0 <= 160 ? 1 : 2);
+  const bool five = path == 1, two = path == 2;
   // lane (row li, k-half kh) of k-step ks reads ax[(kt*8 + ks*2 + kh) * Rp + row]
   const auto ra = make_rsrc(a.ax, (int64_t)(a.K / 8) * a.Rp * 16);
   const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + wm * 32 + li) * 16);
-  const uint32_t avo1 = avo + (uint32_t)((4 - wm) * 512);       // the fifth block's rows
+  // the second block: the fifth block's rows, or row block w + 4
+  const uint32_t avo1 = avo + (uint32_t)(five ? (4 - wm) * 512 : 128 * 16);
   typedef u32x4 AFrag[4][2];
   auto load_a_part = [&](int kt, AFrag& dst, int ks, auto nac) __attribute__((always_inline)) {
     const uint32_t so = (uint32_t)((kt * 8 + ks * 2) * 16) * (uint32_t)a.Rp;
@@ -290,12 +317,14 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     if constexpr (decltype(nac)::value == 2) dst[ks][1] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo1, so, 0);
   };
 
-  f32x16 acc[4], accx;
+  f32x16 acc[4], acc2[4];                           // acc2[0] doubles as the fifth block's accumulator
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
-    accx[r] = 0.f;
+    for (int j = 0; j < 4; ++j) {
+      acc[j][r] = 0.f;
+      acc2[j][r] = 0.f;
+    }
   }
   AFrag af[kAR];
   bf16x8 fb[2][4], fbx[2];                          // B fragments: k-step ks in set ks & 1
@@ -307,60 +336,102 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       fbx[set] = *reinterpret_cast<const bf16x8*>(pbase + swz(wm * 32 + li, ks * 2 + kh));
   };
 
-  auto run = [&](auto fc) __attribute__((always_inline)) {
-    constexpr bool FIVE = decltype(fc)::value;
-    const std::integral_constant<int, FIVE ? 2 : 1> nac;
-    // tiles 0 and 1 of the activations in flight before the first barrier
+  auto run = [&](auto pathc) __attribute__((always_inline)) {
+    constexpr int PATH = decltype(pathc)::value;
+    constexpr bool FIVE = PATH == 1, TWO = PATH == 2;
+    // activation K-tiles in registers: three (two K-tiles ahead), or two on a
+    // full tile, whose 128 accumulator registers leave room for no more
+    constexpr int AR = TWO ? 2 : 3;
+    const std::integral_constant<int, PATH == 0 ? 1 : 2> nac;
+    const std::integral_constant<bool, FIVE> fc;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) load_a_part(0, af[0], ks, nac);
+    if constexpr (AR == 3) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_a_part(clampk(1), af[1], ks, nac);
+      for (int ks = 0; ks < 4; ++ks) load_a_part(clampk(1), af[1], ks, nac);
+    }
     lds_barrier();                                  // tile 0 is published
     read_b(smem, 0, 0, fc);
-    auto cstep = [&](int kt, auto tc) __attribute__((always_inline)) {
-      constexpr int t = decltype(tc)::value;        // kt % 3
+    auto cstep = [&](int kt, auto tc, auto ac) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;        // kt % 3: the LDS stage
+      constexpr int as = decltype(ac)::value;       // kt % AR: the activation slot
       const unsigned char* pb = smem + t * kStage;
       constexpr int nstage = (t + 1) % kS;
-      const int kt2 = clampk(kt + 2);
+      const int ktn = clampk(kt + AR - 1);
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
+        // the next k-step's fragments; in the last k-step those of the next
+        // tile, which the barrier below has published (past the last tile: a
+        // stage that nobody reads)
         if (ks < 3) read_b(pb, ks + 1, (ks + 1) & 1, fc);
-        load_a_part(kt2, af[(t + 2) % kAR], ks, nac);
+        else read_b(smem + nstage * kStage, 0, 0, fc);
+        load_a_part(ktn, af[(as + AR - 1) % AR], ks, nac);
         // the fragment read last feeds the first MFMA: one LDS wait a k-step
         if constexpr (FIVE)
-          accx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[t][ks][1]),
-                                                         fbx[ks & 1], accx, 0, 0, 0);
-        const bf16x8 fa = __builtin_bit_cast(bf16x8, af[t][ks][0]);
+          acc2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[as][ks][1]),
+                                                            fbx[ks & 1], acc2[0], 0, 0, 0);
+        const bf16x8 fa = __builtin_bit_cast(bf16x8, af[as][ks][0]);
 #pragma unroll
         for (int j = 3; j >= 0; --j)
           acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[ks & 1][j], acc[j], 0, 0, 0);
+        if constexpr (TWO) {
+          const bf16x8 fa1 = __builtin_bit_cast(bf16x8, af[as][ks][1]);
+#pragma unroll
+          for (int j = 3; j >= 0; --j)
+            acc2[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, fb[ks & 1][j], acc2[j], 0, 0, 0);
+        }
         // order inside the k-step: the next k-step's fragment reads first (their
         // latency hides under this k-step's MFMAs), the loads spread between the MFMAs
-        if (ks < 3) __builtin_amdgcn_sched_group_barrier(0x100, FIVE ? 5 : 4, 0);
+        constexpr int NM = TWO ? 8 : (FIVE ? 5 : 4);
+        __builtin_amdgcn_sched_group_barrier(0x100, FIVE ? 5 : 4, 0);
 #pragma unroll
-        for (int m = 0; m < (FIVE ? 5 : 4); ++m) {
+        for (int m = 0; m < NM; ++m) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (m < (FIVE ? 2 : 1)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          if (m < (PATH == 0 ? 1 : 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // One barrier a K-tile, before its last k-step: tile kt + 1 is
+        // published (its producers wrote it at the start of their step), and
+        // the producers learn that tile kt - 1 is read (they reuse its stage
+        // in their next step).  The last k-step then fetches the next tile's
+        // first fragments under its own MFMAs.
+        if (ks == 2) lds_barrier();
       }
-      lds_barrier();                                // tile kt + 1 is published, tile kt's stage is free
-      if (kt + 1 < KT) read_b(smem + nstage * kStage, 0, 0, fc);
     };
+    using std::integral_constant;
     int kt = 0;
-    for (; kt + 3 <= KT; kt += 3) {
-      cstep(kt, std::integral_constant<int, 0>{});
-      cstep(kt + 1, std::integral_constant<int, 1>{});
-      cstep(kt + 2, std::integral_constant<int, 2>{});
+    if constexpr (AR == 3) {
+      for (; kt + 3 <= KT; kt += 3) {
+        cstep(kt, integral_constant<int, 0>{}, integral_constant<int, 0>{});
+        cstep(kt + 1, integral_constant<int, 1>{}, integral_constant<int, 1>{});
+        cstep(kt + 2, integral_constant<int, 2>{}, integral_constant<int, 2>{});
+      }
+      if (kt < KT) { cstep(kt, integral_constant<int, 0>{}, integral_constant<int, 0>{}); ++kt; }
+      if (kt < KT) { cstep(kt, integral_constant<int, 1>{}, integral_constant<int, 1>{}); ++kt; }
+    } else {
+      for (; kt + 6 <= KT; kt += 6) {
+        cstep(kt, integral_constant<int, 0>{}, integral_constant<int, 0>{});
+        cstep(kt + 1, integral_constant<int, 1>{}, integral_constant<int, 1>{});
+        cstep(kt + 2, integral_constant<int, 2>{}, integral_constant<int, 0>{});
+        cstep(kt + 3, integral_constant<int, 0>{}, integral_constant<int, 1>{});
+        cstep(kt + 4, integral_constant<int, 1>{}, integral_constant<int, 0>{});
+        cstep(kt + 5, integral_constant<int, 2>{}, integral_constant<int, 1>{});
+      }
+      if (kt < KT) { cstep(kt, integral_constant<int, 0>{}, integral_constant<int, 0>{}); ++kt; }
+      if (kt < KT) { cstep(kt, integral_constant<int, 1>{}, integral_constant<int, 1>{}); ++kt; }
+      if (kt < KT) { cstep(kt, integral_constant<int, 2>{}, integral_constant<int, 0>{}); ++kt; }
+      if (kt < KT) { cstep(kt, integral_constant<int, 0>{}, integral_constant<int, 1>{}); ++kt; }
+      if (kt < KT) { cstep(kt, integral_constant<int, 1>{}, integral_constant<int, 0>{}); ++kt; }
     }
-    if (kt < KT) { cstep(kt, std::integral_constant<int, 0>{}); ++kt; }
-    if (kt < KT) { cstep(kt, std::integral_constant<int, 1>{}); ++kt; }
   };
-  if (five) run(std::true_type{});
-  else run(std::false_type{});
+  if (two) run(std::integral_constant<int, 2>{});
+  else if (five) run(std::integral_constant<int, 1>{});
+  else run(std::integral_constant<int, 0>{});
 
   // ---- epilogue.  D of a 32x32 tile: lane holds column lane % 32 and rows
-  // (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5), r = 0..15.
+  // (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5), r = 0..15.  Block 0 is row block
+  // w over all columns; block 1 the fifth block's column block w, or row
+  // block w + 4 over all columns.
   const bool wide = a.y_dtype != QMM_F32 && (a.N & 7) == 0 &&
                     (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;
   if (wide) {
@@ -368,16 +439,16 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     // share of LDS (free after the last barrier), store 16 bytes a lane
     uint16_t* o16 = reinterpret_cast<uint16_t*>(smem) + wave * (32 * BN);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {                   // 0: row block wm, all columns; 1: the fifth block, column block wm
-      if (i == 1 && !five) break;
-      const int ncb = i == 0 ? 4 : 1;
+    for (int i = 0; i < 2; ++i) {
+      if (i == 1 && !five && !two) break;
+      const int ncb = (i == 0 || two) ? 4 : 1;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (j >= ncb) break;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int rl = (r & 3) + 8 * (r >> 2) + 4 * kh;
-          const float v = i == 0 ? acc[j][r] : accx[r];
+          const float v = i == 0 ? acc[j][r] : acc2[j][r];
           o16[rl * BN + j * 32 + li] =
               (uint16_t)(a.y_dtype == QMM_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
         }
@@ -388,8 +459,8 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
       const int ppr = ncb * 4;                      // 16-byte pieces per row
       for (int q = 0; q < (32 * ppr) / 64; ++q) {
         const int idx = q * 64 + lane, rl = idx / ppr, pc = idx % ppr;
-        const int m = m0 + (i == 0 ? wm : 4) * 32 + rl;
-        const int n = n0 + (i == 0 ? 0 : wm * 32) + pc * 8;
+        const int m = m0 + (i == 0 ? wm : (two ? wm + 4 : 4)) * 32 + rl;
+        const int n = n0 + ((i == 0 || two) ? 0 : wm * 32) + pc * 8;
         if (m < m_end && n < a.N) {
           const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
           *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + n) =
@@ -402,15 +473,20 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {                   // 4: the fifth block
-      if (j == 4 && !five) break;
-      const int n = n0 + (j < 4 ? j : wm) * 32 + li;
+    for (int i = 0; i < 2; ++i) {
+      if (i == 1 && !five && !two) break;
+      const int ncb = (i == 0 || two) ? 4 : 1;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + (j < 4 ? wm : 4) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-        if (m < m_end && n < a.N) {
-          const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
-          store_out(a.y, orow * a.N + n, j < 4 ? acc[j][r] : accx[r], a.y_dtype);
+      for (int j = 0; j < 4; ++j) {
+        if (j >= ncb) break;
+        const int n = n0 + ((i == 0 || two) ? j : wm) * 32 + li;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + (i == 0 ? wm : (two ? wm + 4 : 4)) * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          if (m < m_end && n < a.N) {
+            const int64_t orow = a.out_idx ? (int64_t)a.out_idx[m] : (int64_t)m;
+            store_out(a.y, orow * a.N + n, i == 0 ? acc[j][r] : acc2[j][r], a.y_dtype);
+          }
         }
       }
     }
@@ -420,7 +496,8 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
 template <int MODE, int BITS, bool G64, bool TLDS>
 void launch_k(const Gemm2Args& a, hipStream_t st) {
   const int64_t m_tiles = ceil_div(a.R, kTileRows) + a.E;      // provisioned: a tile never straddles an expert
-  const int64_t total = ceil_div(ceil_div(a.N, BN), 8) * 8 * m_tiles;
+  int64_t total = ceil_div(ceil_div(a.N, BN), 8) * 8 * m_tiles;
+  if (!a.row_offsets) total = ceil_div(ceil_div(a.N, BN) * ceil_div(a.R, kTileRows), 8) * 8;
   const size_t epi = (size_t)4 * 32 * BN * 2;
   const size_t need = (size_t)(kS * kStage) + (TLDS ? 2 * kTabKind : 0);
   const size_t lds = epi > need ? epi : need;
@@ -440,17 +517,18 @@ void launch_s(const Gemm2Args& a, hipStream_t st) {
 
 }  // namespace
 
-// Short row groups (a mean of at most 144 rows an expert) with 16-byte table
-// windows of bf16 (E8M0 for MXFP4) entries; everything else stays on the
-// general kernel.
+// Products whose tables can be fetched as 16-byte windows of bf16 (E8M0 for
+// MXFP4) entries and whose K is a multiple of four K-tiles; everything else
+// stays on the general kernel.
 bool gemm2s_wanted(const g2::Gemm2Args& a, int mode, int bits) {
   static const char* env = experiment_env("QMM_GEMM2S");   // "0": never, "1": whenever it can run
   if (env && env[0] == '0') return false;
-  const bool can = a.row_offsets && a.E > 0 && a.tabfast && a.K % 256 == 0 &&
+  const bool can = (a.row_offsets ? a.E > 0 : a.E == 1) && a.tabfast && a.K % 256 == 0 &&
                    (mode == QMM_MODE_MXFP4 || (a.tab == QMM_BF16 && (bits == 4 || bits == 8)));
   if (!can) return false;
   if (env && env[0] == '1') return true;
-  return a.R / a.E <= 144;
+  if (env && env[0] == '2') return a.row_offsets && a.R / a.E <= 144;    // the rule before full tiles
+  return true;
 }
 
 void gemm2s_launch(const g2::Gemm2Args& a, int mode, int bits, hipStream_t st) {

@@ -578,6 +578,35 @@ def test_c3_prefill_scaled_and_full_size_properties():
     assert torch.equal(y2, y * 2)
 
 
+@pytest.mark.parametrize("bits,gs,k", [(4, 64, 512), (8, 64, 1024), (4, 128, 768), (4, 32, 256)])
+def test_prefill_rows_around_the_borders_of_the_split_role_kernels_tiles(bits, gs, k):
+    """Dense products at M > 16 with bf16 tables and K % 256 == 0 run on the
+    split-role kernel as one expert of all rows: 256-row tiles dealt as
+    contiguous runs, the last tile with 1..256 rows (each of its three loops),
+    a ragged last column tile, both epilogues, a batch axis."""
+    rng = np.random.default_rng(400 + bits + gs + k)
+    n = 264
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+    for m in (17, 128, 129, 160, 161, 255, 256, 257, 256 + 140, 600):
+        x, xd = make_x(rng, m, k)
+        want = O.qmm(x, words, s, b, gs, bits, weight_rounding="bf16")
+        y32 = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32)
+        assert O.rel_l2(out_f32(y32), want) <= 2e-5, (m, O.rel_l2(out_f32(y32), want))
+        # every row by itself: a row block that went missing would hide in the total
+        err = np.abs(out_f32(y32) - want).max(axis=1) / np.abs(want).max()
+        assert err.max() <= 1e-4, (m, int(err.argmax()), err.max())
+        y16 = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits)
+        assert torch.equal(y16, y32.to(torch.bfloat16)), m
+    # two weights at once: the batch axis launches the kernel once per pair
+    _, words2, s2, b2, wd2, sd2, bd2 = make_affine(rng, n, k, bits, gs, lead=(2,))
+    x = O.round_bf16(rng.standard_normal((2, 300, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    y = out_f32(K.quantized_matmul(xd, wd2, sd2, bd2, group_size=gs, bits=bits, out_dtype=torch.float32))
+    for z in range(2):
+        want = O.qmm(x[z], words2[z], s2[z], b2[z], gs, bits, weight_rounding="bf16")
+        assert O.rel_l2(y[z], want) <= 2e-5, z
+
+
 # ----------------------------------------------------------- grouped / MoE ----
 
 def test_grouped_qmm_with_empty_and_ragged_experts():
@@ -620,18 +649,19 @@ def test_grouped_qmm_experts_around_one_row_block_past_half_a_tile(bits, tab):
 
 @pytest.mark.parametrize("bits,gs,k", [(4, 64, 512), (4, 32, 768), (4, 128, 256), (8, 64, 1024)])
 def test_grouped_qmm_short_experts_on_the_split_role_kernel(bits, gs, k):
-    """A mean of at most 144 rows an expert with bf16 tables and K % 256 == 0
-    runs the kernel whose wavefronts are split into dequantizing producers and
-    multiplying consumers: tiles of up to 160 rows (a fifth row block split by
-    columns), longer experts in several tiles, an empty expert, a last column
-    tile of 8 columns, both epilogues, and the gathered form's row scatter."""
+    """bf16 tables and K % 256 == 0 run the kernel whose wavefronts are split
+    into dequantizing producers and multiplying consumers.  Its tiles hold up
+    to 256 rows and pick their loop by the rows they hold: up to 128 (one row
+    block a consumer), up to 160 (a fifth row block split by columns), more
+    (two row blocks a consumer); longer experts in several tiles, an empty
+    expert, a last column tile of 8 columns, both epilogues, and the gathered
+    form's row scatter."""
     rng = np.random.default_rng(91 + bits + gs)
-    sizes = np.array([128, 129, 160, 161, 145, 97, 33, 0, 320, 1])
+    sizes = np.array([128, 129, 160, 161, 145, 97, 33, 0, 320, 1, 200, 257, 256])
     e, n = len(sizes), 264
     _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, lead=(e,))
     ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
     r = int(ro[-1])
-    assert r // e <= 144
     x, xd = make_x(rng, r, k)
     want = O.grouped_qmm(x, words, s, b, ro, gs, bits, weight_rounding="bf16")
     ro_d = torch.from_numpy(ro).to(DEV)
@@ -1136,7 +1166,7 @@ def test_grouped_qmm_short_experts_with_table_rows_longer_than_a_cache_line(bits
         b, bd = None, None
     ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
     r = int(ro[-1])
-    assert r // e <= 144 and k % 256 == 0
+    assert k % 256 == 0
     x, xd = make_x(rng, r, k)
     want = O.grouped_qmm(x, words, s, b, ro, gs, bits, mode, weight_rounding="bf16")
     ro_d = torch.from_numpy(ro).to(DEV)

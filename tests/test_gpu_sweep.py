@@ -112,10 +112,11 @@ def test_grouped_and_gathered_random_case(seed):
 
 @pytest.mark.parametrize("seed", range(10))
 def test_grouped_short_experts_random_case(seed):
-    """Grouped products that run on the split-role kernel (a mean of at most
-    144 rows an expert, bf16 tables, K % 256 == 0): many experts, empty ones,
-    experts past one 160-row tile, any N (also below one column tile and not a
-    multiple of 8), every output type."""
+    """Grouped products that run on the split-role kernel (bf16 tables,
+    K % 256 == 0): many experts, empty ones, experts on either side of the
+    borders between its three loops (128, 160 and 256 rows a tile) and past
+    one tile, any N (also below one column tile and not a multiple of 8),
+    every output type."""
     rng = np.random.default_rng(12000 + seed)
     e = int(rng.integers(1, 13))
     n = int(rng.choice([rng.integers(1, 128), rng.integers(128, 400)]))
@@ -124,8 +125,8 @@ def test_grouped_short_experts_random_case(seed):
     bits = int(rng.choice([4, 8]))
     sizes = rng.integers(0, 150, size=e)
     sizes[rng.integers(0, e)] += int(rng.choice([20, 120, 200]))
-    if sizes.sum() // e > 144:
-        sizes = sizes // 2 + 1
+    if seed % 2:
+        sizes[rng.integers(0, e)] += int(rng.choice([60, 110, 260]))
     ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
     r = int(ro[-1])
     codes = rng.integers(0, 1 << bits, size=(e, n, k), dtype=np.uint8)
