@@ -521,13 +521,12 @@ void launch_s(const Gemm2Args& a, hipStream_t st) {
 // MXFP4) entries and whose K is a multiple of four K-tiles; everything else
 // stays on the general kernel.
 bool gemm2s_wanted(const g2::Gemm2Args& a, int mode, int bits) {
-  static const char* env = experiment_env("QMM_GEMM2S");   // "0": never, "1": whenever it can run
+  static const char* env = experiment_env("QMM_GEMM2S");   // "0": never, "2": short experts only
   if (env && env[0] == '0') return false;
   const bool can = (a.row_offsets ? a.E > 0 : a.E == 1) && a.tabfast && a.K % 256 == 0 &&
                    (mode == QMM_MODE_MXFP4 || (a.tab == QMM_BF16 && (bits == 4 || bits == 8)));
   if (!can) return false;
-  if (env && env[0] == '1') return true;
-  if (env && env[0] == '2') return a.row_offsets && a.R / a.E <= 144;    // the rule before full tiles
+  if (env && env[0] == '2') return a.row_offsets && a.R / a.E <= 144;
   return true;
 }
 
