@@ -336,6 +336,7 @@ def main():
         out["other_shapes"].update({f"C{c}": bench_once(c, check=not args.no_cpu) for c in (3, 4, 5)})
         # the library's bf16 matmul on the same shapes (no dequantization)
         out["dense_bf16"] = {"C3 [2048,4096]x[4096,4096]": bench_dense_bf16(2048, 4096, 4096),
+                             "C4 [256,8192]x[8192,8192]": bench_dense_bf16(256, 8192, 8192),
                              "C5 8 x [128,4096]x[14336,4096]": bench_dense_bf16(128, 14336, 4096, experts=8)}
         # decode shapes outside the named configurations (random codes, timing only)
         out["other_decode_shapes"] = {
