@@ -103,6 +103,62 @@ __device__ __forceinline__ uint32_t byte_perm(uint32_t hi, uint32_t lo, uint32_t
 
 __host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// ---- the row tiles of a grouped product --------------------------------------
+// Rows [offsets[e], offsets[e+1]) belong to expert e and are cut into tiles of
+// `tile_rows` that never straddle two experts.  Which expert and which of its
+// tiles is row tile `tile_m` of the whole product?  The wavefront looks at 64
+// experts at a time, one a lane (two coalesced loads, a prefix sum over the
+// lanes and a ballot), so that the search costs a few memory round trips
+// whatever the number of experts -- walked one expert after the other it cost
+// one round trip an expert in every workgroup's prologue.  Offsets are forced
+// into [0, R] and non-decreasing whatever the array holds.  Every lane of the
+// wavefront must be active; the results are the same in all of them.
+struct RowTile {
+  int e, lo, hi, idx;    // expert, its rows [lo, hi), the tile's number inside the expert
+  int m_tiles;           // row tiles of the whole product
+  bool found;            // false: tile_m is past the last tile
+};
+
+__device__ __forceinline__ RowTile find_row_tile(const int32_t* offsets, int E, int R, int tile_rows, int tile_m) {
+  RowTile r{0, 0, 0, 0, 0, false};
+  const int lane = (int)(threadIdx.x & 63);
+  int base = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int i = e0 + lane;
+    int lo = 0, hi = 0;
+    if (i < E) {
+      lo = offsets[i];
+      hi = offsets[i + 1];
+      lo = lo < 0 ? 0 : (lo > R ? R : lo);
+      hi = hi < lo ? lo : (hi > R ? R : hi);
+    }
+    const int tiles = (hi - lo + tile_rows - 1) / tile_rows;
+    int incl = tiles;                               // tiles of experts e0 .. e0 + lane
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int v = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += v;
+    }
+    const int total = __shfl(incl, 63, 64);
+    if (!r.found && tile_m >= base && tile_m < base + total) {
+      const unsigned long long past = __ballot(base + incl > tile_m);    // lanes at or after the tile's expert
+      const int L = __ffsll((long long)past) - 1;
+      r.e = e0 + L;
+      r.lo = __shfl(lo, L, 64);
+      r.hi = __shfl(hi, L, 64);
+      r.idx = tile_m - base - __shfl(incl - tiles, L, 64);
+      r.found = true;
+    }
+    base += total;
+  }
+  r.e = __builtin_amdgcn_readfirstlane(r.e);
+  r.lo = __builtin_amdgcn_readfirstlane(r.lo);
+  r.hi = __builtin_amdgcn_readfirstlane(r.hi);
+  r.idx = __builtin_amdgcn_readfirstlane(r.idx);
+  r.m_tiles = __builtin_amdgcn_readfirstlane(base);
+  return r;
+}
+
 // ---- host-side helpers ------------------------------------------------------
 
 // Experiment switches (kernel overrides used while measuring).  The shipped

@@ -121,19 +121,14 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
   // workgroups in flight on one XCD still share an expert's rows.
   const int n_tiles = (a.N + BN - 1) / BN;
   int tile_n, tile_m;
+  int e = 0, row_lo = 0, row_hi = a.R, mt_idx = 0;
   if (a.row_offsets) {
-    // the grid is provisioned for the worst raggedness: count the row tiles that exist
-    int m_tiles = 0;
-    for (int i = 0; i < a.E; ++i) {
-      int lo, hi;
-      group_rows(a, i, lo, hi);
-      m_tiles += (hi - lo + BM - 1) / BM;
-    }
-    const int band = (n_tiles + 7) / 8;
-    const int l = blockIdx.x >> 3;
-    tile_m = l / band;
-    tile_n = (blockIdx.x & 7) * band + l % band;
-    if (tile_m >= m_tiles || tile_n >= n_tiles) return;
+    // the grid is provisioned for the worst raggedness: only the row tiles that exist are dealt
+    deal_grouped_tile(n_tiles, blockIdx.x & 7, blockIdx.x >> 3, tile_m, tile_n);
+    if (tile_n >= n_tiles) return;
+    const RowTile rt = find_row_tile(a.row_offsets, a.E, a.R, BM, tile_m);
+    if (!rt.found) return;
+    e = rt.e; row_lo = rt.lo; row_hi = rt.hi; mt_idx = rt.idx;
   } else {
     const int total = n_tiles * a.m_tiles;
     const int per = (total + 7) / 8;
@@ -141,19 +136,7 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm2_kernel(Gemm2Args a) {
     if (tile >= total) return;
     tile_n = tile % n_tiles;
     tile_m = tile / n_tiles;
-  }
-  int e = 0, row_lo = 0, row_hi = a.R, mt_idx = tile_m;
-  if (a.row_offsets) {
-    int t = tile_m;
-    bool found = false;
-    for (int i = 0; i < a.E; ++i) {
-      int lo, hi;
-      group_rows(a, i, lo, hi);
-      const int tiles = (hi - lo + BM - 1) / BM;
-      if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
-      t -= tiles;
-    }
-    if (!found) return;
+    mt_idx = tile_m;
   }
   const int m0 = row_lo + mt_idx * BM;
   if (m0 >= row_hi) return;

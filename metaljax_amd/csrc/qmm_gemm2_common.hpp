@@ -46,12 +46,23 @@ struct Gemm2Args {
   int tabfast;           // table rows are dword-aligned: fetch them as 16-byte windows
 };
 
-// Rows [lo, hi) of expert i, forced into [0, R] and hi >= lo whatever the offsets hold.
-__device__ __forceinline__ void group_rows(const Gemm2Args& a, int i, int& lo, int& hi) {
-  lo = a.row_offsets[i];
-  hi = a.row_offsets[i + 1];
-  lo = lo < 0 ? 0 : (lo > a.R ? a.R : lo);
-  hi = hi < lo ? lo : (hi > a.R ? a.R : hi);
+// How the tiles of a grouped product are dealt to the eight XCDs (workgroup
+// b runs on XCD b % 8; l = b / 8 counts an XCD's workgroups).  A band of
+// column tiles of every row tile per XCD keeps the row tiles of one expert
+// and column on one L2 -- but with few column tiles the bands are uneven (11
+// column tiles: five XCDs get two columns, one gets one, two get none), so
+// when more than a sixteenth of the band slots would be empty the tiles go
+// round the XCDs one by one instead, row tile after row tile.
+__device__ __forceinline__ void deal_grouped_tile(int n_tiles, int xcd, int l, int& tile_m, int& tile_n) {
+  const int band = (n_tiles + 7) / 8;
+  if ((band * 8 - n_tiles) * 16 > n_tiles) {
+    const int g = l * 8 + xcd;
+    tile_m = g / n_tiles;
+    tile_n = g % n_tiles;
+  } else {
+    tile_m = l / band;
+    tile_n = xcd * band + l % band;       // may be past the last column tile: the caller checks
+  }
 }
 
 // 32 codes (one row, one 32-group) -> four 16-byte pieces of bf16 weights

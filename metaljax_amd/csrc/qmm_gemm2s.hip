@@ -45,15 +45,6 @@ constexpr int kS = 3;                 // LDS stages: K-tile t lives in stage t %
 constexpr int kTileRows = 256;        // eight row blocks, two a consumer
 constexpr int kAR = 3;                // activation fragments: K-tile t lives in ring slot t % 3 (t % 2 on full tiles)
 
-// Rows [lo, hi) of expert i; a product without row offsets is one expert of all rows.
-__device__ __forceinline__ void expert_rows(const Gemm2Args& a, int i, int& lo, int& hi) {
-  if (a.row_offsets) {
-    group_rows(a, i, lo, hi);
-  } else {
-    lo = 0;
-    hi = a.R;
-  }
-}
 // Table rows staged in LDS (a row's scales / biases of the whole K when they
 // fit 128 bytes): 128 + 16 bytes a row, so that eight rows fall on different banks.
 constexpr int kTabRow = 144;
@@ -72,42 +63,30 @@ __global__ __launch_bounds__(512) void gemm2s_kernel(Gemm2Args a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  // ---- which tile?  XCD x gets a band of column tiles of every expert,
-  // expert after expert; the grid is provisioned for the worst raggedness and
-  // only the row tiles that exist are dealt.
+  // ---- which tile?  The grid is provisioned for the worst raggedness and
+  // only the row tiles that exist are dealt (deal_grouped_tile: a band of
+  // column tiles of every expert per XCD, expert after expert, or one by one
+  // round the XCDs when the bands would be uneven).
   const int n_tiles = (a.N + BN - 1) / BN;
-  int m_tiles = 0;
-  for (int i = 0; i < a.E; ++i) {
-    int lo, hi;
-    expert_rows(a, i, lo, hi);
-    m_tiles += (hi - lo + kTileRows - 1) / kTileRows;
-  }
-  const int band = (n_tiles + 7) / 8;
   const int xcd = blockIdx.x & 7, l = blockIdx.x >> 3;
-  int tile_m = l / band;
-  int tile_n = xcd * band + l % band;
+  int tile_m, tile_n;
+  deal_grouped_tile(n_tiles, xcd, l, tile_m, tile_n);
+  int e = 0, row_lo = 0, row_hi = a.R, mt_idx = 0;
   if (!a.row_offsets) {
     // one expert of all rows: an eighth of the grid takes a contiguous run of
     // tiles, column tile fastest, so its workgroups share few activation rows
+    const int m_tiles = (a.R + kTileRows - 1) / kTileRows;
     const int total = n_tiles * m_tiles, per = (total + 7) / 8;
     const int t = xcd * per + l;
     if (l >= per || t >= total) return;
     tile_m = t / n_tiles;
     tile_n = t % n_tiles;
-  }
-  if (tile_m >= m_tiles || tile_n >= n_tiles) return;
-  int e = 0, row_lo = 0, row_hi = 0, mt_idx = 0;
-  {
-    int t = tile_m;
-    bool found = false;
-    for (int i = 0; i < a.E; ++i) {
-      int lo, hi;
-      expert_rows(a, i, lo, hi);
-      const int tiles = (hi - lo + kTileRows - 1) / kTileRows;
-      if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt_idx = t; found = true; break; }
-      t -= tiles;
-    }
-    if (!found) return;
+    mt_idx = tile_m;
+  } else {
+    if (tile_n >= n_tiles) return;
+    const RowTile rt = find_row_tile(a.row_offsets, a.E, a.R, kTileRows, tile_m);
+    if (!rt.found) return;
+    e = rt.e; row_lo = rt.lo; row_hi = rt.hi; mt_idx = rt.idx;
   }
   const int m0 = row_lo + mt_idx * kTileRows;
   if (m0 >= row_hi) return;

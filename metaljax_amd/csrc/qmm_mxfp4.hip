@@ -164,14 +164,6 @@ struct MxArgs {
   int m_tiles, n_tiles;  // provisioned row tiles (>= the tiles that exist when grouped)
 };
 
-// Rows [lo, hi) of expert i, forced into [0, R] and hi >= lo whatever the offsets hold.
-__device__ __forceinline__ void mx_group_rows(const MxArgs& a, int i, int& lo, int& hi) {
-  lo = a.row_offsets[i];
-  hi = a.row_offsets[i + 1];
-  lo = lo < 0 ? 0 : (lo > a.R ? a.R : lo);
-  hi = hi < lo ? lo : (hi > a.R ? a.R : hi);
-}
-
 // The two FP6 terms of a lane's 48 bytes (three 16-byte planes, hi | lo).
 __device__ __forceinline__ i32x8 fp6_term(const u32x4 (&p)[3], int term) {
   if (term == 0) return i32x8{(int)p[0][0], (int)p[0][1], (int)p[0][2], (int)p[0][3], (int)p[1][0], (int)p[1][1], 0, 0};
@@ -195,14 +187,8 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   // that exist are counted first and only those are dealt; a tile never
   // straddles two experts.
   int m_tiles = a.m_tiles;
-  if (a.row_offsets) {
-    m_tiles = 0;
-    for (int i = 0; i < a.E; ++i) {
-      int lo, hi;
-      mx_group_rows(a, i, lo, hi);
-      m_tiles += (hi - lo + TM - 1) / TM;
-    }
-  }
+  if (a.row_offsets) m_tiles = find_row_tile(a.row_offsets, a.E, a.R, TM, -1).m_tiles;   // counted only
+  if (m_tiles == 0) return;
   const int total = m_tiles * a.n_tiles;
   const int per = (total + 7) / 8;
   const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
@@ -210,16 +196,9 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   int e = 0, row_hi = a.R, m0 = (tile % m_tiles) * TM;
   const int n0 = (tile / m_tiles) * TN;
   if (a.row_offsets) {
-    int t = tile % m_tiles;
-    bool found = false;
-    for (int i = 0; i < a.E; ++i) {
-      int lo, hi;
-      mx_group_rows(a, i, lo, hi);
-      const int tiles = (hi - lo + TM - 1) / TM;
-      if (t < tiles) { e = i; m0 = lo + t * TM; row_hi = hi; found = true; break; }
-      t -= tiles;
-    }
-    if (!found) return;
+    const RowTile rt = find_row_tile(a.row_offsets, a.E, a.R, TM, tile % m_tiles);
+    if (!rt.found) return;
+    e = rt.e; m0 = rt.lo + rt.idx * TM; row_hi = rt.hi;
   }
 
   const int nquads = a.K / 512;

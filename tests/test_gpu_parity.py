@@ -835,6 +835,43 @@ def test_grouped_and_gathered_mxfp4_experts(k):
     assert O.rel_l2(yg, want[perm]) <= tol, O.rel_l2(yg, want[perm])
 
 
+@pytest.mark.parametrize("kind", ["bf16 tables", "f32 tables", "mxfp4"])
+def test_grouped_qmm_over_many_experts(kind):
+    """More experts than a wavefront has lanes (the kernels find a tile's
+    expert 64 experts at a time): 150 experts, most with a few rows, some
+    empty, some longer than one row tile of any kernel, the last one not
+    empty; each of the three grouped prefill kernels; the gathered form."""
+    rng = np.random.default_rng(len(kind))
+    e, n, k = 150, 136, 512
+    sizes = rng.integers(0, 6, size=e)
+    sizes[rng.choice(e, size=20, replace=False)] = 0
+    sizes[[3, 70, 149]] = [300, 170, 7]
+    ro = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    r = int(ro[-1])
+    x, xd = make_x(rng, r, k)
+    ro_d = torch.from_numpy(ro).to(DEV)
+    if kind == "mxfp4":
+        _, words, s, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+        b, bd, gs, mode, rounding, tol = None, None, 32, "mxfp4", "f32", TOL_F32_OUT
+    else:
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, "bf16" if kind == "bf16 tables" else "f32",
+                                                 lead=(e,))
+        gs, mode, rounding, tol = 64, "affine", "bf16", 2e-5
+    want = O.grouped_qmm(x, words, s, b, ro, gs, 4, mode, weight_rounding=rounding)
+    y = out_f32(K.grouped_qmm(xd, wd, sd, bd, ro_d, group_size=gs, bits=4, mode=mode, out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= tol, O.rel_l2(y, want)
+    for i in range(e):                       # every expert's rows by themselves
+        lo, hi = ro[i], ro[i + 1]
+        if hi > lo:
+            assert O.rel_l2(y[lo:hi], want[lo:hi]) <= 10 * tol, (i, O.rel_l2(y[lo:hi], want[lo:hi]))
+    rhs = np.repeat(np.arange(e), sizes).astype(np.int32)
+    perm = rng.permutation(r)
+    yg = out_f32(K.gather_qmm(xd, wd, sd, bd, torch.from_numpy(perm.astype(np.int32)).to(DEV),
+                              torch.from_numpy(rhs[perm]).to(DEV), group_size=gs, bits=4, mode=mode,
+                              out_dtype=torch.float32))
+    assert O.rel_l2(yg, want[perm]) <= tol, O.rel_l2(yg, want[perm])
+
+
 def test_c5_moe_scaled():
     wl = synth.make(5, scale=1 / 56)                  # N = 256, 18 tokens... of the same draw
     x, w, s, b, ro = synth.to_device(wl)
