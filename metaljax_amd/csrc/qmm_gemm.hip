@@ -130,15 +130,9 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs a) {
   // ---- which (expert, row tile)?
   int e = 0, row_lo = 0, row_hi = a.R, mt = tile_m;
   if (a.row_offsets) {
-    int t = tile_m;
-    bool found = false;
-    for (int i = 0; i < a.E; ++i) {
-      const int lo = a.row_offsets[i], hi = a.row_offsets[i + 1];
-      const int tiles = (hi - lo + BM - 1) / BM;
-      if (t < tiles) { e = i; row_lo = lo; row_hi = hi; mt = t; found = true; break; }
-      t -= tiles;
-    }
-    if (!found) return;
+    const RowTile rt = find_row_tile(a.row_offsets, a.E, a.R, BM, tile_m);
+    if (!rt.found) return;
+    e = rt.e; row_lo = rt.lo; row_hi = rt.hi; mt = rt.idx;
   }
   const int m0 = row_lo + mt * BM;
   if (m0 >= row_hi) return;
