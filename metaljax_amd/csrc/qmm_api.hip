@@ -28,6 +28,11 @@ void gemm_dispatch(const void* x, const void* w, const void* s, const void* b, i
                    const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
                    int64_t K, int gs, int bits, int mode, hipStream_t st);
 int64_t gemm_row_tile(int64_t R, int64_t E);
+bool gemv_runs_general(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* s, const void* b);
+void gemv_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                           int y_dtype, const int32_t* segments, const int32_t* src_row,
+                           const int32_t* out_row, int64_t max_segments, int64_t x_rows, int64_t N,
+                           int64_t K, int gs, int bits, int mode, hipStream_t st);
 bool gemm2_supported(int64_t R, int64_t N, int64_t K);
 size_t gemm2_workspace_bytes(int64_t R, int64_t K);
 void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
@@ -481,6 +486,32 @@ static int gather_bf16(const void* x, int x_dtype, const void* w, const void* sc
     return check_launch("grouped decode launch");
   }
   if (P <= kGatherGemvMaxPairs) {
+    // From sixteen pairs on, and half a pair an expert, shapes that only the
+    // general decode kernels serve are grouped by expert as well: an expert's
+    // weights are then read once for up to sixteen of its pairs instead of
+    // once per pair.  (The sort costs a launch of its own, and with fewer
+    // pairs than that few of them share an expert.  Measured on 32 MXFP4
+    // experts of [5760, 2880]: 16 pairs 61 against 60 us, 32 pairs 86 against
+    // 110, 64 pairs 109 against 216; on 128 experts: 32 pairs 128 against 110,
+    // 64 pairs 194 against 217; 8 experts of [4096, 11008] with four-bit
+    // codes: 16 pairs 108 against 206 us, 32 pairs 110 against 397.)
+    if (P >= 16 && 2 * P >= E && grouped_decode_pairs(P, E) && workspace &&
+        workspace_bytes >= route_bytes_segments(P, E) &&
+        gemv_runs_general(N, K, group_size, bits, mode, table_dtype, scales, biases) &&
+        !experiment_env("QMM_NO_GROUPED_GEMV")) {
+      int32_t* ro = static_cast<int32_t*>(workspace);
+      int32_t* cursor = ro + E + 1;
+      int32_t* src_row = cursor + E;
+      int32_t* out_row = src_row + P;
+      int32_t* segments = out_row + P;
+      hipLaunchKernelGGL(route_kernel, dim3(1), dim3(1024), 0, st, lhs_idx, rhs_idx, (int)P, (int)E,
+                         ro, cursor, src_row, out_row, segments);
+      rc = check_launch("route launch");
+      if (rc) return rc;
+      gemv_grouped_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, segments, src_row, out_row,
+                            skinny2_max_segments(P, E), T, N, K, group_size, bits, mode, st);
+      return check_launch("grouped gemv launch");
+    }
     gemv_dispatch(x, w, scales, biases, table_dtype, y, y_dtype, P, 1, N, K, group_size, bits,
                   mode, lhs_idx, rhs_idx, E, T, st);
     return check_launch("gather gemv launch");

@@ -66,13 +66,21 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
   const int64_t ng = (int64_t)((a.K / CH) >> a.gshift);     // table entries per row
 
   int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
-  const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
   bool x_ok = true;
-  if (a.rhs_idx) {                                  // gather form: indices are data
+  int M = a.M, seg_lo = 0;
+  if (a.segments) {                                 // grouped form: up to 16 sorted pairs of one expert
+    if (bz >= a.segments[0]) return;                // uniform, before any barrier
+    wz = a.segments[1 + 3 * bz];
+    seg_lo = a.segments[2 + 3 * bz];
+    M = a.segments[3 + 3 * bz];
+    xz = 0;
+  } else if (a.rhs_idx) {                           // gather form: indices are data
     if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
     if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
   }
-  const auto rx = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? (int64_t)a.M * a.K * 2 : 0);
+  const auto rx = a.segments ? make_rsrc(a.x, (int64_t)a.x_rows * a.K * 2)
+                             : make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? (int64_t)a.M * a.K * 2 : 0);
   const auto rw = make_rsrc(a.w + wz * a.N * wpr, a.N * wpr * 4);
   const auto rs = make_rsrc(static_cast<const char*>(a.s) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
   const auto rb = make_rsrc(static_cast<const char*>(a.b) + wz * a.N * ng * TABSZ, a.N * ng * TABSZ);
@@ -89,7 +97,11 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
     woff[t] = (uint32_t)((n * wpr + kg * WPL) * 4);
     toff[t] = (uint32_t)(n * ng * TABSZ);
   }
-  const uint32_t xoff = r < a.M ? (uint32_t)(((int64_t)r * a.K + kg * (CH / 4)) * 2) : kOutOfRange;
+  uint32_t xoff = r < M ? (uint32_t)(((int64_t)r * a.K + kg * (CH / 4)) * 2) : kOutOfRange;
+  if (a.segments && r < M) {                        // row r of the segment is row src_row[first + r] of x
+    const int64_t src = a.src_row[seg_lo + r];
+    xoff = src >= 0 && src < a.x_rows ? (uint32_t)((src * a.K + kg * (CH / 4)) * 2) : kOutOfRange;
+  }
 
   f32x4 acc[T];
 #pragma unroll
@@ -212,7 +224,11 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_affine_kernel(GemvArgs a) {
     for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][i][l];
     const int m = 4 * (l >> 4) + i;
     const int64_t n = n0 + t * 16 + (l & 15);
-    if (m < a.M && n < a.N) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+    if (m < M && n < a.N) {
+      int64_t orow = bz * a.M + m;
+      if (a.segments) orow = a.out_row[seg_lo + m];
+      if (orow >= 0) store_out(a.y, orow * (int64_t)a.N + n, v, a.y_dtype);
+    }
   }
 }
 
@@ -235,9 +251,16 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
   const int nblk = a.K / 32;                       // MX blocks per row
 
   int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
-  const int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
+  int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
   bool x_ok = true;
-  if (a.rhs_idx) {                                  // gather form: indices are data
+  int M = a.M, seg_lo = 0;
+  if (a.segments) {                                 // grouped form: up to 16 sorted pairs of one expert
+    if (bz >= a.segments[0]) return;                // uniform, before any barrier
+    wz = a.segments[1 + 3 * bz];
+    seg_lo = a.segments[2 + 3 * bz];
+    M = a.segments[3 + 3 * bz];
+    xz = 0;
+  } else if (a.rhs_idx) {                           // gather form: indices are data
     if (wz < 0 || wz >= a.n_experts) return;        // uniform, before any barrier
     if (xz < 0 || xz >= a.n_xrows) { xz = 0; x_ok = false; }
   }
@@ -258,8 +281,13 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
     wrow[t] = wb + n * wpr;
     srow[t] = sb + n * nblk;
   }
-  const bool xvalid = r < a.M && x_ok;
+  bool xvalid = r < M && x_ok;
   const uint16_t* xrow = xb + (int64_t)(xvalid ? r : 0) * a.K;
+  if (a.segments) {                                 // row r of the segment is row src_row[first + r] of x
+    const int64_t src = r < M ? (int64_t)a.src_row[seg_lo + r] : -1;
+    xvalid = src >= 0 && src < a.x_rows;
+    xrow = a.x + (xvalid ? src : 0) * a.K;
+  }
 
   f32x4 acc[T];
 #pragma unroll
@@ -321,7 +349,11 @@ __global__ __launch_bounds__(kWave* WAVES) void gemv_mxfp4_kernel(GemvArgs a) {
     for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][i][l];
     const int m = 4 * (l >> 4) + i;
     const int64_t n = n0 + t * 16 + (l & 15);
-    if (m < a.M && n < a.N) store_out(a.y, (bz * a.M + m) * (int64_t)a.N + n, v, a.y_dtype);
+    if (m < M && n < a.N) {
+      int64_t orow = bz * a.M + m;
+      if (a.segments) orow = a.out_row[seg_lo + m];
+      if (orow >= 0) store_out(a.y, orow * (int64_t)a.N + n, v, a.y_dtype);
+    }
   }
 }
 
@@ -469,6 +501,61 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
   } else {
     if (ch == 64) launch_affine<8, 64>(a, batch, tab, g, st);
     else launch_affine<8, 32>(a, batch, tab, g, st);
+  }
+}
+
+// The general kernels would serve this shape (no staged decode kernel does).
+bool gemv_runs_general(int64_t N, int64_t K, int gs, int bits, int mode, int tab, const void* s, const void* b) {
+  if (skinny_supported(N, K, gs, bits, mode, tab, s, b)) return false;
+  if ((tab == QMM_F16 || tab == QMM_F32) && K * bits / 8 / 256 >= 8 &&
+      skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b))
+    return false;
+  if (mode == QMM_MODE_MXFP4 && skinny2_mx_supported(N, K, s)) return false;
+  return true;
+}
+
+// Expert-indexed pairs sorted by expert (segments / src_row / out_row as the
+// routing pass writes them) on the general kernels: one decode product per
+// expert and sixteen pairs, so that an expert's weights are read once for all
+// of its pairs instead of once per pair.  `max_segments` rows of workgroups
+// are launched; the ones past the list's count exit at once.
+void gemv_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, int tab, void* y,
+                           int y_dtype, const int32_t* segments, const int32_t* src_row,
+                           const int32_t* out_row, int64_t max_segments, int64_t x_rows, int64_t N,
+                           int64_t K, int gs, int bits, int mode, hipStream_t st) {
+  GemvArgs a;
+  a.x = static_cast<const uint16_t*>(x);
+  a.w = static_cast<const uint32_t*>(w);
+  a.s = s;
+  a.b = b;
+  a.y = y;
+  a.M = 16;
+  a.N = (int)N;
+  a.K = (int)K;
+  a.y_dtype = y_dtype;
+  a.lhs_idx = nullptr;
+  a.rhs_idx = nullptr;
+  a.segments = segments;
+  a.src_row = src_row;
+  a.out_row = out_row;
+  a.x_rows = (int)x_rows;
+  Geometry g;
+  gemv_geometry(16, N, K, &g.t, &g.waves);
+  if (mode == QMM_MODE_MXFP4) {
+    a.gshift = 0;
+    g.u = 4;
+    launch_mxfp4(a, max_segments, g, st);
+    return;
+  }
+  g.u = 8;
+  const int ch = gs >= 64 ? 64 : 32;
+  a.gshift = (gs == 128) ? 1 : 0;
+  if (bits == 4) {
+    if (ch == 64) launch_affine<4, 64>(a, max_segments, tab, g, st);
+    else launch_affine<4, 32>(a, max_segments, tab, g, st);
+  } else {
+    if (ch == 64) launch_affine<8, 64>(a, max_segments, tab, g, st);
+    else launch_affine<8, 32>(a, max_segments, tab, g, st);
   }
 }
 

@@ -1013,6 +1013,58 @@ def test_gather_qmm_few_pairs_grouped_by_expert_float32_tables(gs):
     assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
 
 
+@pytest.mark.parametrize("kind,bits,gs,tab,t,pairs,e,n,k,skew", [
+    ("mxfp4", 4, 32, "bf16", 16, 64, 8, 700, 2880, False),      # the gpt-oss width: 5.6 slices, 90 scale bytes a row
+    ("mxfp4", 4, 32, "bf16", 9, 40, 3, 300, 1120, True),        # most pairs on one expert: several chunks of sixteen
+    ("affine", 4, 64, "bf16", 12, 48, 5, 520, 1088, False),     # K not a whole number of 256-byte slices
+    ("affine", 8, 32, "f16", 7, 16, 6, 200, 736, False),        # sixteen pairs: the smallest grouped launch
+    ("affine", 4, 128, "f32", 20, 64, 4, 333, 2176, True),
+])
+def test_gather_qmm_few_pairs_on_the_general_decode_kernels(kind, bits, gs, tab, t, pairs, e, n, k, skew):
+    """Sixteen to 64 pairs on shapes that no staged decode kernel serves: the
+    pairs are sorted by expert and the general decode kernels multiply up to
+    sixteen rows of one expert at a time; a pair naming no expert keeps its
+    output row, a pair naming a row outside x multiplies zeros."""
+    from metaljax_amd import _lib
+    rng = np.random.default_rng(pairs * 7 + k)
+    if kind == "mxfp4":
+        _, words, s, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+        b, bd = None, None
+    else:
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs, tab, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    lhs = rng.integers(0, t, size=pairs).astype(np.int32)
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    if skew:
+        rhs[rng.random(pairs) < 0.8] = e - 1
+    lhs[3], rhs[5], rhs[11] = t + 2, e, -1                 # a row outside x, two pairs naming no expert
+    lib = _lib.load()
+    nbytes = int(lib.qmm_gather_workspace_bytes(pairs, e, n, k, _lib.BF16))
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    ld, rd = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    tabd = {"bf16": _lib.BF16, "f16": _lib.F16, "f32": _lib.F32}[tab]
+    for yd, ydt in ((_lib.F32, torch.float32), (_lib.BF16, torch.bfloat16)):
+        y = torch.full((pairs, n), 7.0, dtype=ydt, device=DEV)
+        rc = lib.qmm_gather_qmm(xd.data_ptr(), _lib.BF16, wd.data_ptr(), sd.data_ptr(),
+                                None if bd is None else bd.data_ptr(), tabd, y.data_ptr(), yd,
+                                ld.data_ptr(), rd.data_ptr(), pairs, t, e, n, k, gs, bits,
+                                1 if kind == "mxfp4" else 0, ws.data_ptr(), nbytes,
+                                torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc)
+        got = out_f32(y)
+        tol = 2e-5 if yd == _lib.F32 else TOL_BF16_OUT
+        for i in range(pairs):
+            if not 0 <= rhs[i] < e:
+                np.testing.assert_array_equal(got[i], np.full(n, 7.0, np.float32))
+            elif not 0 <= lhs[i] < t:
+                np.testing.assert_array_equal(got[i], np.zeros(n, np.float32))
+            else:
+                want = O.qmm(x[lhs[i]][None], words[rhs[i]], s[rhs[i]], None if b is None else b[rhs[i]],
+                             gs, bits, kind)[0]
+                assert O.rel_l2(got[i], want) <= tol, (i, O.rel_l2(got[i], want))
+
+
 def test_gather_qmm_few_pairs_invalid_indices_touch_nothing():
     """Grouped decode: a pair naming no expert keeps its output row as it was,
     a pair naming a row outside x multiplies zeros."""
