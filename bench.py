@@ -345,6 +345,7 @@ def main():
             "int4 g64 f16 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f16"),
             "int4 g64 f32 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f32"),
             "int8 g64 [14336,4096] M=4": bench_decode_random(4, 14336, 4096, bits=8),
+            "int4 g64 [37888,3584] M=4": bench_decode_random(4, 37888, 3584),
             "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
         }
     if not args.no_cpu:

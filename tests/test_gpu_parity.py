@@ -607,6 +607,37 @@ def test_prefill_rows_around_the_borders_of_the_split_role_kernels_tiles(bits, g
         assert O.rel_l2(y[z], want) <= 2e-5, z
 
 
+@pytest.mark.parametrize("bits,gs,k", [(4, 64, 3584), (4, 64, 3072), (4, 128, 2560), (4, 64, 2048), (8, 64, 1536),
+                                       (8, 128, 1024)])
+def test_decode_with_four_to_seven_k_slices_a_row(bits, gs, k):
+    """K between four and seven 256-byte slices a row (hidden sizes 2048 to
+    3584 with four-bit codes) runs the one-pass loader-wavefront kernel with
+    some compute wavefronts idle: every row count's way of fetching the
+    activations (direct, whole lines, staged), small and large N (one tile a
+    workgroup up to several, and above 64 rows a workgroup also at M > 8), a
+    ragged last tile, float16 tables, both outputs, a batch axis."""
+    rng = np.random.default_rng(bits * 100 + k)
+    for n, ms in ((200, (1, 3, 8, 16)), (5000, (2, 5, 12)), (20011, (1, 4, 7, 9, 16))):
+        _, words, s, b, wd, sd, bd = make_affine(rng, n, k, bits, gs)
+        for m in ms:
+            x, xd = make_x(rng, m, k)
+            want = O.qmm(x, words, s, b, gs, bits)
+            y32 = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits, out_dtype=torch.float32)
+            assert O.rel_l2(out_f32(y32), want) <= 2e-5, (n, m, O.rel_l2(out_f32(y32), want))
+            err = np.abs(out_f32(y32) - want).max(axis=0) / np.abs(want).max()      # every output column
+            assert err.max() <= 1e-4, (n, m, int(err.argmax()), err.max())
+            y16 = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits)
+            assert torch.equal(y16, y32.to(torch.bfloat16)), (n, m)
+    # float16 tables and a batch of two weights
+    _, words, s, b, wd, sd, bd = make_affine(rng, 3000, k, bits, gs, "f16", lead=(2,))
+    x = O.round_bf16(rng.standard_normal((2, 6, k)).astype(np.float32))
+    y = out_f32(K.quantized_matmul(bf16_dev(O.f32_to_bf16_bits(x)), wd, sd, bd, group_size=gs, bits=bits,
+                                   out_dtype=torch.float32))
+    for z in range(2):
+        want = O.qmm(x[z], words[z], s[z], b[z], gs, bits)
+        assert O.rel_l2(y[z], want) <= 2e-5, z
+
+
 # ----------------------------------------------------------- grouped / MoE ----
 
 def test_grouped_qmm_with_empty_and_ragged_experts():
