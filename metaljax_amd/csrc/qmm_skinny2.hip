@@ -1031,8 +1031,9 @@ bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   // compute unit: with one pass over K the direct variant stages the
   // activations through LDS patches (whole-line loads) and is ahead of the
   // ring (4096 x 14336 at M = 16: 12.1 against 12.9 us a launch, 4096 x 4096:
-  // 6.5 against 7.6); with several passes the ring variant stays.
-  if (M > 8 && per <= 64 && K * bits / 8 / 256 != 8) return false;
+  // 6.5 against 7.6; fewer than eight slices: 9216 x 3072 8.6 against 12.2 on
+  // the self-loading kernel); with several passes the ring variant stays.
+  if (M > 8 && per <= 64 && K * bits / 8 / 256 > 8) return false;
   // Several passes over K: the next pass's activations are fetched when the
   // pass begins, which costs about 0.8 us a pass; measured against the other
   // kernels at M = 4 (us): 28672 x 8192 30.8 / 38.4, 57344 x 8192 61 / 79,
@@ -1040,7 +1041,7 @@ bool direct_x(int64_t M, int64_t N, int64_t K, int bits) {
   // 4096 25.2 / 30.8, but 8192 x 8192 14.2 / 12.9 and 4096 x 14336 15.3 / 12.3:
   // it pays from three tiles a workgroup on.
   const int64_t slices = K * bits / 8 / 256;
-  if (slices != 8) {
+  if (slices > 8) {
     // ... unless the kernel can pack every pass's activations into the sixteen
     // operand rows at once (passes x M <= 16), which takes the fetches away
     const int64_t passes = ceil_div(slices, (int64_t)8);

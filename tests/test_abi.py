@@ -86,8 +86,8 @@ def test_plan_of_the_decode_variants(lib):
     assert k.value == _lib.KERNEL_GEMV and b.value < 768
     assert lib.qmm_plan(4, 16384, 3072, 64, 4, 0, k, g, b) == 0         # six slices: loader wavefronts again
     assert k.value == _lib.KERNEL_GEMV and b.value == 768
-    assert lib.qmm_plan(16, 3072, 3072, 64, 4, 0, k, g, b) == 0         # ... but not sixteen rows on a small weight
-    assert b.value < 768
+    assert lib.qmm_plan(16, 3072, 3072, 64, 4, 0, k, g, b) == 0         # ... at sixteen rows too
+    assert b.value == 768
 
 
 def test_gather_workspace_covers_the_grouped_decode(lib):
