@@ -1064,15 +1064,17 @@ bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg) {
   int waves, rows;
   skinny_geometry(N, K, bits, &waves, &rows);
   if (waves != 8) {
-    // Four to seven K-slices a row (K = 2048 ... 3584 with four-bit codes):
+    // Three to seven K-slices a row (K = 1536 ... 3584 with four-bit codes):
     // the one-pass direct variant with some of its compute wavefronts idle is
     // still well ahead of the self-loading kernel, whose four wavefronts a
     // workgroup keep too little in flight (M = 4, us a launch: 37888 x 3584
     // 21.2 against 27.4, 16384 x 3072 9.0 / 13.6, 20480 x 2560 9.6 / 15.9,
-    // 8192 x 2048 5.6 / 6.2, eight-bit 16384 x 1536 7.5 / 10.4).
+    // 8192 x 2048 5.6 / 6.2, 32768 x 1536 11.7 / 15.4, eight-bit 16384 x 1536
+    // 7.5 / 10.4; with two slices it loses on large weights: 65536 x 1024
+    // 19.9 / 13.7).
     static const bool off = experiment_env("QMM_S2_NO_FEW_SLICES") != nullptr;
     const int64_t slices = K * bits / 8 / 256;
-    if (off || slices < 4 || !direct_x(M, N, K, bits)) return false;
+    if (off || slices < 3 || !direct_x(M, N, K, bits)) return false;
   }
   if (direct_x(M, N, K, bits)) {
     const int64_t cus = device_cus();

@@ -608,9 +608,9 @@ def test_prefill_rows_around_the_borders_of_the_split_role_kernels_tiles(bits, g
 
 
 @pytest.mark.parametrize("bits,gs,k", [(4, 64, 3584), (4, 64, 3072), (4, 128, 2560), (4, 64, 2048), (8, 64, 1536),
-                                       (8, 128, 1024)])
-def test_decode_with_four_to_seven_k_slices_a_row(bits, gs, k):
-    """K between four and seven 256-byte slices a row (hidden sizes 2048 to
+                                       (8, 128, 1024), (4, 64, 1536), (8, 64, 768)])
+def test_decode_with_three_to_seven_k_slices_a_row(bits, gs, k):
+    """K between three and seven 256-byte slices a row (hidden sizes 1536 to
     3584 with four-bit codes) runs the one-pass loader-wavefront kernel with
     some compute wavefronts idle: every row count's way of fetching the
     activations (direct, whole lines, staged), small and large N (one tile a
