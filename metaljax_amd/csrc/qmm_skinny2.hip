@@ -1137,7 +1137,7 @@ bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
 
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E) {
-  if (mode == QMM_MODE_MXFP4) return skinny2_mx_supported(N, K, s);
+  if (mode == QMM_MODE_MXFP4) return K / 512 >= 8 && skinny2_mx_supported(N, K, s);
   if (!skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b)) return false;   // bf16, float16 and float32 tables alike
   return K * bits / 8 / 256 >= 8;
 }
@@ -1177,11 +1177,14 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   }
 }
 
-// MXFP4 decode on the direct variants: K a multiple of 512 with at least eight
-// slices, scale rows dword-aligned (they are fetched as 16-byte runs).
+// MXFP4 decode on the direct variants: K a multiple of 512 with at least
+// three slices (with fewer than eight some compute wavefronts idle; M = 4, us
+// a launch against the general kernel: 16384 x 3072 8.2 / 16.4, 37888 x 3584
+// 19.4 / 33.3, 32768 x 1536 9.9 / 13.6), scale rows dword-aligned (they are
+// fetched as 16-byte runs).
 bool skinny2_mx_supported(int64_t N, int64_t K, const void* s) {
   static const bool off = experiment_env("QMM_NO_SKINNY_MX") != nullptr;
-  if (off || K % 512 || K / 512 < 8) return false;
+  if (off || K % 512 || K / 512 < 3) return false;
   if (reinterpret_cast<uintptr_t>(s) & 3u) return false;
   return N * (K / 2) < 0x7FFFFFFFll;                          // 32-bit lane offsets
 }

@@ -638,6 +638,25 @@ def test_decode_with_three_to_seven_k_slices_a_row(bits, gs, k):
         assert O.rel_l2(y[z], want) <= 2e-5, z
 
 
+@pytest.mark.parametrize("k", [1536, 2048, 3072, 3584])
+def test_mxfp4_decode_with_three_to_seven_k_slices_a_row(k):
+    """MXFP4 weights with K between three and seven 512-code slices a row on
+    the one-pass loader-wavefront kernel: every row count's way of fetching the
+    activations, small and large N, a ragged last tile, both outputs."""
+    rng = np.random.default_rng(k)
+    for n, ms in ((200, (1, 3, 8, 16)), (5000, (2, 5, 12)), (20011, (1, 4, 9, 16))):
+        _, words, sb, wd, sd = make_mxfp4(rng, n, k)
+        for m in ms:
+            x, xd = make_x(rng, m, k)
+            want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+            y32 = K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32)
+            assert O.rel_l2(out_f32(y32), want) <= 2e-5, (n, m, O.rel_l2(out_f32(y32), want))
+            err = np.abs(out_f32(y32) - want).max(axis=0) / np.abs(want).max()      # every output column
+            assert err.max() <= 1e-4, (n, m, int(err.argmax()), err.max())
+            y16 = K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4")
+            assert torch.equal(y16, y32.to(torch.bfloat16)), (n, m)
+
+
 # ----------------------------------------------------------- grouped / MoE ----
 
 def test_grouped_qmm_with_empty_and_ragged_experts():
