@@ -628,14 +628,15 @@ def test_decode_with_three_to_seven_k_slices_a_row(bits, gs, k):
             assert err.max() <= 1e-4, (n, m, int(err.argmax()), err.max())
             y16 = K.quantized_matmul(xd, wd, sd, bd, group_size=gs, bits=bits)
             assert torch.equal(y16, y32.to(torch.bfloat16)), (n, m)
-    # float16 tables and a batch of two weights
-    _, words, s, b, wd, sd, bd = make_affine(rng, 3000, k, bits, gs, "f16", lead=(2,))
-    x = O.round_bf16(rng.standard_normal((2, 6, k)).astype(np.float32))
-    y = out_f32(K.quantized_matmul(bf16_dev(O.f32_to_bf16_bits(x)), wd, sd, bd, group_size=gs, bits=bits,
-                                   out_dtype=torch.float32))
-    for z in range(2):
-        want = O.qmm(x[z], words[z], s[z], b[z], gs, bits)
-        assert O.rel_l2(y[z], want) <= 2e-5, z
+    # float16 and float32 tables, a batch of two weights, few and many rows of activations
+    for tab, m in (("f16", 6), ("f32", 3), ("f16", 13), ("f32", 16)):
+        _, words, s, b, wd, sd, bd = make_affine(rng, 3000, k, bits, gs, tab, lead=(2,))
+        x = O.round_bf16(rng.standard_normal((2, m, k)).astype(np.float32))
+        y = out_f32(K.quantized_matmul(bf16_dev(O.f32_to_bf16_bits(x)), wd, sd, bd, group_size=gs, bits=bits,
+                                       out_dtype=torch.float32))
+        for z in range(2):
+            want = O.qmm(x[z], words[z], s[z], b[z], gs, bits)
+            assert O.rel_l2(y[z], want) <= 2e-5, (tab, m, z)
 
 
 @pytest.mark.parametrize("k", [1536, 2048, 3072, 3584])
