@@ -431,7 +431,11 @@ void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st);
 // override it for experiments (read once).
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves) {
   static const int env_t = env_int("QMM_GEMV_T"), env_w = env_int("QMM_GEMV_WAVES");
-  int tt = (M > 8 && N >= 4096) ? 2 : 1;
+  // two 16-row tiles a workgroup only where that still leaves a workgroup per
+  // compute unit (256 x 32 rows); below, one tile: 4096 x 11008 at M = 16
+  // 24.3 against 33.4 us, 4096 x 14336 with groups of 32 32.3 against 49.9
+  // (8192 x 11008: 45.0 against 35.6 the other way)
+  int tt = (M > 8 && N >= 8192) ? 2 : 1;
   int ww = (K >= 4096) ? 8 : 4;
   if (env_t) tt = env_t;
   if (env_w) ww = env_w;
