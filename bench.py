@@ -42,11 +42,13 @@ def _events_ms(fn_timed, stream):
 
 
 def run_rotating(make_call, n_sets, steps, warmup):
-    """Time `steps` launches that cycle through `n_sets` bound calls.
+    """Time launches that cycle through `n_sets` bound calls.
 
-    A HIP graph holding one launch per set is replayed steps // n_sets times and
-    the remainder is launched eagerly, all inside one event bracket on the
-    current stream.  Returns milliseconds for exactly `steps` launches."""
+    A HIP graph holding one launch per set is replayed a whole number of times:
+    the `steps` asked for are rounded up to a multiple of `n_sets`, at least
+    two replays, so that no launch inside the event bracket is an eager one
+    (a kernel of a few microseconds launched call by call measures the host).
+    Returns (milliseconds, launches timed)."""
     import torch
     calls = [make_call(i) for i in range(n_sets)]
     stream = torch.cuda.Stream()
@@ -60,15 +62,13 @@ def run_rotating(make_call, n_sets, steps, warmup):
                 c.launch()
         graph.replay()                      # one untimed replay
         torch.cuda.synchronize()
-        reps, rem = divmod(steps, n_sets)
+        reps = max(2, -(-steps // n_sets))
 
         def timed():
             for _ in range(reps):
                 graph.replay()
-            for i in range(rem):
-                calls[i].launch()
         ms = _events_ms(timed, torch.cuda.current_stream())
-    return ms
+    return ms, reps * n_sets
 
 
 def bench_decode(cfg, M, steps, warmup):
@@ -85,8 +85,8 @@ def bench_decode(cfg, M, steps, warmup):
     def make_call(i):
         wi, si, bi = sets[i]
         return K.BoundQmm(x, wi, si, bi, ys[i], group_size=wl.group_size, bits=wl.bits, mode=wl.mode)
-    ms = run_rotating(make_call, n_sets, steps, warmup)
-    return wl, ms, n_sets, ys[0]
+    ms, launches = run_rotating(make_call, n_sets, steps, warmup)
+    return wl, ms / launches * 1e3, launches, n_sets, ys[0]
 
 
 def bench_decode_random(m, n, k, bits=4, mode="affine", tables="bf16", steps=200, warmup=20):
@@ -111,9 +111,9 @@ def bench_decode_random(m, n, k, bits=4, mode="affine", tables="bf16", steps=200
     ws = [torch.randint(-2**31, 2**31 - 1, (n, words), dtype=torch.int32, device="cuda", generator=g)
           for _ in range(n_sets)]
     ys = [torch.empty((m, n), dtype=torch.bfloat16, device="cuda") for _ in range(n_sets)]
-    ms = run_rotating(lambda i: K.BoundQmm(x, ws[i], s, b, ys[i], group_size=gs, bits=bits, mode=mode),
-                      n_sets, steps, warmup)
-    us = ms * 1e3 / steps
+    ms, launches = run_rotating(lambda i: K.BoundQmm(x, ws[i], s, b, ys[i], group_size=gs, bits=bits, mode=mode),
+                                n_sets, steps, warmup)
+    us = ms * 1e3 / launches
     nbytes = n * words * 4 + s.numel() * s.element_size() * (1 if b is None else 2) + (m * k + m * n) * 2
     return {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
@@ -160,11 +160,11 @@ def bench_once(cfg, steps=40, warmup=4, check=True):
         if cfg == 5:        # every row of C5 belongs to an expert, so the output needs no zero fill
             return K.BoundGrouped(x, wi, si, bi, ro, ys[i], group_size=64, bits=4)
         return K.BoundQmm(x, wi, si, bi, ys[i], group_size=wl.group_size, bits=wl.bits, mode=wl.mode)
-    ms = run_rotating(make_call, n_sets, steps, warmup)
-    us = ms * 1e3 / steps
+    ms, launches = run_rotating(make_call, n_sets, steps, warmup)
+    us = ms * 1e3 / launches
     tf = wl.flops / us / 1e6
     out = {"workload": wl.name, "us": round(us, 2), "TFLOP/s": round(tf, 1),
-           "GB/s": round(wl.algorithmic_bytes / us / 1e3, 1), "weight_sets": n_sets}
+           "GB/s": round(wl.algorithmic_bytes / us / 1e3, 1), "weight_sets": n_sets, "timed_launches": launches}
     if wl.mode == "mxfp4":
         # block-scaled matrix cores: each useful MFMA is issued twice (two FP6
         # activation terms), so both the useful and the issued rate are given
@@ -257,9 +257,6 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="time read-only and empty launches instead (what one launch over the "
                          "headline's bytes can reach on this GPU whatever its arithmetic)")
-    ap.add_argument("--probe-mfma", action="store_true",
-                    help="time a stream of matrix instructions with and without operand loads beside it "
-                         "(what bounds the prefill kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU; --gpus {args.gpus} is not supported "
@@ -285,22 +282,18 @@ def main():
         from metaljax_amd import profiling
         print(json.dumps({"probe": profiling.stream_probe()}))
         return 0
-    if args.probe_mfma:
-        from metaljax_amd import profiling
-        print(json.dumps({"mfma_feed": profiling.mfma_feed_probe()}))
-        return 0
     if args.shape:
         print(json.dumps({args.shape: bench_once(int(args.shape[1]), check=not args.no_cpu)}))
         return 0
-    wl, ms, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
+    wl, us, launches, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
     headline_rel_l2 = None if args.no_cpu else oracle_check(wl, y, True)     # outside the timed region
     assert headline_rel_l2 is None or headline_rel_l2 <= 1e-2, headline_rel_l2
-    us = ms * 1e3 / args.steps
     gbs = wl.algorithmic_bytes / us / 1e3
     kern, grid, block = K.plan(wl.M, wl.N, wl.K, wl.group_size, wl.bits, wl.mode)
     out = {
         "metric": METRIC, "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms / args.steps, 6),
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6),
+        "timed_launches": launches,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (seeded numpy draws, rng 1000+cfg; weights rotate through "
                 f"{n_sets} distinct buffers so each launch streams from HBM)",
@@ -321,18 +314,16 @@ def main():
         print(json.dumps(out))
         return 0
     # second decode point: the same weight at M = 1
-    wl1, ms1, _, _ = bench_decode(2, 1, max(args.steps // 4, 50), max(args.warmup // 4, 5))
-    us1 = ms1 * 1e3 / max(args.steps // 4, 50)
-    out["decode_M1"] = {"us": round(us1, 2), "GB/s": round(wl1.algorithmic_bytes / us1 / 1e3, 1),
-                        "frac_of_hbm_peak": round(wl1.algorithmic_bytes / us1 / 1e3 / HBM_PEAK_GBS, 4)}
+    def decode_leg(cfg, m):
+        wlx, usx, nx, _, _ = bench_decode(cfg, m, max(args.steps // 4, 50), max(args.warmup // 4, 5))
+        return {"workload": wlx.name, "us": round(usx, 2), "bytes": wlx.algorithmic_bytes,
+                "GB/s": round(wlx.algorithmic_bytes / usx / 1e3, 1),
+                "frac_of_hbm_peak": round(wlx.algorithmic_bytes / usx / 1e3 / HBM_PEAK_GBS, 4), "timed_launches": nx}
+    out["decode_M1"] = decode_leg(2, 1)
     if not args.no_extra:
         # C1 is a decode shape: graph replay over rotating weight sets like the
         # headline leg (a 6-7 us kernel timed call by call would measure the host)
-        wlc1, msc1, _, _ = bench_decode(1, 1, max(args.steps // 4, 50), max(args.warmup // 4, 5))
-        usc1 = msc1 * 1e3 / max(args.steps // 4, 50)
-        out["other_shapes"] = {"C1": {"workload": wlc1.name, "us": round(usc1, 2),
-                                      "GB/s": round(wlc1.algorithmic_bytes / usc1 / 1e3, 1),
-                                      "frac_of_hbm_peak": round(wlc1.algorithmic_bytes / usc1 / 1e3 / HBM_PEAK_GBS, 4)}}
+        out["other_shapes"] = {"C1": decode_leg(1, 1)}
         out["other_shapes"].update({f"C{c}": bench_once(c, check=not args.no_cpu) for c in (3, 4, 5)})
         # the library's bf16 matmul on the same shapes (no dequantization)
         out["dense_bf16"] = {"C3 [2048,4096]x[4096,4096]": bench_dense_bf16(2048, 4096, 4096),

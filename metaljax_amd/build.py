@@ -1,6 +1,7 @@
 """Builds libqmm_hip.so (the gfx950 kernels + the C ABI) with hipcc, in-tree.
 
-    python -m metaljax_amd.build
+    python -m metaljax_amd.build            the library (and the PJRT plugin)
+    python -m metaljax_amd.build --probe    libqmm_probe.so only (bench.py --probe)
 """
 
 from __future__ import annotations
@@ -49,7 +50,6 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
-    build_probe(verbose)
     return LIB
 
 
@@ -58,7 +58,9 @@ PROBE_LIB = os.path.join(LIBDIR, "libqmm_probe.so")
 
 def build_probe(verbose: bool = False) -> str:
     """The measuring kernels of `bench.py --probe` (read-only and empty
-    launches), a library of their own: not part of the quantized-matmul ABI."""
+    launches), a library of their own: not part of the quantized-matmul ABI and
+    not built by default (`python -m metaljax_amd.build --probe`)."""
+    os.makedirs(LIBDIR, exist_ok=True)
     cmd = ["hipcc", *FLAGS, "-shared", os.path.join(CSRC, "probe_stream.hip"), "-o", PROBE_LIB]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode:
@@ -108,5 +110,8 @@ def build_pjrt(verbose: bool = False):
 
 
 if __name__ == "__main__":
-    build(verbose=True)
-    build_pjrt(verbose=True)
+    if "--probe" in sys.argv[1:]:
+        build_probe(verbose=True)
+    else:
+        build(verbose=True)
+        build_pjrt(verbose=True)

@@ -569,7 +569,7 @@ int qmm_quantized_matmul(const void* x, int x_dtype, const void* w, const void* 
                 xs + ps + inner, workspace ? workspace_bytes : (size_t)0);
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  split_terms_dispatch(x, x_dtype, ws, batch, M, K, nullptr, 0, st);
+  split_terms_dispatch(x, x_dtype, ws, batch, M, K, nullptr, -1, st);
   int rc = check_launch("activation split launch");
   if (rc) return rc;
   rc = dense_bf16(ws, QMM_BF16, w, scales, biases, table_dtype, ws + xs, QMM_F32, batch, terms * M, N, K,
@@ -598,7 +598,7 @@ int qmm_grouped_qmm(const void* x, int x_dtype, const void* w, const void* scale
                 xs + ps + inner, workspace ? workspace_bytes : (size_t)0);
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  split_terms_dispatch(x, x_dtype, ws, 1, R, K, nullptr, 0, st);
+  split_terms_dispatch(x, x_dtype, ws, 1, R, K, nullptr, -1, st);
   int rc = check_launch("activation split launch");
   for (int t = 0; t < terms && !rc; ++t)
     rc = grouped_bf16(ws + (size_t)t * R * K * 2, QMM_BF16, w, scales, biases, table_dtype,

@@ -119,6 +119,8 @@ __global__ void split_terms_kernel(const T* __restrict__ x, uint16_t* __restrict
     const int64_t row = j / k, sr = src_row[row];
     ok = sr >= 0 && sr < x_rows;                   // a row outside x gathers zeros
     src = sr * k + (j - row * k);
+  } else if (x_rows >= 0) {                        // pair p reads row p of x: rows past the end read as zeros
+    ok = j / k < x_rows;
   }
   float v = 0.f;
   if (ok) {
@@ -128,9 +130,11 @@ __global__ void split_terms_kernel(const T* __restrict__ x, uint16_t* __restrict
   uint16_t* o = out + z * TERMS * rows_k + j;
 #pragma unroll
   for (int t = 0; t < TERMS; ++t) {
-    const uint32_t hi = __float_as_uint(v) & 0xFFFF0000u;       // truncation: the remainder is exact
+    uint32_t hi = __float_as_uint(v) & 0xFFFF0000u;             // truncation: the remainder is exact
+    if (v != v) hi |= 0x00400000u;                              // a NaN stays a NaN when its payload is cut
     o[(int64_t)t * rows_k] = (uint16_t)(hi >> 16);
-    v -= __uint_as_float(hi);
+    // inf / NaN stay in the first term alone (inf - inf would put NaN into the others)
+    v = (hi & 0x7F800000u) == 0x7F800000u ? 0.f : v - __uint_as_float(hi);
   }
 }
 
@@ -201,7 +205,8 @@ void dequant_dispatch(const void* w, const void* s, const void* b, int tab, void
 }
 
 // x (float16 / float32) [batch, rows, K] -> bf16 terms [batch, terms, rows, K];
-// with src_row (batch = 1): out row r = x row src_row[r] of x [x_rows, K]
+// with src_row (batch = 1): out row r = x row src_row[r] of x [x_rows, K]; without it and x_rows >= 0:
+// out row r = x row r, rows past x_rows read as zeros; x_rows < 0: no gather, rows is what x holds
 void split_terms_dispatch(const void* x, int x_dtype, void* out, int64_t batch, int64_t rows,
                           int64_t K, const int32_t* src_row, int64_t x_rows, hipStream_t st) {
   const int64_t total = batch * rows * K;

@@ -60,11 +60,13 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
 
     import torch
     here = os.path.dirname(os.path.abspath(__file__))
-    lib = ctypes.CDLL(os.path.join(here, "lib", "libqmm_probe.so"))
+    path = os.path.join(here, "lib", "libqmm_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libqmm_probe.so is not built: run `python -m metaljax_amd.build --probe`")
+    lib = ctypes.CDLL(path)
     vp, ci, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
     lib.probe_read.argtypes = [vp, i64, vp, ci, ci, ci, ci, vp]
     lib.probe_empty.argtypes = [vp, ci, ci, ci, vp]
-    lib.probe_loaders.argtypes = [vp, i64, vp, ci, ci, ci, ci, ci, ci, vp]
     n_sets = (2 * (256 << 20)) // nbytes + 1
     bufs = [torch.randint(-2**31, 2**31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda")
             for _ in range(n_sets)]
@@ -92,7 +94,7 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
             torch.cuda.synchronize()
             return a.elapsed_time(b) * 1e3 / (n * n_sets)
 
-    out = {"bytes": nbytes, "buffers": n_sets, "read": {}, "loaders": {}, "empty": {}}
+    out = {"bytes": nbytes, "buffers": n_sets, "read": {}, "empty": {}}
     for blocks, threads, unroll, lds in ((256, 1024, 8, 0), (256, 768, 8, 0), (256, 768, 8, 147456),
                                          (512, 512, 8, 0), (1024, 256, 8, 0), (2048, 256, 4, 0),
                                          (4096, 256, 2, 0), (8192, 256, 1, 0)):
@@ -102,61 +104,12 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
         us = timed(launch)
         out["read"][f"{blocks}x{threads} unroll {unroll} lds {lds}"] = {
             "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1)}
-    if nbytes // 256 <= 128 << 10:
-        for active in (4, 8, 12):
-            for dma in (0, 1):
-                for nt in (0, 1):
-                    def launch(i, st, a=active, d=dma, h=nt):
-                        rc = lib.probe_loaders(bufs[i].data_ptr(), nbytes, sink.data_ptr(), 256, 768, a, d, h,
-                                               147456, st)
-                        assert rc == 0, rc
-                    us = timed(launch)
-                    out["loaders"][f"256x768, {active} wavefronts ask, {'into LDS' if dma else 'into registers'}"
-                                   f"{', non-temporal' if nt else ''}"] = {
-                        "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1)}
     for blocks, threads, lds in ((256, 768, 147456), (256, 768, 0), (256, 256, 0)):
         def launch(i, st, b=blocks, t=threads, l=lds):
             rc = lib.probe_empty(sink.data_ptr(), b, t, l, st)
             assert rc == 0, rc
         out["empty"][f"{blocks}x{threads} lds {lds}"] = {"us": round(timed(launch), 2)}
     return out
-
-
-def mfma_feed_probe(iters: int = 1998):
-    """What feeding the matrix cores costs: per group of eight MFMAs, the
-    median over all wavefronts of the loop time in shader clocks (and ns), for
-    a pure MFMA stream and with 1 KB register loads / LDS reads beside it, one
-    and two wavefronts a SIMD, bf16 32x32x16 and block-scaled FP6 x FP4
-    32x32x64.  Returns a dict of results."""
-    import ctypes
-    import os
-
-    import numpy as np
-    import torch
-    here = os.path.dirname(os.path.abspath(__file__))
-    lib = ctypes.CDLL(os.path.join(here, "lib", "libqmm_probe.so"))
-    vp, ci = ctypes.c_void_p, ctypes.c_int
-    lib.probe_mfma_feed.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, vp]
-    data = torch.randint(-2**31, 2**31 - 1, ((16 << 20) // 4,), dtype=torch.int32, device="cuda")
-    out = torch.zeros(256 * 8 * 2, dtype=torch.int64, device="cuda")
-    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
-    res = {}
-    cases = [(0, 0, 0), (0, 2, 0), (0, 4, 0), (0, 8, 0), (0, 0, 8), (0, 0, 16), (0, 8, 16),
-             (1, 0, 0), (1, 2, 0), (1, 4, 0), (1, 8, 0), (1, 0, 8),
-             (100, 2, 8), (100, 4, 8), (100, 8, 8), (101, 2, 8), (101, 4, 8)]
-    for kind, loads, reads in cases:
-        for waves in (4, 8):
-            for _ in range(2):                      # the second run is the measured one
-                rc = lib.probe_mfma_feed(data.data_ptr(), out.data_ptr(), sink.data_ptr(), waves, loads, reads, kind,
-                                         iters, None)
-                assert rc == 0, rc
-                torch.cuda.synchronize()
-            t = out.cpu().numpy()[:256 * waves * 2].reshape(-1, 2)
-            name = (f"{'bf16 32x32x16' if kind % 100 == 0 else 'fp6 x fp4 32x32x64'}, {waves // 4} wavefront(s) a SIMD, "
-                    f"{loads} KB {'loads into LDS' if kind >= 100 else 'register loads'} + {reads} KB LDS reads a group")
-            res[name] = {"clocks_per_group": round(float(np.median(t[:, 1])) / iters, 1),
-                         "ns_per_group": round(float(np.median(t[:, 0])) * 10.0 / iters, 1)}
-    return res
 
 
 def decode_timeline(cfg: int = 2, rows=(1, 16)):

@@ -1212,6 +1212,59 @@ def test_gather_qmm_independent_decode_products_check_their_indices(pairs, n, k,
             assert O.rel_l2(got[i], want) <= 2e-5, i
 
 
+@pytest.mark.parametrize("xdt", ["f32", "f16"])
+def test_gather_qmm_wide_activations_without_lhs_read_zeros_past_x(xdt):
+    """float16 / float32 activations, no lhs indices, more pairs than rows of
+    x: pair p reads row p, and the pairs past the last row multiply zeros (the
+    split into bf16 terms must not read beyond x), as on the bf16 path."""
+    from metaljax_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(77)
+    e, t, pairs, n, k = 3, 4, 9, 128, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64, lead=(e,))
+    x = rng.standard_normal((t, k)).astype(np.float32)
+    if xdt == "f16":
+        x = x.astype(np.float16).astype(np.float32)
+        xd, code = torch.from_numpy(x).to(DEV).half(), _lib.F16
+    else:
+        xd, code = torch.from_numpy(x).to(DEV), _lib.F32
+    rhs = rng.integers(0, e, size=pairs).astype(np.int32)
+    rd = torch.from_numpy(rhs).to(DEV)
+    y = torch.full((pairs, n), 7.0, dtype=torch.float32, device=DEV)
+    nbytes = int(lib.qmm_gather_workspace_bytes(pairs, e, n, k, code))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    rc = lib.qmm_gather_qmm(xd.data_ptr(), code, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), _lib.BF16,
+                            y.data_ptr(), _lib.F32, None, rd.data_ptr(), pairs, t, e, n, k, 64, 4, 0,
+                            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc)
+    got = y.cpu().numpy()
+    for i in range(pairs):
+        if i >= t:
+            np.testing.assert_array_equal(got[i], np.zeros(n, np.float32))
+        else:
+            want = O.qmm(x[i][None], words[rhs[i]], s[rhs[i]], b[rhs[i]], 64, 4, "affine")[0]
+            assert O.rel_l2(got[i], want) <= 2e-5, i
+
+
+def test_wide_activations_non_finite_rows_stay_non_finite():
+    """A float32 activation row holding inf or NaN gives a non-finite output
+    row (the split into bf16 terms keeps inf / NaN in the first term and cuts
+    no NaN payload down to inf), and leaves the other rows alone."""
+    rng = np.random.default_rng(5)
+    n, k = 64, 512
+    _, words, s, b, wd, sd, bd = make_affine(rng, n, k, 4, 64)
+    x = rng.standard_normal((4, k)).astype(np.float32)
+    x[0, 3] = np.inf
+    x[1, 5] = np.nan
+    x[3, 7] = np.uint32(0x7F800001).view(np.float32)        # a NaN whose payload sits in the low mantissa bits
+    y = K.quantized_matmul(torch.from_numpy(x).to(DEV), wd, sd, bd, group_size=64, bits=4,
+                           out_dtype=torch.float32).cpu().numpy()
+    assert not np.isfinite(y[0]).any()
+    assert np.isnan(y[1]).all() and np.isnan(y[3]).all()
+    want = O.qmm(x[2][None], words, s, b, 64, 4)[0]
+    assert O.rel_l2(y[2], want) <= 2e-5
+
+
 # ------------------------------------- the named configurations at full size ----
 
 def _report(name, **figures):
