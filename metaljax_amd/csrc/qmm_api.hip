@@ -42,7 +42,7 @@ void gemm2_dispatch(const void* x, const void* w, const void* s, const void* b, 
                     hipStream_t st);
 bool mxfp4_mfma_supported(int64_t R, int64_t N, int64_t K);
 size_t mxfp4_workspace_bytes(int64_t R, int64_t K);
-void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block);
+void mxfp4_geometry(int64_t R, int64_t N, int64_t K, int* grid, int* block);
 void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, int y_dtype,
                          const int32_t* row_offsets, const int32_t* lhs_idx,
                          const int32_t* out_idx, int64_t R, int64_t x_rows, int64_t E, int64_t N,
@@ -301,7 +301,7 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
              int* grid, int* block) {
   if (mode == QMM_MODE_MXFP4 && M > kGemvMaxM && mxfp4_mfma_supported(M, N, K)) {
     int g, b;
-    mxfp4_geometry(M, N, &g, &b);
+    mxfp4_geometry(M, N, K, &g, &b);
     if (kernel) *kernel = QMM_KERNEL_MXFP4_MFMA;
     if (grid) *grid = g;
     if (block) *block = b;

@@ -41,6 +41,7 @@
 // row tiles x 4 column tiles) against 24 + 8 loads.  (The 16x16x128 form of
 // the instruction sustains well under half the rate of the 32x32x64 form.)
 #include <type_traits>
+#include <utility>
 
 #include "qmm_common.hpp"
 
@@ -348,9 +349,10 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
         for (int mt = 0; mt < 2; ++mt) {
           const i32x8 af = fp6_term(areg[t][u][mt], term);
 #pragma unroll
-          for (int nt = 0; nt < 4; ++nt)
+          for (int nt = 0; nt < 4; ++nt) {
             acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                 af, bfq[t & 1][u][nt], acc[mt][nt], kFp6, kFp4, t, (int)sa[u][mt][term], 0, sb[u][nt]);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         if (g < 2) {
@@ -457,6 +459,233 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(MxArgs a) {
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// The eight-wavefront form (K a multiple of 2048).  What bounds the kernel
+// above is not the matrix core: with the MFMAs compiled out it is 10 % faster,
+// with the weight loads emptied 40 %.  A wavefront keeps about sixteen loads in
+// flight, so four wavefronts have 64 KB a compute unit out against latencies of
+// 0.8 us (activation terms out of L2) to 1.6 us and more (weight lines), and a
+// wavefront that sits in issue behind its loads issues no MFMA either.  Here
+// the same 64 x 128 tile is worked by eight wavefronts, two a SIMD: K quarter
+// kq = wave % 4 as before, and the tile's rows in halves mh = wave / 4, so a
+// wavefront multiplies 32 x 128 (64 accumulator registers, 16 MFMAs a K-step)
+// and the SIMD has the other wavefront's MFMAs to issue while one waits.
+//   * weight codes: the two wavefronts of a K quarter share one ring of two
+//     stages, a stage = 128 rows x 128 bytes = two K-steps, i.e. whole cache
+//     lines (the 64-byte halves of the form above fetch every line twice);
+//     each of the two requests half of the rows; piece p of row r at position
+//     p ^ ((r >> 1) & 7), so that a 16-lane read pass covers every bank once.
+//   * one workgroup barrier a stage: before it a wavefront waits for its share
+//     of the stage's codes and finishes its reads of the stage before; after
+//     it the stage before is refilled with the stage after.
+//   * activation terms: straight into registers as above, two K-steps ahead.
+constexpr int kStage8 = TN * 128;
+constexpr int kKqLds8 = 2 * kStage8 + 2 * kScaleBytes;     // 36864
+constexpr int kLds8 = 4 * kKqLds8;                         // 147456
+
+__device__ __forceinline__ void stage_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__global__ __launch_bounds__(512) void mxfp4_mfma8_kernel(MxArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kq = wave & 3, mh = wave >> 2;
+  const int li = lane & 31, kh = lane >> 5;
+
+  int m_tiles = a.m_tiles;
+  if (a.row_offsets) m_tiles = find_row_tile(a.row_offsets, a.E, a.R, TM, -1).m_tiles;   // counted only
+  if (m_tiles == 0) return;
+  const int total = m_tiles * a.n_tiles;
+  const int per = (total + 7) / 8;
+  const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per || tile >= total) return;
+  int e = 0, row_hi = a.R, m0 = (tile % m_tiles) * TM;
+  const int n0 = (tile / m_tiles) * TN;
+  if (a.row_offsets) {
+    const RowTile rt = find_row_tile(a.row_offsets, a.E, a.R, TM, tile % m_tiles);
+    if (!rt.found) return;
+    e = rt.e; m0 = rt.lo + rt.idx * TM; row_hi = rt.hi;
+  }
+
+  const int nq = a.K / 2048;                      // quads of this K quarter: kq, kq + 4, ...
+  const int64_t wpitch = a.K / 2, spitch = a.K / 32;
+  const auto rw = make_rsrc(static_cast<const char*>(a.w) + (int64_t)e * a.N * wpitch, (int64_t)a.N * wpitch);
+  const auto rs = make_rsrc(static_cast<const char*>(a.s) + (int64_t)e * a.N * spitch, (int64_t)a.N * spitch);
+  const auto ra = make_rsrc(a.aq, (int64_t)(a.K / 128) * 192 * a.Rp);
+  const auto rsa = make_rsrc(a.as, (int64_t)(a.K / 512) * 32 * a.Rp);
+
+  unsigned char* wring = smem + kq * kKqLds8;
+  unsigned char* sring = wring + 2 * kStage8;
+
+  // weight codes: request j of this wavefront covers rows 64 mh + 8 j + lane / 8, a row's 128 bytes
+  uint32_t wvo[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = 64 * mh + 8 * j + (lane >> 3);
+    const int n = n0 + row;
+    const int gp = (lane & 7) ^ ((row >> 1) & 7);
+    wvo[j] = n < a.N ? (uint32_t)(n * wpitch + gp * 16) : kOutOfRange;
+  }
+  const int sn = n0 + 64 * mh + lane;             // weight scales: this lane's row
+  const uint32_t svo = sn < a.N ? (uint32_t)(sn * spitch) : kOutOfRange;
+  const uint32_t avo = (uint32_t)((kh * a.Rp + m0 + 32 * mh + li) * 16);
+  const uint32_t savo = (uint32_t)((kh * a.Rp + m0 + 32 * mh + li) * 4);
+  // codes of tile row r, piece p (16 bytes = one 32-block; a K-step is four) at r*128 + ((p ^ ((r >> 1) & 7)) << 4)
+  const uint32_t rd_row = (uint32_t)(li * 128);
+  const uint32_t rd_swz = (uint32_t)((li >> 1) & 7);
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nt][r] = 0.f;
+
+  u32x4 areg[4][2][3];                            // [K-step of the quad][u][plane]
+  uint32_t sa[2][2], sa_nxt[2][2];                // [u][term]
+
+  // (Requests past the last quad repeat the last quad's: every wavefront issues the same number of
+  // loads a stage whatever its position, the waits count loads.)
+  auto issue_a = [&](int i, int tq, u32x4 (&dst)[2][3]) {      // K-step tq of this wavefront's quad i
+    const int ks = 4 * (kq + 4 * (i < nq ? i : nq - 1)) + tq;
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint32_t so = (uint32_t)(((ks * 3 + p) * 4 + 2 * u) * 16) * (uint32_t)a.Rp;
+        dst[u][p] = __builtin_amdgcn_raw_buffer_load_b128(ra, avo, so, 0);
+      }
+  };
+  auto issue_scales = [&](int i) {                // activation and weight scales of quad i: 5 loads
+    const int quad = kq + 4 * (i < nq ? i : nq - 1);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint32_t so = (uint32_t)(((quad * 2 + t) * 4 + 2 * u) * 4) * (uint32_t)a.Rp;
+        sa_nxt[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rsa, savo, so, 0);
+      }
+    dma16(rs, sring + (i & 1) * kScaleBytes + mh * 1024, svo, (uint32_t)quad * 16);
+  };
+  auto dma_w = [&](int i, int h) {                // stage (quad i, half h) into slot h: 8 loads
+    const uint32_t so = (uint32_t)((kq + 4 * (i < nq ? i : nq - 1)) * 256 + h * 128);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      dma16(rw, wring + h * kStage8 + mh * 8192 + j * 1024, wvo[j], so);
+  };
+
+  // Loads retire in order; the order of issue is
+  //   [scales of quad 0] W(0) A(0) A(1) | after barrier s: [scales of the next quad, in the second
+  //   stage of a quad] W(s+1), then A(2s+2) and A(2s+3) during the stage's two K-steps,
+  // so before barrier s only this stage's two A sets (12 loads) may be out, and before K-step t of a
+  // stage the A set after it, W(s+1) and the scale loads: 14 or 19.
+  issue_scales(0);
+  dma_w(0, 0);
+  issue_a(0, 0, areg[0]);
+  issue_a(0, 1, areg[1]);
+
+  auto stage = [&](int i, auto hc) __attribute__((always_inline)) {
+    constexpr int h = decltype(hc)::value;
+    wait_vmcnt<12>();
+    stage_barrier();
+    if constexpr (h == 0) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) { sa[u][0] = sa_nxt[u][0]; sa[u][1] = sa_nxt[u][1]; }
+    } else {
+      issue_scales(i + 1);
+    }
+    if constexpr (h == 0) dma_w(i, 1); else dma_w(i + 1, 0);
+    const unsigned char* st = wring + h * kStage8;
+    const unsigned char* sq = sring + (i & 1) * kScaleBytes + li * 16;
+    auto kstep = [&](auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;
+      constexpr int tq = 2 * h + t;
+      wait_vmcnt<(h == 1 ? 19 : 14)>();
+      if constexpr (tq < 2) issue_a(i, tq + 2, areg[(tq + 2) & 3]); else issue_a(i + 1, tq - 2, areg[(tq + 2) & 3]);
+      uint32_t sbw[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) sbw[nt] = *reinterpret_cast<const uint32_t*>(sq + nt * 512 + tq * 4);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        i32x8 bf[4];
+        const uint32_t pc = (uint32_t)(4 * t + 2 * u + kh);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+          bf[nt] = as_fp4_operand(*reinterpret_cast<const u32x4*>(st + nt * 4096 + rd_row + ((pc ^ rd_swz) << 4)));
+#pragma unroll
+        for (int term = 0; term < 2; ++term) {
+          const i32x8 af = fp6_term(areg[tq][u], term);
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt) {
+            acc[nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                af, bf[nt], acc[nt], kFp6, kFp4, tq, (int)sa[u][term], 0, (int)(sbw[nt] >> (8 * kh + 16 * u)));
+          }
+        }
+      }
+    };
+    kstep(std::integral_constant<int, 0>{});
+    kstep(std::integral_constant<int, 1>{});
+  };
+  for (int i = 0; i < nq; ++i) {
+    stage(i, std::integral_constant<int, 0>{});
+    stage(i, std::integral_constant<int, 1>{});
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // ---- sum the four K quarters: red[wave][nt][r][lane]
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[(((wave * 4 + nt) * 16) + r) * 64 + lane] = acc[nt][r];
+  __syncthreads();
+  // wavefront w finishes the 32 x 32 block of row half w / 4, column block w % 4
+  const int fm = wave >> 2, fn = wave & 3;
+  float v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float t = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) t += red[((((q + 4 * fm) * 4 + fn) * 16) + r) * 64 + lane];
+    v[r] = t;
+  }
+  const bool wide = a.y_dtype != QMM_F32 && (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;
+  if (wide) {
+    // 16-bit outputs: transpose the block through the LDS left over beside `red`, store 16 bytes a lane
+    uint16_t* o16 = reinterpret_cast<uint16_t*>(smem + 8 * 4 * 16 * 64 * 4) + wave * (32 * 32);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rl = 8 * (r >> 2) + 4 * kh + (r & 3);
+      o16[rl * 32 + li] = (uint16_t)(a.y_dtype == QMM_BF16 ? f32_to_bf16_bits(v[r]) : f32_to_f16_bits(v[r]));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int idx = q * 64 + lane, rl = idx >> 2, pc = idx & 3;
+      const int row = m0 + 32 * fm + rl, col = n0 + 32 * fn + pc * 8;
+      if (row < row_hi && col < a.N) {
+        const int64_t orow = a.out_idx ? (int64_t)a.out_idx[row] : (int64_t)row;
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.y) + orow * a.N + col) =
+            *reinterpret_cast<const u32x4*>(o16 + rl * 32 + pc * 8);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = m0 + 32 * fm + 8 * (r >> 2) + 4 * kh + (r & 3), col = n0 + 32 * fn + li;
+      if (row < row_hi && col < a.N) {
+        const int64_t orow = a.out_idx ? (int64_t)a.out_idx[row] : (int64_t)row;
+        store_out(a.y, orow * a.N + col, v[r], a.y_dtype);
+      }
+    }
+  }
+}
+
 }  // namespace
 
 // Rows of the split-activation workspace (row count rounded up to the tile).
@@ -474,10 +703,10 @@ size_t mxfp4_workspace_bytes(int64_t R, int64_t K) {
   return (size_t)(rp * K * 3 / 2 + (K / 512) * 32 * rp);
 }
 
-void mxfp4_geometry(int64_t R, int64_t N, int* grid, int* block) {
+void mxfp4_geometry(int64_t R, int64_t N, int64_t K, int* grid, int* block) {
   const int64_t tiles = ceil_div(R, TM) * ceil_div(N, TN);
   *grid = (int)(ceil_div(tiles, 8) * 8);
-  *block = 256;
+  *block = K % 2048 == 0 ? 512 : 256;            // the eight-wavefront form | the four-wavefront form
 }
 
 // x bf16 [x_rows, K] (rows gathered through lhs_idx when given); w uint8 [E, N, K/2];
@@ -503,6 +732,11 @@ void mxfp4_mfma_dispatch(const void* x, const void* w, const void* s, void* y, i
   a.m_tiles = (int)(ceil_div(R, TM) + (row_offsets ? E : 0));
   a.n_tiles = (int)ceil_div(N, TN);
   const int grid = (int)(ceil_div((int64_t)a.m_tiles * a.n_tiles, 8) * 8), block = 256;
+  if (K % 2048 == 0) {
+    if (!lds_limit<mxfp4_mfma8_kernel>(kLds8)) return;
+    hipLaunchKernelGGL(mxfp4_mfma8_kernel, dim3(grid), dim3(512), kLds8, st, a);
+    return;
+  }
   if (!lds_limit<mxfp4_mfma_kernel>(kLds)) return;
   hipLaunchKernelGGL(mxfp4_mfma_kernel, dim3(grid), dim3(block), kLds, st, a);
 }
