@@ -204,6 +204,46 @@ def bench_dense_bf16(m, n, k, steps=40, experts=1):
     return {"us": round(us, 2), "TFLOP/s": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / PEAK_TFLOPS["bf16"], 4)}
 
 
+def bench_engine_execute(cfg=2, m=16, calls=100):
+    """Wall-clock time of `engine.execute` on the recognized program of a
+    decode shape (a sub-channel int4 dot, the weight as i8 codes + scales +
+    zero points, as a checkpoint holds it), buffers resident on the device:
+    what the fused kernel costs behind the recognizer, the interpreter and the
+    ctypes call, per call, after the first call has packed the weight.  Not a
+    kernel figure: the host work of one call is most of it."""
+    import numpy as np
+    import torch
+    from metaljax_amd import engine, qmm, synth
+    sh = synth.SHAPES[cfg]
+    n, k = sh["N"], sh["K"]
+    rng = np.random.default_rng(7)
+    q = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    scale = synth._bf16(rng.uniform(0.005, 0.02, size=(n, k // 64)))          # bf16 bit patterns
+    zero = np.zeros((n, k // 64), np.int8)
+    x = synth._bf16(rng.standard_normal((m, k)))
+    ex = engine.compile_program(synth.affine_program_text(m, n, k), "mlir")
+    bufs = [engine.buffer_from_host(q, engine._ENUM["S8"], q.shape),
+            engine.buffer_from_host(scale, engine._ENUM["BF16"], scale.shape),
+            engine.buffer_from_host(zero, engine._ENUM["S8"], zero.shape),
+            engine.buffer_from_host(x, engine._ENUM["BF16"], x.shape)]
+    qmm.reset_stats()
+    out = engine.execute(ex, bufs)          # packs the weight
+    torch.cuda.synchronize()
+    fused = qmm.stats().get("fused", 0)
+    for _ in range(5):
+        out = engine.execute(ex, bufs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        out = engine.execute(ex, bufs)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / calls
+    return {"us_per_call": round(us, 1), "calls": calls, "fused_dots": fused,
+            "result_on_device": bool(getattr(out[0].data, "is_cuda", False)),
+            "what": f"engine.execute of the recognized int4 g64 [{n},{k}] dot at M={m}, device-resident buffers, "
+                    "wall clock including the interpreter and the ctypes call"}
+
+
 def cpu_baseline(wl, budget_s=4.0):
     """The C restatement of the reference's unfused chain (oracle/qmm_oracle.c),
     timed on the host cores: the checker used as the reported CPU baseline."""
@@ -339,6 +379,7 @@ def main():
             "int4 g64 [37888,3584] M=4": bench_decode_random(4, 37888, 3584),
             "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
         }
+        out["engine_execute_C2"] = bench_engine_execute(2, 16)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))

@@ -28,11 +28,13 @@ call (csrc/pjrt_plugin.cc).
 from __future__ import annotations
 
 import hashlib
+import os
 
 import numpy as np
 
 from . import qmm
 from .interpreter import HostArray, Interpreter, from_numpy, host
+from .ir import np_dtype as ir_np_dtype
 
 # PJRT_Buffer_Type enumerators, in the order of the PJRT C API
 PJRT_TYPES = [
@@ -89,9 +91,52 @@ def buffer_from_host(data, type_enum: int, dims, byte_strides=None, offset: int 
         arr = np.array(arr, order="C", copy=True).reshape(dims)
     # (the bytes are copied either way: the caller's memory is free again when
     # this returns, which is what the plugin tells PJRT, pjrt_plugin.cc)
+    if device_resident():
+        return Buffer(_upload(arr, el), type_enum, dims)
     if el == "bf16":
-        arr = (arr.astype(np.uint32) << 16).view(np.float32)      # held as float32 values
+        h = from_numpy((arr.astype(np.uint32) << 16).view(np.float32), el)   # held as float32 values
+        h.bits = np.ascontiguousarray(arr)                                   # and as the type's own bytes
+        return Buffer(h, type_enum, dims)
     return Buffer(from_numpy(arr, el), type_enum, dims)
+
+
+def device_resident() -> bool:
+    """Do buffers live on the GPU?  Yes whenever one is visible (the
+    reference's `MetalBuffer.data` is a device array, engine.py:118-159);
+    METALJAX_HOST_BUFFERS=1 keeps them on the host."""
+    if os.environ.get("METALJAX_HOST_BUFFERS") == "1":
+        return False
+    try:
+        import torch
+        return torch.cuda.is_available()
+    except Exception:
+        return False
+
+
+def _upload(arr: np.ndarray, el: str):
+    """Host bytes in the element type's own storage -> a device tensor of that
+    type (bf16: the 16-bit patterns become a bfloat16 tensor)."""
+    import torch
+    arr = np.ascontiguousarray(arr)
+    if el == "bf16":
+        return torch.from_numpy(arr.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(arr).cuda()
+
+
+def _resident(v, el):
+    """A result value as what a Buffer of this engine holds: a device tensor
+    when buffers are device-resident, the value itself otherwise."""
+    if not device_resident() or not isinstance(v, HostArray):
+        return v
+    if el == "bf16":
+        from .packing import f32_to_bf16_bits
+        return _upload(f32_to_bf16_bits(np.ascontiguousarray(v.a, np.float32)), "bf16")
+    if el in ("i4", "ui4"):
+        return v                                    # no 4-bit tensor type: stays a host array
+    a = np.ascontiguousarray(v.a)
+    if not a.flags.writeable:
+        a = a.copy()
+    return _upload(a, el)
 
 
 def to_host(buf) -> bytes:
@@ -119,6 +164,13 @@ def buffer_pointer(buf) -> int:
     host address of a host array (stable while the Buffer is alive)."""
     v = buf.data if isinstance(buf, Buffer) else buf
     if isinstance(v, HostArray):
+        if v.el == "bf16" and v.bits is not None:
+            return int(v.bits.ctypes.data)
+        if v.el == "bf16" or v.a.dtype != ir_np_dtype(v.el):
+            # host bf16 values are held as float32: a reader of `nbytes` bytes
+            # at this address would get something else than the advertised type
+            raise UnsupportedProgram(f"Unsupported: a host-held {v.el} buffer has no storage in its own "
+                                     "element type to point at")
         return int(v.a.ctypes.data)
     return int(v.data_ptr())
 
@@ -147,7 +199,10 @@ class Executable:
         self.num_params = len(interp.main.body.args)
         self.num_outputs = len(interp.main.result_types)
         # PJRT_Buffer_Type integers, as the plugin reads them (metal_pjrt.cc:558)
-        self.out_types = [_EL_ENUM.get(t.el, 0) for t in interp.main.result_types]
+        unknown = [t.el for t in interp.main.result_types if t.el not in _EL_ENUM]
+        if unknown:
+            raise UnsupportedProgram(f"Unsupported result element type(s) {unknown}: no PJRT buffer type for them here")
+        self.out_types = [_EL_ENUM[t.el] for t in interp.main.result_types]
         self.out_els = [t.el for t in interp.main.result_types]
         self.out_dims = [list(t.shape) for t in interp.main.result_types]
         self.donated_params = sorted(interp.donated_args)
@@ -210,5 +265,6 @@ def execute(ex: Executable, buffers):
     outs = ex.interp.run(args)
     # every output as a buffer object (data, type_enum, dims, nbytes), which is
     # what the plugin wraps (metal_pjrt.cc:990-1010); `data` is a device tensor
-    # for a fused dot's result, a host array otherwise
-    return [Buffer(v, t, d) for v, t, d in zip(outs, ex.out_types, ex.out_dims)]
+    # whenever a GPU is visible (a literal op's host result is uploaded), as the
+    # reference's buffers hold device arrays
+    return [Buffer(_resident(v, el), t, d) for v, el, t, d in zip(outs, ex.out_els, ex.out_types, ex.out_dims)]

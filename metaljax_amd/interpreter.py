@@ -46,11 +46,12 @@ class UnsupportedOp(NotImplementedError):
 class HostArray:
     """A host tensor: numpy storage + the StableHLO element type."""
 
-    __slots__ = ("a", "el", "__weakref__")
+    __slots__ = ("a", "el", "bits", "__weakref__")
 
     def __init__(self, a, el):
         self.a = a
         self.el = el
+        self.bits = None            # bf16 only, optional: the 16-bit patterns, for callers that need the type's own bytes
 
     @property
     def shape(self):
@@ -103,6 +104,15 @@ def from_numpy(a, el=None) -> HostArray:
     return settle(a, el)
 
 
+# Host copies of device tensors, one per tensor object while it lives: a
+# program argument that several literal ops (or several pack builds) read is
+# copied back once.  Engine buffers and fused results are never written in
+# place, which is what makes the copy reusable.
+_MIRRORS = {}
+MIRROR_MAX_BYTES = 16 << 20     # larger tensors (weights) are copied back whenever read: no second copy is kept
+HOST_COPIES = [0]               # device -> host copies made (tests count them)
+
+
 def host(v) -> HostArray:
     """Any runtime value as a HostArray (device tensors are copied back)."""
     if isinstance(v, HostArray):
@@ -111,9 +121,20 @@ def host(v) -> HostArray:
         return host(v.data)
     import torch
     if isinstance(v, torch.Tensor):
+        key = id(v)
+        hit = _MIRRORS.get(key)
+        if hit is not None and hit[0]() is v:
+            return hit[1]
+        if v.is_cuda:
+            HOST_COPIES[0] += 1
         if v.dtype == torch.bfloat16:
-            return HostArray(v.float().cpu().numpy(), "bf16")
-        return from_numpy(v.cpu().numpy())
+            h = HostArray(v.float().cpu().numpy(), "bf16")
+        else:
+            h = from_numpy(v.cpu().numpy())
+        if v.is_cuda and v.numel() * v.element_size() <= MIRROR_MAX_BYTES:
+            import weakref
+            _MIRRORS[key] = (weakref.ref(v, lambda _, key=key: _MIRRORS.pop(key, None)), h)
+        return h
     return from_numpy(v)
 
 

@@ -25,6 +25,23 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+# One scratch allocation per (device, stream), grown to the largest request seen:
+# calls on one stream are ordered, so the next call may overwrite what the
+# previous one used; nothing is allocated per call once it has grown.
+_SCRATCH = {}
+
+
+def _scratch(need: int, like: torch.Tensor):
+    if not need:
+        return None
+    key = (like.device.index, _stream(like))
+    ws = _SCRATCH.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=like.device)
+        _SCRATCH[key] = ws
+    return ws
+
+
 def _need_cuda(*ts):
     for t in ts:
         if t is not None and not t.is_cuda:
@@ -85,7 +102,7 @@ def quantized_matmul(x, w, scales, biases=None, transpose=True, group_size=64, b
     tab = _dt(scales.dtype) if mode == "affine" else BF16
     need = int(lib.qmm_workspace_bytes(batch, mrows, n, k, group_size, bits, _MODE[mode],
                                        _dt(x2.dtype)))
-    ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    ws = _scratch(need, x)
     rc = lib.qmm_quantized_matmul(
         _ptr(x2), _dt(x2.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y), _dt(out_dtype),
         batch, mrows, n, k, group_size, bits, _MODE[mode], _ptr(ws), need, _stream(x))
@@ -118,7 +135,7 @@ def grouped_qmm(x, w, scales, biases, row_offsets, group_size=64, bits=4, mode="
     ro = row_offsets.to(torch.int32).contiguous()
     tab = _dt(scales.dtype) if mode == "affine" else BF16
     need = int(lib.qmm_workspace_bytes(1, r, n, k, group_size, bits, _MODE[mode], _dt(x.dtype)))
-    ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    ws = _scratch(need, x)
     rc = lib.qmm_grouped_qmm(_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab,
                              _ptr(y), _dt(out_dtype), _ptr(ro), r, e, n, k, group_size, bits,
                              _MODE[mode], _ptr(ws), need, _stream(x))
@@ -162,7 +179,7 @@ def gather_qmm(x, w, scales, biases=None, lhs_indices=None, rhs_indices=None, tr
     x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
     biases = None if biases is None else biases.contiguous()
     nbytes = int(lib.qmm_gather_workspace_bytes(p, e, n, k, _dt(x.dtype)))
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
+    ws = _scratch(nbytes, x)
     tab = _dt(scales.dtype) if mode == "affine" else BF16
     rc = lib.qmm_gather_qmm(_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab,
                             _ptr(y), _dt(out_dtype), _ptr(lhs), _ptr(rhs), p, t, e, n, k,

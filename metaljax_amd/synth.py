@@ -125,3 +125,32 @@ def to_device(wl: Workload, device="cuda"):
         s, b = torch.from_numpy(wl.scales).to(device), None
     ro = None if wl.row_offsets is None else torch.from_numpy(wl.row_offsets).to(device)
     return x, w, s, b, ro
+
+
+def affine_program_text(m: int, n: int, k: int, group_size: int = 64, el: str = "bf16") -> str:
+    """A StableHLO module whose one dot the recognizer rewrites into the fused
+    call: signed 4-bit-range codes i8 [N, K] viewed by groups, one scale and
+    one zero point per group, `x @ ((q - z) * s)^T` (the sub-channel form of
+    reference tests/test_qmm.py:991-1027).  Arguments: q i8 [N, K], scale
+    [N, K/gs] (`el`), zero i8 [N, K/gs], x [M, K]; result [M, N]."""
+    ng = k // group_size
+
+    def t(shape, e):
+        return "tensor<" + "x".join([*map(str, shape), e]) + ">"
+    s3, q3 = t((n, ng, group_size), el), t((n, ng, group_size), "i8")
+    return f"""
+module @jit_affine_grouped {{
+  func.func public @main(%q: {t((n, k), "i8")}, %scale: {t((n, ng), el)}, %zero: {t((n, ng), "i8")}, %x: {t((m, k), el)}) -> {t((m, n), el)} {{
+    %qs = stablehlo.reshape %q : ({t((n, k), "i8")}) -> {q3}
+    %qf = stablehlo.convert %qs : ({q3}) -> {s3}
+    %sb = stablehlo.broadcast_in_dim %scale, dims = [0, 1] : ({t((n, ng), el)}) -> {s3}
+    %zc = stablehlo.convert %zero : ({t((n, ng), "i8")}) -> {t((n, ng), el)}
+    %zb = stablehlo.broadcast_in_dim %zc, dims = [0, 1] : ({t((n, ng), el)}) -> {s3}
+    %d = stablehlo.subtract %qf, %zb : {s3}
+    %w3 = stablehlo.multiply %d, %sb : {s3}
+    %w = stablehlo.reshape %w3 : ({s3}) -> {t((n, k), el)}
+    %y = stablehlo.dot_general %x, %w, contracting_dims = [1] x [1] : ({t((m, k), el)}, {t((n, k), el)}) -> {t((m, n), el)}
+    return %y : {t((m, n), el)}
+  }}
+}}
+"""

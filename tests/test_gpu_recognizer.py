@@ -268,3 +268,56 @@ def test_a_dot_left_to_the_interpreter_runs_on_the_device():
     np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2 * np.abs(want).max())
     from metaljax_amd.packing import f32_to_bf16_bits
     assert engine.to_host(buf) == f32_to_bf16_bits(got).tobytes()
+
+
+# ------------------------------------------ device-resident engine buffers ----
+
+def test_engine_buffers_live_on_the_device():
+    """`buffer_from_host` uploads once (reference engine.py:118-159: a buffer's
+    data is a device array): the tensor has the advertised element type,
+    `buffer_pointer` is its device address and `to_host` gives the bytes back."""
+    from metaljax_amd.packing import f32_to_bf16_bits
+    rng = np.random.default_rng(0)
+    cases = [("BF16", f32_to_bf16_bits(rng.standard_normal((3, 8)).astype(np.float32)), torch.bfloat16),
+             ("F32", rng.standard_normal((2, 5)).astype(np.float32), torch.float32),
+             ("S8", rng.integers(-8, 8, (4, 4)).astype(np.int8), torch.int8),
+             ("U32", rng.integers(0, 2**32, (3, 3), dtype=np.uint64).astype(np.uint32), torch.uint32),
+             ("PRED", rng.integers(0, 2, (7,)).astype(np.bool_), torch.bool)]
+    for name, arr, dt in cases:
+        b = engine.buffer_from_host(arr, engine._ENUM[name], arr.shape)
+        assert isinstance(b.data, torch.Tensor) and b.data.is_cuda and b.data.dtype == dt, name
+        assert b.nbytes == arr.nbytes and engine.buffer_pointer(b) == b.data.data_ptr()
+        assert engine.to_host(b) == arr.tobytes(), name
+
+
+def test_execute_reads_resident_buffers_without_host_copies():
+    """After the first call has packed the weight, `execute` on device-resident
+    buffers copies nothing back to the host: the activation goes to the kernel
+    as it lies, the result stays a device tensor (reference engine.py:385-417)."""
+    from metaljax_amd import synth
+    from metaljax_amd.packing import f32_to_bf16_bits
+    m, n, k = 4, 128, 512
+    rng = np.random.default_rng(12)
+    q = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    s = T.bf16_round(rng.uniform(0.005, 0.02, size=(n, k // 64)).astype(np.float32))
+    z = rng.integers(-2, 3, size=(n, k // 64)).astype(np.int8)
+    x = T.bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    ex = engine.compile_program(synth.affine_program_text(m, n, k))
+    bufs = [engine.buffer_from_host(q, engine._ENUM["S8"], q.shape),
+            engine.buffer_from_host(f32_to_bf16_bits(s), engine._ENUM["BF16"], s.shape),
+            engine.buffer_from_host(z, engine._ENUM["S8"], z.shape),
+            engine.buffer_from_host(f32_to_bf16_bits(x), engine._ENUM["BF16"], x.shape)]
+    assert all(b.data.is_cuda for b in bufs)
+    (y0,) = engine.execute(ex, bufs)
+    assert qmm.stats()["packs"] == 1 and qmm.stats()["fallbacks"] == 0
+    before = I.HOST_COPIES[0]
+    (y1,) = engine.execute(ex, bufs)
+    assert I.HOST_COPIES[0] == before                      # nothing came back to the host
+    assert qmm.stats()["packs"] == 1                       # the pack was found by buffer identity
+    assert y1.data.is_cuda and y1.data.dtype == torch.bfloat16
+    w = (q.astype(np.float32) - np.repeat(z, 64, axis=1)) * np.repeat(s, 64, axis=1)
+    want = x @ w.T
+    got = np.frombuffer(engine.to_host(y1), np.uint16).reshape(m, n)
+    got = (got.astype(np.uint32) << 16).view(np.float32)
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+    assert engine.to_host(y0) == engine.to_host(y1)
