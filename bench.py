@@ -204,6 +204,38 @@ def bench_dense_bf16(m, n, k, steps=40, experts=1):
     return {"us": round(us, 2), "TFLOP/s": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / PEAK_TFLOPS["bf16"], 4)}
 
 
+def bench_moe_decode(tokens, experts=8, topk=2, n=14336, k=4096, steps=60, warmup=6):
+    """Expert-indexed decode (the call a recognized mixture-of-experts block
+    makes per projection, reference src/metaljax/moe.py:1320): `tokens` tokens,
+    each routed to `topk` of `experts` int4 g64 experts of [n, k], pairs in
+    token order (unsorted, as the reference hands them over).  Graph replay
+    over rotating weight sets; GB/s counts the weights and tables of the
+    experts the routing touches, once each."""
+    import torch
+    from metaljax_amd import kernels as K
+    g = torch.Generator(device="cuda").manual_seed(tokens * 131 + experts)
+    words = k // 8
+    per_set = experts * n * words * 4
+    n_sets = max(2, (2 * LLC_BYTES) // per_set + 1)
+    ws = [torch.randint(-2**31, 2**31 - 1, (experts, n, words), dtype=torch.int32, device="cuda", generator=g)
+          for _ in range(n_sets)]
+    s = (torch.rand((experts, n, k // 64), device="cuda", generator=g) * 0.015 + 0.005).bfloat16()
+    b = (-8 * s.float()).bfloat16()
+    x = torch.randn((tokens, k), device="cuda", generator=g).bfloat16()
+    logits = torch.randn((tokens, experts), device="cuda", generator=g)
+    rhs = torch.topk(logits, topk, dim=-1).indices.reshape(-1).to(torch.int32).contiguous()
+    lhs = torch.arange(tokens, device="cuda", dtype=torch.int32).repeat_interleave(topk).contiguous()
+    ys = [torch.empty((tokens * topk, n), dtype=torch.bfloat16, device="cuda") for _ in range(n_sets)]
+    ms, launches = run_rotating(lambda i: K.BoundGather(x, ws[i], s, b, lhs, rhs, ys[i], group_size=64, bits=4),
+                                n_sets, steps, warmup)
+    us = ms * 1e3 / launches
+    touched = int(torch.unique(rhs).numel())
+    nbytes = touched * (n * words * 4 + 2 * n * (k // 64) * 2) + tokens * k * 2 + tokens * topk * n * 2
+    return {"us": round(us, 2), "pairs": tokens * topk, "experts_touched": touched, "bytes": nbytes,
+            "GB/s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+            "timed_launches": launches}
+
+
 def bench_engine_execute(cfg=2, m=16, calls=100):
     """Wall-clock time of `engine.execute` on the recognized program of a
     decode shape (a sub-channel int4 dot, the weight as i8 codes + scales +
@@ -229,7 +261,7 @@ def bench_engine_execute(cfg=2, m=16, calls=100):
     qmm.reset_stats()
     out = engine.execute(ex, bufs)          # packs the weight
     torch.cuda.synchronize()
-    fused = qmm.stats().get("fused", 0)
+    stats = qmm.stats()
     for _ in range(5):
         out = engine.execute(ex, bufs)
     torch.cuda.synchronize()
@@ -238,7 +270,8 @@ def bench_engine_execute(cfg=2, m=16, calls=100):
         out = engine.execute(ex, bufs)
     torch.cuda.synchronize()
     us = (time.perf_counter() - t0) * 1e6 / calls
-    return {"us_per_call": round(us, 1), "calls": calls, "fused_dots": fused,
+    return {"us_per_call": round(us, 1), "calls": calls, "dots_recognized": stats.get("recognized", 0),
+            "packs_built": stats.get("packs", 0), "fallbacks": stats.get("fallbacks", 0),
             "result_on_device": bool(getattr(out[0].data, "is_cuda", False)),
             "what": f"engine.execute of the recognized int4 g64 [{n},{k}] dot at M={m}, device-resident buffers, "
                     "wall clock including the interpreter and the ctypes call"}
@@ -286,6 +319,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other named shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--m16-only", action="store_true", help="run the headline decode leg only")
+    ap.add_argument("--moe-decode", action="store_true",
+                    help="time the expert-indexed decode legs only (for profiling those kernels)")
     ap.add_argument("--shape", choices=["C3", "C4", "C5"], default=None,
                     help="time one of the other named shapes only (for profiling that kernel)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -324,6 +359,9 @@ def main():
         return 0
     if args.shape:
         print(json.dumps({args.shape: bench_once(int(args.shape[1]), check=not args.no_cpu)}))
+        return 0
+    if args.moe_decode:
+        print(json.dumps({"moe_decode": {f"{t} token(s)": bench_moe_decode(t) for t in (1, 16)}}))
         return 0
     wl, us, launches, n_sets, y = bench_decode(2, 16, args.steps, args.warmup)
     headline_rel_l2 = None if args.no_cpu else oracle_check(wl, y, True)     # outside the timed region
@@ -379,6 +417,7 @@ def main():
             "int4 g64 [37888,3584] M=4": bench_decode_random(4, 37888, 3584),
             "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
         }
+        out["moe_decode"] = {f"8 experts int4 g64 [14336,4096], top-2, {t} token(s)": bench_moe_decode(t) for t in (1, 16)}
         out["engine_execute_C2"] = bench_engine_execute(2, 16)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)

@@ -321,3 +321,38 @@ class BoundGrouped:
         if rc:
             _lib.check(rc)
         return self.y
+
+
+class BoundGather:
+    """A gather_qmm call with every argument resolved once (see BoundQmm):
+    x [T, K]; lhs / rhs indices int32 [P] on the device (pair p reads row
+    lhs[p] of x and expert rhs[p]); results into the preallocated `y` [P, N]
+    (a pair whose expert index is outside the weight leaves its row alone)."""
+
+    def __init__(self, x, w, scales, biases, lhs_indices, rhs_indices, y, group_size=64, bits=4, mode="affine"):
+        _need_cuda(x, w, scales, biases, lhs_indices, rhs_indices, y)
+        (e,), n, k = _weight_dims(w, bits, mode)
+        for t in (x, w, scales, biases, lhs_indices, rhs_indices, y):
+            if t is not None and not t.is_contiguous():
+                raise _lib.QmmError(1, "BoundGather needs contiguous tensors")
+        p = rhs_indices.numel()
+        if rhs_indices.dtype != torch.int32 or (lhs_indices is not None and lhs_indices.dtype != torch.int32):
+            raise _lib.QmmError(1, "indices must be int32")
+        if x.dim() != 2 or tuple(y.shape) != (p, n):
+            raise _lib.QmmError(1, "x must be [T, K] and y [P, N]")
+        self._lib = _lib.load()
+        tab = _dt(scales.dtype) if mode == "affine" else BF16
+        need = int(self._lib.qmm_gather_workspace_bytes(p, e, n, k, _dt(x.dtype)))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+        self._keep = (x, w, scales, biases, lhs_indices, rhs_indices, y, ws)
+        self._args = (_ptr(x), _dt(x.dtype), _ptr(w), _ptr(scales), _ptr(biases), tab, _ptr(y),
+                      _dt(y.dtype), _ptr(lhs_indices), _ptr(rhs_indices), p, x.shape[0], e, n, k,
+                      group_size, bits, _MODE[mode], _ptr(ws), need)
+        self.y = y
+
+    def launch(self, stream=None):
+        st = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        rc = self._lib.qmm_gather_qmm(*self._args, st)
+        if rc:
+            _lib.check(rc)
+        return self.y

@@ -54,7 +54,7 @@ MOE_ENABLED = os.environ.get("METALJAX_MOE", "1") != "0"
 VERIFY = os.environ.get("METALJAX_MOE_VERIFY", "1") != "0"
 VERIFY_DRAWS = int(os.environ.get("METALJAX_MOE_VERIFY_DRAWS", "3"))
 _DEBUG = os.environ.get("METALJAX_DEBUG", "") == "1"
-STATS = {"recognized": 0, "verified": 0, "fallbacks": 0, "gather_qmm": 0, "dispatches": 0}
+STATS = {"recognized": 0, "verified": 0, "fallbacks": 0, "gather_qmm": 0, "dispatches": 0, "host_copies": 0}
 
 
 def stats() -> dict:
@@ -83,6 +83,97 @@ _ELEMENTWISE = frozenset("""
 
 
 # ------------------------------------------------------- run-time pieces ----
+
+class DevArray:
+    """A device tensor plus its StableHLO element type: what a slot of a
+    running dispatch holds.  Everything between the per-expert products runs
+    on these, on the device (reference moe.py:1425-1461 runs its closure list
+    on device arrays)."""
+
+    __slots__ = ("t", "el")
+
+    def __init__(self, t, el):
+        self.t = t
+        self.el = el
+
+
+_TORCH_EL = {"i1": "bool", "i8": "int8", "i16": "int16", "i32": "int32", "i64": "int64", "ui8": "uint8",
+             "f16": "float16", "bf16": "bfloat16", "f32": "float32", "f64": "float64"}
+_FLOATS = ("f16", "bf16", "f32", "f64")
+
+
+class _HostOnly(Exception):
+    """This op / element type is not modelled on the device: the fill runs on
+    the host (a copy each way) instead."""
+
+
+def _tdtype(el):
+    import torch
+    return getattr(torch, _TORCH_EL[el])
+
+
+def dev(v) -> DevArray:
+    """Any runtime value as a DevArray (host values are uploaded)."""
+    import torch
+    from . import qmm
+    if isinstance(v, DevArray):
+        return v
+    if hasattr(v, "type_enum") and hasattr(v, "data"):
+        v = v.data
+    if isinstance(v, torch.Tensor):
+        el = {getattr(torch, name): e for e, name in _TORCH_EL.items()}.get(v.dtype)
+        if el is None:
+            raise _HostOnly(str(v.dtype))
+        return DevArray(v if v.is_cuda else v.cuda(), el)
+    h = host(v)
+    if h.el not in _TORCH_EL:
+        raise _HostOnly(h.el)
+    return DevArray(qmm.to_device(h), h.el)
+
+
+def _dev_elementwise(op, args, out_el):
+    """One elementwise StableHLO op on device tensors, with the literal
+    path's meaning: 16-bit floats are widened, computed in float32 and rounded
+    once (what torch's elementwise kernels do), comparisons give i1."""
+    import torch
+    if out_el not in _TORCH_EL or any(a.el not in _TORCH_EL for a in args):
+        raise _HostOnly(op.name)
+    name = op.name[len("stablehlo."):]
+    t = [a.t for a in args]
+    fl = all(a.el in _FLOATS for a in args)
+    binary = {"add": torch.add, "subtract": torch.sub, "multiply": torch.mul, "divide": torch.div,
+              "maximum": torch.maximum, "minimum": torch.minimum, "power": torch.pow}
+    unary = {"abs": torch.abs, "ceil": torch.ceil, "floor": torch.floor, "exponential": torch.exp,
+             "log": torch.log, "logistic": torch.sigmoid, "negate": torch.neg, "rsqrt": torch.rsqrt,
+             "sqrt": torch.sqrt, "tanh": torch.tanh, "sign": torch.sign, "round_nearest_even": torch.round}
+    logic = {"and": torch.bitwise_and, "or": torch.bitwise_or, "xor": torch.bitwise_xor}
+    if name in binary and fl:
+        return binary[name](t[0], t[1])
+    if name in unary and fl:
+        return unary[name](t[0])
+    if name in logic and not fl:
+        return logic[name](t[0], t[1])
+    if name == "not" and not fl:
+        return torch.bitwise_not(t[0])
+    if name == "compare":
+        fn = {"EQ": torch.eq, "NE": torch.ne, "LT": torch.lt, "LE": torch.le, "GT": torch.gt,
+              "GE": torch.ge}[op.attrs["comparison_direction"]]
+        return fn(t[0], t[1])
+    if name == "select":
+        return torch.where(t[0], t[1], t[2])
+    if name == "clamp" and fl:
+        return torch.minimum(torch.maximum(t[1], t[0]), t[2])
+    if name == "convert":
+        src = args[0].el
+        if out_el == "i1":
+            return t[0] != 0
+        if src in _FLOATS and out_el not in _FLOATS:
+            info = torch.iinfo(_tdtype(out_el))
+            x = torch.nan_to_num(torch.trunc(t[0].double()), nan=0.0).clamp(info.min, info.max)
+            return x.to(_tdtype(out_el))
+        return t[0].to(_tdtype(out_el))
+    raise _HostOnly(op.name)
+
 
 def split_experts(arrays, e):
     """Packed arrays whose leading dims multiply to `e` expert slots (a batched
@@ -316,8 +407,9 @@ class PairPlan:
     `lower(value, e, t)` returns the slot that will hold `value` in pair space
     (`[P] + rest`, or its dense self when it has neither axis) and appends the
     closure that fills it.  Closures take a run context with `env` (the
-    program's values), `eidx` / `tidx` (expert / token of every pair, host
-    int64) and `slots`."""
+    program's values), `eidx_dev` / `tidx_dev` (expert / token of every pair,
+    int64 on the device; `eidx32` / `tidx32` as the kernels take them) and
+    `slots` (DevArrays: every closure runs on the device)."""
 
     def __init__(self, interp, qst, E, T):
         self.interp, self.qst, self.E, self.T = interp, qst, E, T
@@ -360,25 +452,36 @@ class PairPlan:
 
     # -- values from outside the region: gathered on the way in
     def _external(self, v, e, t):
-        self.reads.append(v)
+        op = _producer(v)
+        fixed = []                        # a constant is evaluated when planned and uploaded once
+        if op is not None and op.name == "stablehlo.constant":
+            out = REGISTRY[op.name](self.interp, op, [], {})
+            fixed.append(out[0] if isinstance(out, (list, tuple)) else out)
+        else:
+            self.reads.append(v)
 
         def fill(ctx):
-            a = host(ctx.env[v])
+            if fixed:
+                if not isinstance(fixed[0], DevArray):
+                    fixed[0] = dev(fixed[0])
+                a = fixed[0]
+            else:
+                a = dev(ctx.env[v])
             if e is None and t is None:
                 return a
-            x = a.a
+            x = a.t
             if e is not None and t is not None:
-                x = np.moveaxis(x, (e, t), (0, 1))[ctx.eidx, ctx.tidx]
+                x = x.movedim((e, t), (0, 1))[ctx.eidx_dev, ctx.tidx_dev]
             elif e is not None:
-                x = np.moveaxis(x, e, 0)[ctx.eidx]
+                x = x.movedim(e, 0).index_select(0, ctx.eidx_dev)
             else:
-                x = np.moveaxis(x, t, 0)[ctx.tidx]
-            return HostArray(x, a.el)
+                x = x.movedim(t, 0).index_select(0, ctx.tidx_dev)
+            return DevArray(x, a.el)
         return self._new_slot(fill, e is not None or t is not None)
 
     def _lead(self, slot, a, P):
-        """A slot's array with a leading pair axis of extent P or 1."""
-        return a if self.paired[slot] else a.reshape((1,) + a.shape)
+        """A slot's tensor with a leading pair axis of extent P or 1."""
+        return a if self.paired[slot] else a.reshape((1,) + tuple(a.shape))
 
     # -- shape-preserving ops
     def _elementwise(self, op, e, t):
@@ -393,17 +496,21 @@ class PairPlan:
             else:
                 raise Reject(f"{op.name} mixes shapes {xs} and {shape}")
         handler = REGISTRY[op.name]
+        out_el = elem(op.results[0])
 
         def fill(ctx):
             args = []
             for s in ins:
                 h = ctx.slots[s]
                 # an unpaired full-shape operand (a splat) broadcasts along the pair axis
-                if not self.paired[s] and h.a.ndim:
-                    h = HostArray(h.a.reshape((1,) + h.a.shape), h.el)
+                if not self.paired[s] and h.t.dim():
+                    h = DevArray(h.t.reshape((1,) + tuple(h.t.shape)), h.el)
                 args.append(h)
-            out = handler(self.interp, op, args, {})
-            return out[0] if isinstance(out, (list, tuple)) else out
+            try:
+                return DevArray(_dev_elementwise(op, args, out_el), out_el)
+            except _HostOnly:
+                out = handler(self.interp, op, [host(a.t) for a in args], {})
+                return dev(out[0] if isinstance(out, (list, tuple)) else out)
         return self._new_slot(fill, True)
 
     def _concatenate(self, op, e, t):
@@ -414,10 +521,11 @@ class PairPlan:
         pos = 1 + _rest_pos(e, t, axis)
 
         def fill(ctx):
-            parts = [self._lead(s, ctx.slots[s].a, ctx.P) for s in ins]
+            import torch
+            parts = [self._lead(s, ctx.slots[s].t, ctx.P) for s in ins]
             lead = max(p.shape[0] for p in parts)
-            parts = [np.broadcast_to(p, (lead,) + p.shape[1:]) for p in parts]
-            return HostArray(np.concatenate(parts, axis=pos), ctx.slots[ins[0]].el)
+            parts = [p.expand((lead,) + tuple(p.shape[1:])) for p in parts]
+            return DevArray(torch.cat(parts, dim=pos), ctx.slots[ins[0]].el)
         return self._new_slot(fill, True)
 
     # -- shape ops
@@ -455,14 +563,14 @@ class PairPlan:
 
         def fill(ctx):
             h = ctx.slots[inner]
-            a = self._lead(inner, h.a, ctx.P)
+            a = self._lead(inner, h.t, ctx.P)
             index = [slice(None)] + [0 if s is None else slice(None) for s in spots]
             a = a[tuple(index)]
             view = [1] * len(out_rest)
             for s, extent in zip([s for s in spots if s is not None], a.shape[1:]):
                 view[s] = extent
             a = a.reshape([a.shape[0]] + view)
-            return HostArray(np.broadcast_to(a, [a.shape[0]] + out_rest), h.el)
+            return DevArray(a.expand([a.shape[0]] + out_rest), h.el)
         return self._new_slot(fill, True)
 
     def _transpose(self, op, e, t):
@@ -475,8 +583,8 @@ class PairPlan:
 
         def fill(ctx):
             h = ctx.slots[inner]
-            a = self._lead(inner, h.a, ctx.P)
-            return HostArray(np.transpose(a, [0] + [1 + i for i in order]), h.el)
+            a = self._lead(inner, h.t, ctx.P)
+            return DevArray(a.permute([0] + [1 + i for i in order]), h.el)
         return self._new_slot(fill, True)
 
     def _reshape(self, op, e, t):
@@ -490,8 +598,8 @@ class PairPlan:
 
         def fill(ctx):
             h = ctx.slots[inner]
-            a = self._lead(inner, h.a, ctx.P)
-            return HostArray(a.reshape([a.shape[0]] + out_rest), h.el)
+            a = self._lead(inner, h.t, ctx.P)
+            return DevArray(a.reshape([a.shape[0]] + out_rest), h.el)
         return self._new_slot(fill, True)
 
     def _slice(self, op, e, t):
@@ -506,8 +614,8 @@ class PairPlan:
 
         def fill(ctx):
             h = ctx.slots[inner]
-            a = self._lead(inner, h.a, ctx.P)
-            return HostArray(a[(slice(None),) + cut], h.el)
+            a = self._lead(inner, h.t, ctx.P)
+            return DevArray(a[(slice(None),) + cut], h.el)
         return self._new_slot(fill, True)
 
     # -- the per-expert products
@@ -604,24 +712,22 @@ class PairPlan:
                 dense = qmm.to_device(ctx.env[data])
                 dense = dense.permute([t_dim] + [d for d in row_axes + list(dcontract)])
                 x = dense.reshape(T, M, K)
-                lhs = ctx.tidx_dev
+                lhs = ctx.tidx32
             else:
-                h = ctx.slots[inner]
-                a = self._lead(inner, h.a, ctx.P)
-                a = np.broadcast_to(a, (ctx.P,) + a.shape[1:])
-                a = np.transpose(a, [0] + [1 + i for i in to_rows_k]).reshape(ctx.P, M, K)
-                x = qmm.to_device(HostArray(np.ascontiguousarray(a), h.el))
+                h = ctx.slots[inner]                 # the previous slot as it lies on the device
+                a = self._lead(inner, h.t, ctx.P)
+                a = a.expand((ctx.P,) + tuple(a.shape[1:]))
+                x = a.permute([0] + [1 + i for i in to_rows_k]).reshape(ctx.P, M, K)
                 lhs = None
             if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
                 x = x.to(qmm._torch_dtype(out_el))
             arrays = qmm.pack_arrays(ctx.interp, m)
-            y = emit_dot(x.contiguous(), arrays, m.mode, m.gs, m.bits, lhs, ctx.eidx_dev, E,
+            y = emit_dot(x.contiguous(), arrays, m.mode, m.gs, m.bits, lhs, ctx.eidx32, E,
                          out_dtype=qmm._torch_dtype(out_el), has_perm=m.has_perm)
-            y = host(y.reshape([ctx.P] + mshape + nshape))
-            a = y.a
+            y = y.reshape([ctx.P] + mshape + nshape)
             if order != sorted(order):
-                a = np.transpose(a, [0] + [1 + i for i in order])
-            return HostArray(a.reshape([ctx.P] + out_rest), out_el)
+                y = y.permute([0] + [1 + i for i in order])
+            return DevArray(y.reshape([ctx.P] + out_rest), out_el)
         return self._new_slot(fill, True)
 
     _rules = {"stablehlo.concatenate": _concatenate, "stablehlo.broadcast_in_dim": _broadcast,
@@ -630,7 +736,7 @@ class PairPlan:
 
 
 class _Run:
-    __slots__ = ("interp", "env", "slots", "P", "eidx", "tidx", "eidx_dev", "tidx_dev")
+    __slots__ = ("interp", "env", "slots", "P", "eidx_dev", "tidx_dev", "eidx32", "tidx32")
 
 
 class Dispatch:
@@ -640,28 +746,39 @@ class Dispatch:
     def __init__(self):
         self.disabled = False
         self.verified = not VERIFY
+        self._tidx = None
 
     def run(self, interp, env):
+        """The closure list on the device, then the routing-weighted sum over
+        each token's K pairs.  The only host data read are the router's indices
+        when the program computed them on the host (an upload, no copy back)."""
         import torch
+        from . import qmm
+        from .interpreter import HOST_COPIES
+        copies = HOST_COPIES[0]
         r, plan = self.router, self.plan
-        idx = host(env[r.indices]).a.reshape(-1).astype(np.int64)
         ctx = _Run()
         ctx.interp, ctx.env, ctx.P = interp, env, self.P
-        ctx.eidx = idx
-        ctx.tidx = np.repeat(np.arange(self.T, dtype=np.int64), self.K)
-        ctx.eidx_dev = torch.from_numpy(idx.astype(np.int32)).cuda()
-        ctx.tidx_dev = torch.from_numpy(ctx.tidx.astype(np.int32)).cuda()
+        iv = env[r.indices]
+        if hasattr(iv, "type_enum") and hasattr(iv, "data"):
+            iv = iv.data
+        if isinstance(iv, torch.Tensor):
+            ctx.eidx32 = iv.cuda().reshape(-1).to(torch.int32)
+        else:
+            ctx.eidx32 = torch.from_numpy(np.ascontiguousarray(host(iv).a.reshape(-1), np.int32)).cuda()
+        if self._tidx is None:                      # token of pair p: p // K, the same every call
+            t32 = torch.arange(self.T, dtype=torch.int32, device="cuda").repeat_interleave(self.K)
+            self._tidx = (t32, t32.long())
+        ctx.tidx32, ctx.tidx_dev = self._tidx
+        ctx.eidx_dev = ctx.eidx32.long()
         ctx.slots = []
         for fill in plan.program:
             ctx.slots.append(fill(ctx))
         out = ctx.slots[self.out_slot]
-        y = out.a
+        yd = out.t
         if not plan.paired[self.out_slot]:
-            y = y.reshape((1,) + y.shape)
-        y = np.broadcast_to(y, (self.P,) + y.shape[1:])
-        # the routing-weighted sum over each token's K pairs, on the device
-        from . import qmm
-        yd = qmm.to_device(HostArray(np.ascontiguousarray(y), out.el))
+            yd = yd.reshape((1,) + tuple(yd.shape))
+        yd = yd.expand((self.P,) + tuple(yd.shape[1:]))
         wd = qmm.to_device(env[r.weights]).reshape(self.T, self.K)
         if self.sum_el != out.el:
             yd = yd.to(qmm._torch_dtype(self.sum_el))         # the dense graph converts the products before summing
@@ -671,6 +788,7 @@ class Dispatch:
         if list(total.shape) != self.out_shape:
             raise RuntimeError(f"expert dispatch produced {list(total.shape)}, expected {self.out_shape}")
         STATS["dispatches"] += 1
+        STATS["host_copies"] += HOST_COPIES[0] - copies
         return [total.to(qmm._torch_dtype(self.out_el))]
 
 

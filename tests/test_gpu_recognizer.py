@@ -190,6 +190,46 @@ def test_mxfp4_experts_gathered(E, K, Tk):
     assert qmm.stats()["packs"] == 2 and moe.stats()["dispatches"] == 2
 
 
+def test_the_dispatch_runs_between_its_projections_on_the_device():
+    """The gpt-oss block at the model's own widths (hidden and intermediate size
+    2880, reference scripts/model_bench/mxfp4_gpt_oss.py:90-110; eight experts,
+    top-4, 16 tokens): the buffers are device-resident, and from the first
+    expert-indexed product to the routing-weighted sum nothing is copied back to
+    the host -- the second projection reads the first one's result where it
+    lies (reference moe.py:1283-1340, :1425-1461 run the closure list on device
+    arrays)."""
+    import stablehlo_text as S
+    moe.reset_stats()
+    E, K, Tk, H, Ii = 8, 4, 16, 2880, 2880
+    rng = np.random.default_rng(2880)
+    gu_c, gu_s, gu_ref = S.make_mxfp4_experts(2 * Ii, H, E, seed=51)
+    d_c, d_s, d_ref = S.make_mxfp4_experts(H, Ii, E, seed=52)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    wr = (rng.standard_normal((H, E)) / 8).astype(np.float32)
+    br = rng.standard_normal(E).astype(np.float32)
+    bgu = (rng.standard_normal((E, 2 * Ii)) / 8).astype(np.float32)
+    bd = (rng.standard_normal((E, H)) / 8).astype(np.float32)
+    text = S.moe_block_mxfp4(E, Tk, H, Ii, K)
+    f32, u8 = engine._ENUM["F32"], engine._ENUM["U8"]
+    bufs = [engine.buffer_from_host(a, f32 if a.dtype == np.float32 else u8, a.shape)
+            for a in (x, wr, br, gu_c, gu_s, d_c, d_s, bgu, bd)]
+    assert all(b.data.is_cuda for b in bufs)
+    ex = engine.compile_program(text)
+    (buf,) = engine.execute(ex, bufs)
+    st, qst = moe.stats(), qmm.stats()
+    assert st["recognized"] == 1 and st["verified"] == 1 and st["fallbacks"] == 0, st
+    assert st["gather_qmm"] == 2 and st["dispatches"] == 1, st
+    assert st["host_copies"] == 0, st                      # nothing came back between the projections
+    assert qst["mxfp4"] == 2 and qst["fallbacks"] == 0, qst
+    assert buf.data.is_cuda
+    got = buf.data.float().cpu().numpy()
+    want = S.moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd, K)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-4
+    (again,) = engine.execute(ex, bufs)                    # a decode step later: same packs, still no copy back
+    assert qmm.stats()["packs"] == 2 and moe.stats()["dispatches"] == 2 and moe.stats()["host_copies"] == 0
+    assert torch.equal(again.data, buf.data)
+
+
 def test_an_expert_nobody_selects_is_never_evaluated():
     """The one intended divergence from the dense block (reference
     tests/test_moe.py:428-458): an expert whose output is not finite and whose
