@@ -221,15 +221,26 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
   const int64_t wpr = (int64_t)a.K * BITS / 8;                  // bytes per weight row
   // float16 / float32 entries are split into two / three bf16 terms, exactly,
   // where they have to be matrix operands.
-  constexpr bool MX = GSHIFT == 2;
+  // GSHIFT = 7: MXFP4 whose K is any multiple of 64 up to one pass (the hidden
+  // size 2880 of gpt-oss: five and a half slices a row, 90 scale bytes a row):
+  // the last slice is ragged -- the code pieces and activation chunks past K are
+  // requested out of range and read as zeros -- and a tile's scale rows, which
+  // are not dword-aligned one by one, come in as the one contiguous run they
+  // are in memory and are picked apart by byte offset.
+  constexpr bool MXR = GSHIFT == 7;
+  constexpr bool MX = GSHIFT == 2 || MXR;
   constexpr bool F16T = GSHIFT == 3 || GSHIFT == 4;
-  constexpr bool F32T = GSHIFT >= 5;
+  constexpr bool F32T = GSHIFT == 5 || GSHIFT == 6;
+  static_assert(!MXR || XD == 1, "the ragged MXFP4 form is a one-pass direct variant");
   constexpr int ES = F32T ? 4 : 2;                             // bytes per table entry
   constexpr int GLOG = (GSHIFT == 1 || GSHIFT == 4 || GSHIFT == 6) ? 1 : 0;   // log2(group / 64)
   static_assert(!MX || (BITS == 4 && XD != 0), "MXFP4: four-bit codes, direct variants");
   const int64_t ng = MX ? (int64_t)(a.K / 64) : (int64_t)(a.K / 64) >> GLOG;   // table row = ng * ES bytes (MXFP4: K/32 bytes)
-  const int slices = a.K / KS;
+  const int slices = MXR ? (a.K + KS - 1) / KS : a.K / KS;
   const int passes = (slices + CW - 1) / CW;
+  const int tail_codes = MXR ? a.K % KS : 0;                   // codes of a ragged last slice (0: it is whole)
+  const int tailp = tail_codes / 32, tailc = tail_codes / 64;  // its 16-byte pieces | its 64-code chunks
+  const uint32_t spitch = (uint32_t)(ng * ES);                 // bytes of a table row
 
   int64_t xz = a.lhs_idx ? (int64_t)a.lhs_idx[bz] : bz;
   int64_t wz = a.rhs_idx ? (int64_t)a.rhs_idx[bz] : bz;
@@ -275,7 +286,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     // Load q of this wavefront is instruction j = lw + q*NL of the item: slice
     // j / 4, row quad j % 4 = (lw + o) % 4 with o = q*NL % 4 known at compile
     // time, so the lane offsets are kept per o.
-    uint32_t wv[4], xv[4];
+    uint32_t wv[4], xv[4], wvt[4];
     int wrow[4];
 #pragma unroll
     for (int o = 0; o < 4; ++o) {
@@ -284,6 +295,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       const uint32_t gp = (uint32_t)(lp ^ (row & 15));
       wrow[o] = row;
       wv[o] = (uint32_t)((n_begin + row) * wpr) + gp * 16;
+      wvt[o] = MXR && tailp != 0 && (int)gp >= tailp ? kOutOfRange : wv[o];   // in a ragged last slice
       xv[o] = row < a.M ? (uint32_t)((int64_t)row * a.K * 2) + gp * 16 : kOutOfRange;
     }
     const int trow = lane & 15, tsl = lane >> 4;  // table loads: lane = (slice within four, row)
@@ -295,10 +307,12 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
       // every load turns into a loop over its distinct values: a row past the
       // end is a lane offset out of range, a slice past the end both.)
       const bool full = n_begin + t * 16 + 16 <= n_end;                // uniform
-      uint32_t vt[4];
+      uint32_t vt[4], vtt[4];
 #pragma unroll
-      for (int o = 0; o < 4; ++o)
+      for (int o = 0; o < 4; ++o) {
         vt[o] = full || n_begin + t * 16 + wrow[o] < n_end ? wv[o] : kOutOfRange;
+        vtt[o] = full || n_begin + t * 16 + wrow[o] < n_end ? wvt[o] : kOutOfRange;
+      }
       const uint32_t tile_off = (uint32_t)(t * 16 * wpr);
       // The table rows go first (their sixteen quarter lines are the slow part
       // of a tile's requests; ahead of the codes they measured 0.1-0.2 us a
@@ -307,6 +321,16 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
       for (int q = 0; q < QT; ++q) {
         const int jt = lw + q * NL;               // uniform
+        if constexpr (MXR) {
+          // the tile's scale rows as the contiguous run they are: request jt covers its bytes [1024 jt, 1024 jt + 1024)
+          const int64_t n0t = n_begin + t * 16;
+          const int rows_here = n_end - n0t < 16 ? (int)(n_end - n0t) : 16;
+          const uint32_t off = (uint32_t)(jt * 1024 + lane * 16);
+          const uint32_t vo = rows_here > 0 && off < (uint32_t)rows_here * spitch ? (uint32_t)(n0t * spitch) + off
+                                                                                   : kOutOfRange;
+          dma16<kStream>(rs, tb + jt * 1024, vo, 0u);
+          continue;
+        }
         const int kind = jt / (NTAB / 2), rem = jt % (NTAB / 2);
         const int h = WIDE ? rem >> 1 : rem, h2 = WIDE ? rem & 1 : 0;   // four-slice group; 16-byte half of a wide row
         const int sloc = 4 * h + tsl;
@@ -330,7 +354,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const int sl = p * CW + sloc;
         const bool sok = sl < slices;             // uniform; false for passes past the last
         const uint32_t so = sok ? (uint32_t)sl * 256u + tile_off : 0u;
-        dma16<kStream>(rw, base + sloc * 4096 + rq * 1024, sok ? vt[o] : kOutOfRange, so);
+        const bool rag = MXR && sl == slices - 1;  // uniform
+        dma16<kStream>(rw, base + sloc * 4096 + rq * 1024, sok ? (rag ? vtt[o] : vt[o]) : kOutOfRange, so);
       });
     };
     // item `i` (compile-time kind) of pass `p` into ring slot `slot`
@@ -503,7 +528,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
     const int sw = XD == 1 ? (wave + (int)(blockIdx.x >> 3)) & (CW - 1) : wave;
     const uint32_t rowb = (uint32_t)(sw * 4096 + r * 256);      // this lane's row inside its slice's 4 KB
     // the operand row r of this lane is row xrow(r) of x (gathered in the grouped form)
-    const int tab_row = (sw >> 2) * (WIDE ? 2048 : 1024) + (sw & 3) * 256 + r * 16;   // this lane's table row inside a kind
+    const int tab_row = MXR ? 0 : (sw >> 2) * (WIDE ? 2048 : 1024) + (sw & 3) * 256 + r * 16;   // this lane's table row inside a kind
+    // chunks of this wavefront's slice that lie inside K (a ragged last slice has fewer)
+    const int vc = MXR && tailc != 0 && sw == slices - 1 ? tailc : CPS;
     const int64_t xrows = src_row ? (int64_t)a.x_rows : (int64_t)a.M;
     const auto rxc = make_rsrc(a.x + xz * a.M * (int64_t)a.K, x_ok ? xrows * a.K * 2 : 0);
     auto xrow = [&](int m) -> int64_t {
@@ -573,13 +600,25 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         // by the 32-block's power-of-two scale (exact in bf16), so the chunks
         // chain straight through the MFMA accumulator.  Lane kg holds codes
         // [16 kg, 16 kg + 16) of the chunk: block 2c + kg/2 of the slice.
-        const u32x4 sv = *reinterpret_cast<const u32x4*>(tb);
+        u32x4 sv;
+        if constexpr (MXR) {
+          // this row's sixteen scale bytes of the slice, at an even byte offset of the tile's run
+          const uint32_t off = (uint32_t)r * spitch + 16u * (uint32_t)sw;
+          const uint32_t* pw = reinterpret_cast<const uint32_t*>(tb + (off & ~3u));
+          const uint32_t d0 = pw[0], d1 = pw[1], d2 = pw[2], d3 = pw[3], d4 = pw[4];
+          const uint32_t sh = (off & 2u) * 8u;
+          sv = u32x4{__builtin_amdgcn_alignbit(d1, d0, sh), __builtin_amdgcn_alignbit(d2, d1, sh),
+                     __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh)};
+        } else {
+          sv = *reinterpret_cast<const u32x4*>(tb);
+        }
         f32x4 at = acc_in;
 #pragma unroll
         for (int c = 0; c < CPS; ++c) {
           const uint32_t pc = (uint32_t)(2 * c + (kg >> 1));
           const u32x2 q = *reinterpret_cast<const u32x2*>(base + ((pc ^ swz) << 4) + (kg & 1) * 8);
-          const float sc = e8m0_to_f32((sv[c >> 1] >> (16 * (c & 1) + 8 * (kg >> 1))) & 255u);
+          float sc = e8m0_to_f32((sv[c >> 1] >> (16 * (c & 1) + 8 * (kg >> 1))) & 255u);
+          if constexpr (MXR) sc = c < vc ? sc : 1.0f;        // past K: zero codes times a finite scale
           at = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][0], widen_e2m1(q[0], sc), at, 0, 0, 0);
           at = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[c][1], widen_e2m1(q[1], sc), at, 0, 0, 0);
         }
@@ -698,7 +737,7 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
 #pragma unroll
           for (int j = 0; j < 2; ++j)
             raw[c][j] = __builtin_amdgcn_raw_buffer_load_b128(
-                rxc, active ? lane_off + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
+                rxc, active && (!MXR || c < vc) ? lane_off + (uint32_t)(c * 128 + j * 16) : kOutOfRange, so, 0);
 #pragma unroll
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
@@ -747,7 +786,8 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         for (int c = 0; c < CPS; ++c)
 #pragma unroll
           for (int h = 0; h < 2; ++h)
-            raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo[h], so + (uint32_t)(((c + ROT) % CPS) * 128), 0);
+            raw[c][h] = __builtin_amdgcn_raw_buffer_load_b128(
+                rxc, !MXR || (c + ROT) % CPS < vc ? lo[h] : kOutOfRange, so + (uint32_t)(((c + ROT) % CPS) * 128), 0);
         const uint32_t wr = (uint32_t)(srow * 128 + ((sp ^ ((srow >> 1) & 3)) << 4));
         const uint32_t rkey = (uint32_t)((r >> 1) & 3);
         const bool upper = r >= 8;
@@ -803,7 +843,9 @@ __global__ __launch_bounds__(kWave*(CW + NL)) void skinny2_kernel(GemvArgs a, in
         const uint32_t so = active ? (uint32_t)(sw * KS) * 2u : 0u;
         u32x4 raw[NI];
 #pragma unroll
-        for (int i = 0; i < NI; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(rxc, lo, so + (uint32_t)(i * W), 0);
+        for (int i = 0; i < NI; ++i)
+          raw[i] = __builtin_amdgcn_raw_buffer_load_b128(
+              rxc, !MXR || i * CPI + (sp >> 3) < vc ? lo : kOutOfRange, so + (uint32_t)(i * W), 0);
         const uint32_t wr = (uint32_t)(srow * W + ((sp ^ key(srow)) << 4));
         const int rr = r % R;
         const uint32_t rd = (uint32_t)(rr * W), rkey = (uint32_t)key(rr);
@@ -992,6 +1034,9 @@ void launch_k(const GemvArgs& a, int64_t batch, int rows_per_wg, hipStream_t st,
   if constexpr (BITS == 4 && XD != 0) {
     if (a.gshift == 2) return launch_one<BITS, CW, NL, TMAX, 2, XD>(a, batch, rows_per_wg, st, chunks);
   }
+  if constexpr (BITS == 4 && XD == 1) {
+    if (a.gshift == 7) return launch_one<BITS, CW, NL, TMAX, 7, XD>(a, batch, rows_per_wg, st, chunks);
+  }
   switch (a.gshift) {
     case 1: return launch_one<BITS, CW, NL, TMAX, 1, XD>(a, batch, rows_per_wg, st, chunks);
     case 3: return launch_one<BITS, CW, NL, TMAX, 3, XD>(a, batch, rows_per_wg, st, chunks);
@@ -1134,10 +1179,13 @@ bool skinny_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
 // leave at once; an empty workgroup still costs about a microsecond of a
 // compute unit, which is why the grid is not expert x chunk).
 bool skinny2_mx_supported(int64_t N, int64_t K, const void* s);
+static int64_t mx_rows_per_wg(int64_t N, int64_t K, int64_t products);
 
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E) {
-  if (mode == QMM_MODE_MXFP4) return K / 512 >= 8 && skinny2_mx_supported(N, K, s);
+  // (MXFP4 whose K is no whole number of slices has no other staged kernel to go to: its ragged
+  // one-pass form takes the grouped decode from three slices on)
+  if (mode == QMM_MODE_MXFP4) return (K / 512 >= 8 || K % 512 != 0) && skinny2_mx_supported(N, K, s);
   if (!skinny_supported(N, K, gs, bits, mode, QMM_BF16, s, b)) return false;   // bf16, float16 and float32 tables alike
   return K * bits / 8 / 256 >= 8;
 }
@@ -1155,7 +1203,8 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   a.b = b;
   a.y = y;
   a.M = 1; a.N = (int)N; a.K = (int)K;
-  a.gshift = mode == QMM_MODE_MXFP4 ? 2 : (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : tab == QMM_F32 ? 5 : 0);
+  a.gshift = mode == QMM_MODE_MXFP4 ? (K % 512 ? 7 : 2)
+                                    : (gs == 128 ? 1 : 0) + (tab == QMM_F16 ? 3 : tab == QMM_F32 ? 5 : 0);
   a.y_dtype = y_dtype;
   a.lhs_idx = nullptr;
   a.rhs_idx = nullptr;
@@ -1167,6 +1216,7 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
   const int64_t rounds = ceil_div(ceil_div(N, cus), (int64_t)128);
   int64_t rows = ceil_div(N, cus * rounds);
   if (rows < 16) rows = 16;
+  if (mode == QMM_MODE_MXFP4) rows = mx_rows_per_wg(N, K, P < E ? P : E);
   const int64_t segs = skinny2_max_segments(P, E);
   if (K * bits / 8 / 256 <= 8) {
     if (bits == 4) launch_k<4, 8, 4, 4, 1>(a, segs, (int)rows, st);
@@ -1184,19 +1234,34 @@ void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const
 // fetched as 16-byte runs).
 bool skinny2_mx_supported(int64_t N, int64_t K, const void* s) {
   static const bool off = experiment_env("QMM_NO_SKINNY_MX") != nullptr;
-  if (off || K % 512 || K / 512 < 3) return false;
-  if (reinterpret_cast<uintptr_t>(s) & 3u) return false;
-  return N * (K / 2) < 0x7FFFFFFFll;                          // 32-bit lane offsets
+  if (off || N * (K / 2) >= 0x7FFFFFFFll) return false;       // 32-bit lane offsets
+  if (K % 512 == 0) return K / 512 >= 3 && (reinterpret_cast<uintptr_t>(s) & 3u) == 0;
+  // the ragged one-pass form: K any multiple of 64 between three and eight slices, a tile's
+  // scale rows a 16-byte-aligned run (every expert's table a multiple of 16 bytes, rows dealt by eights)
+  return K % 64 == 0 && K > 1024 && K < 4096 && (N * (K / 32)) % 16 == 0 &&
+         (reinterpret_cast<uintptr_t>(s) & 15u) == 0;
+}
+
+// Rows a workgroup for the MXFP4 decode: `products` decode products run side by side (batch entries,
+// the segments of a grouped product), so each gets its share of the compute units -- a workgroup's
+// fixed cost (its first tile lands about 3.5 us after it starts) is then paid once a compute unit, not
+// once per product.  For the ragged form a multiple of eight (see above).
+static int64_t mx_rows_per_wg(int64_t N, int64_t K, int64_t products) {
+  const int64_t cus = device_cus();
+  if (products < 1) products = 1;
+  const int64_t wgs = products >= cus ? 1 : cus / products;      // workgroups a product
+  int64_t rows = ceil_div(N, wgs);
+  if (rows > 128) rows = ceil_div(N, ceil_div(N, (int64_t)128));
+  if (rows < 16) rows = 16;
+  if (K % 512) rows = ceil_div(rows, (int64_t)8) * 8;
+  return rows;
 }
 
 void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st) {
   GemvArgs a = a0;
-  a.gshift = 2;
-  const int64_t cus = device_cus();
-  const int64_t rounds = ceil_div(ceil_div((int64_t)a.N, cus), (int64_t)128);
-  int64_t rows = ceil_div((int64_t)a.N, cus * rounds);
-  if (rows < 16) rows = 16;
-  if (a.K / 512 <= 8) launch_k<4, 8, 4, 4, 1>(a, batch, (int)rows, st);
+  a.gshift = a.K % 512 ? 7 : 2;
+  const int64_t rows = mx_rows_per_wg(a.N, a.K, batch);
+  if (a.K <= 4096) launch_k<4, 8, 4, 4, 1>(a, batch, (int)rows, st);
   else launch_k<4, 8, 4, 8, 2>(a, batch, (int)rows, st);
 }
 

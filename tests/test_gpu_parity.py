@@ -248,6 +248,74 @@ def test_decode_mxfp4_big_weights_on_the_loader_wavefront_kernel(m, n, k):
     np.testing.assert_array_equal(y16, O.round_bf16(y32))
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (1, 5760, 2880),      # gpt-oss gate / up projection: five and a half slices, 90 scale bytes a row
+    (2, 2880, 2880),      # its down projection
+    (4, 5760, 2880),      # whole-line activation loads, four rows an instruction
+    (7, 2880, 2880),      # ... eight rows an instruction
+    (16, 5760, 2880),     # staged through the patches
+    (16, 2880, 2880),
+    (3, 1016, 1088),      # two slices and a piece; the weight's last tile is ragged too
+    (9, 520, 3520),       # six slices and seven eighths
+    (1, 4104, 4032),      # one 64-code chunk short of eight slices
+    (5, 136, 1600),
+])
+def test_decode_mxfp4_ragged_k_on_the_loader_wavefront_kernel(m, n, k):
+    """MXFP4 decode whose K is no whole number of 512-code slices (reference
+    scripts/model_bench/mxfp4_gpt_oss.py:90-110: hidden size 2880): the last
+    slice's pieces and chunks past K read as zeros, the scale rows (K / 32
+    bytes, not dword-aligned one by one) are picked out of the tile's
+    contiguous run.  Exact products, float32 accumulate: as the whole-slice form."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, lo=100, hi=150)
+    x, xd = make_x(rng, m, k)
+    want = O.qmm(x, words, sb, None, 32, 4, "mxfp4")
+    y32 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4",
+                                     out_dtype=torch.float32))
+    assert O.rel_l2(y32, want) <= 2e-5, O.rel_l2(y32, want)
+    y16 = out_f32(K.quantized_matmul(xd, wd, sd, None, group_size=32, bits=4, mode="mxfp4"))
+    np.testing.assert_array_equal(y16, O.round_bf16(y32))
+
+
+def test_decode_mxfp4_ragged_k_batched_next_to_non_finite_neighbours():
+    """The ragged form reads nothing past K: a batch entry's activations end
+    where the next entry's begin, and those are infinite here; scale byte 255
+    (NaN) in the neighbouring rows' tables must not leak in either."""
+    rng = np.random.default_rng(77)
+    e, n, k, m = 3, 264, 2880, 2
+    codes, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+    x = O.round_bf16(rng.standard_normal((e, m, k)).astype(np.float32))
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    want = [O.qmm(x[z], words[z], sb[z], None, 32, 4, "mxfp4") for z in range(e)]
+    # entry 1 becomes poison for its neighbours: infinite activations, NaN scales
+    x[1] = np.inf
+    xd = bf16_dev(O.f32_to_bf16_bits(x))
+    sb2 = sb.copy()
+    sb2[1] = 255
+    y = out_f32(K.quantized_matmul(xd, wd, torch.from_numpy(sb2).to(DEV), None, group_size=32, bits=4,
+                                   mode="mxfp4", out_dtype=torch.float32))
+    for z in (0, 2):
+        assert np.isfinite(y[z]).all() and O.rel_l2(y[z], want[z]) <= 2e-5
+
+
+@pytest.mark.parametrize("t,topk,e,n", [(1, 4, 32, 5760), (4, 4, 32, 2880), (16, 4, 32, 5760), (16, 2, 5, 264)])
+def test_gather_qmm_grouped_decode_mxfp4_ragged_k(t, topk, e, n):
+    """gpt-oss expert projections (32 MXFP4 experts, top-4, K = 2880) as the
+    expert-indexed product: pairs sorted by expert, an expert's weight streamed
+    once for up to sixteen of its pairs, on the ragged form of the
+    loader-wavefront kernel."""
+    rng = np.random.default_rng(t * 100 + n)
+    k = 2880
+    _, words, sb, wd, sd = make_mxfp4(rng, n, k, lead=(e,))
+    x, xd = make_x(rng, t, k)
+    rhs = np.stack([rng.choice(e, size=topk, replace=False) for _ in range(t)]).reshape(-1).astype(np.int32)
+    lhs = np.repeat(np.arange(t, dtype=np.int32), topk)
+    want = O.gather_qmm(x[:, None, :], words, sb, None, lhs, rhs, 32, 4, "mxfp4")[:, 0]
+    y = out_f32(K.gather_qmm(xd, wd, sd, None, torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV),
+                             group_size=32, bits=4, mode="mxfp4", out_dtype=torch.float32))
+    assert O.rel_l2(y, want) <= 2e-5, O.rel_l2(y, want)
+
+
 def test_decode_mxfp4_big_weights_batched_with_extreme_scales():
     rng = np.random.default_rng(404)
     e, n, k, m = 2, 1500, 4096, 3
