@@ -51,7 +51,12 @@ def run_rotating(make_call, n_sets, steps, warmup):
     Returns (milliseconds, launches timed)."""
     import torch
     calls = [make_call(i) for i in range(n_sets)]
+    # The operands were produced on the default stream and the launches below run on a stream of their
+    # own: everything queued so far (the weight sets' fills, the routing indices) has to be finished
+    # first, or the first launches read buffers that are still being written.
+    torch.cuda.synchronize()
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
         for i in range(max(warmup, 1)):
             calls[i % n_sets].launch()
@@ -416,6 +421,8 @@ def main():
             "int8 g64 [14336,4096] M=4": bench_decode_random(4, 14336, 4096, bits=8),
             "int4 g64 [37888,3584] M=4": bench_decode_random(4, 37888, 3584),
             "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
+            "mxfp4 [5760,2880] M=1 (K no whole number of slices)": bench_decode_random(1, 5760, 2880, mode="mxfp4"),
+            "mxfp4 [5760,2880] M=16": bench_decode_random(16, 5760, 2880, mode="mxfp4"),
         }
         out["moe_decode"] = {f"8 experts int4 g64 [14336,4096], top-2, {t} token(s)": bench_moe_decode(t) for t in (1, 16)}
         out["engine_execute_C2"] = bench_engine_execute(2, 16)

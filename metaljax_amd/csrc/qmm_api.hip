@@ -180,6 +180,9 @@ __global__ __launch_bounds__(1024) void route_kernel(const int32_t* __restrict__
     const int e = rhs_idx[p];
     if (e < 0 || e >= E) continue;
     const int pos = atomicAdd(&cursor[e], 1);
+    // (the indices are read twice, to count and to place: were the caller to change them meanwhile, a
+    // slot past the expert's counted range would run into the next array -- such a pair is dropped)
+    if (pos >= row_offsets[e + 1]) continue;
     src_row[pos] = lhs_idx ? lhs_idx[p] : p;
     out_row[pos] = p;
   }

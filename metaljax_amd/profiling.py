@@ -73,6 +73,7 @@ def stream_probe(nbytes: int = 32 << 20, reps: int = 400):
     sink = torch.zeros(4096, dtype=torch.int32, device="cuda")
 
     def timed(launch):
+        torch.cuda.synchronize()            # the buffers were filled on the default stream
         stream = torch.cuda.Stream()
         with torch.cuda.stream(stream):
             st = stream.cuda_stream
