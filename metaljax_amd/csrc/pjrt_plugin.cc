@@ -28,6 +28,7 @@
 #include <atomic>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <string>
 #include <utility>
 #include <vector>
@@ -144,7 +145,11 @@ void ensure_python() {
 }  // namespace
 
 // ----------------------------------------------------------------- objects --
+// (An event's state is read and written under its own mutex: a client may set
+// an event it created on one thread while another asks whether it is ready.
+// Callbacks run after the lock is released.)
 struct PJRT_Event {
+  std::mutex mu;
   bool ready = true;
   PJRT_Error_Code code = PJRT_Error_Code_OK;
   std::string text;
@@ -243,8 +248,9 @@ struct PJRT_Buffer {
   PJRT_Buffer_Type type = PJRT_Buffer_Type_INVALID;
   std::vector<int64_t> dims, minor_to_major;
   size_t nbytes = 0;
-  int external_refs = 0;
-  bool deleted = false;
+  // touched by entry points that do not take the interpreter lock
+  std::atomic<int> external_refs{0};
+  std::atomic<bool> deleted{false};
 };
 
 struct PJRT_ExecuteContext {};
@@ -364,7 +370,11 @@ PJRT_Error* PluginAttributes(PJRT_Plugin_Attributes_Args* a) {
   // asks for it before serialising a module
   static int64_t current[3] = {1, 0, 0}, minimum[3] = {0, 9, 0};
   static PJRT_NamedValue attrs[2];
-  static const bool made = [] {               // once, whichever thread asks first
+  static std::once_flag once;
+  // A thread that arrives holding the interpreter lock lets go of it while it
+  // waits for the one that initialises (which needs that lock), and takes it back after.
+  PyThreadState* released = Py_IsInitialized() && PyGILState_Check() ? PyEval_SaveThread() : nullptr;
+  std::call_once(once, [] {                   // once, whichever thread asks first
     ensure_python();
     Gil g;
     if (PyObject* mod = PyImport_ImportModule("metaljax_amd.engine")) {
@@ -388,9 +398,8 @@ PJRT_Error* PluginAttributes(PJRT_Plugin_Attributes_Args* a) {
       attrs[i].int64_array_value = values[i];
       attrs[i].value_size = 3;
     }
-    return true;
-  }();
-  (void)made;
+  });
+  if (released) PyEval_RestoreThread(released);
   a->attributes = attrs;
   a->num_attributes = 2;
   return nullptr;
@@ -405,19 +414,32 @@ PJRT_Error* EventDestroy(PJRT_Event_Destroy_Args* a) {
   return nullptr;
 }
 PJRT_Error* EventIsReady(PJRT_Event_IsReady_Args* a) {
+  std::lock_guard<std::mutex> lock(a->event->mu);
   a->is_ready = a->event->ready;
   return nullptr;
 }
-PJRT_Error* EventError(PJRT_Event_Error_Args* a) { return event_error(a->event); }
+PJRT_Error* EventError(PJRT_Event_Error_Args* a) {
+  std::lock_guard<std::mutex> lock(a->event->mu);
+  return event_error(a->event);
+}
 PJRT_Error* EventAwait(PJRT_Event_Await_Args* a) {
   // nothing runs behind the caller's back: an event that is not ready is one
   // the caller created and has not set
+  std::lock_guard<std::mutex> lock(a->event->mu);
   REQUIRE(a->event->ready, "PJRT_Event_Await on an event nobody has set");
   return event_error(a->event);
 }
 PJRT_Error* EventOnReady(PJRT_Event_OnReady_Args* a) {
-  if (a->event->ready) a->callback(event_error(a->event), a->user_arg);
-  else a->event->waiting.emplace_back(a->callback, a->user_arg);
+  PJRT_Error* now = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(a->event->mu);
+    if (!a->event->ready) {
+      a->event->waiting.emplace_back(a->callback, a->user_arg);
+      return nullptr;
+    }
+    now = event_error(a->event);
+  }
+  a->callback(now, a->user_arg);
   return nullptr;
 }
 PJRT_Error* EventCreate(PJRT_Event_Create_Args* a) {
@@ -427,13 +449,23 @@ PJRT_Error* EventCreate(PJRT_Event_Create_Args* a) {
 }
 PJRT_Error* EventSet(PJRT_Event_Set_Args* a) {
   PJRT_Event* e = a->event;
-  REQUIRE(!e->ready, "PJRT_Event_Set on an event that is already set");
-  e->code = a->error_code;
-  if (a->error_message) e->text.assign(a->error_message, a->error_message_size);
-  e->ready = true;
-  auto waiting = std::move(e->waiting);
-  e->waiting.clear();
-  for (auto& w : waiting) w.first(event_error(e), w.second);
+  std::vector<std::pair<PJRT_Event_OnReadyCallback, void*>> waiting;
+  {
+    std::lock_guard<std::mutex> lock(e->mu);
+    REQUIRE(!e->ready, "PJRT_Event_Set on an event that is already set");
+    e->code = a->error_code;
+    if (a->error_message) e->text.assign(a->error_message, a->error_message_size);
+    e->ready = true;
+    waiting.swap(e->waiting);
+  }
+  for (auto& w : waiting) {
+    PJRT_Error* err = nullptr;
+    {
+      std::lock_guard<std::mutex> lock(e->mu);
+      err = event_error(e);
+    }
+    w.first(err, w.second);
+  }
   return nullptr;
 }
 
@@ -900,7 +932,9 @@ PJRT_Error* LoadedExecute(PJRT_LoadedExecutable_Execute_Args* a) {
   for (int64_t d : p->donated) {
     if (d < 0 || (size_t)d >= a->num_args) continue;
     bool keep = false;
-    if (a->options)
+    // (a caller built against an older header passes a shorter options struct)
+    if (a->options &&
+        a->options->struct_size >= PJRT_STRUCT_SIZE(PJRT_ExecuteOptions, num_non_donatable_input_indices))
       for (size_t k = 0; k < a->options->num_non_donatable_input_indices; ++k)
         keep = keep || a->options->non_donatable_input_indices[k] == d;
     if (keep) continue;

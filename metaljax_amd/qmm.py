@@ -135,6 +135,20 @@ def _kernel_limits(m):
         raise Reject("the weight exceeds the kernels' index range")
 
 
+def _device_failure(err) -> bool:
+    """Is this exception the device failing (a HIP error reported by the
+    library, a torch accelerator error) rather than a weight that does not
+    verify or pack?  Such an error must reach the caller: disabling the match
+    would run the program literally and hide it."""
+    from ._lib import QmmError
+    if isinstance(err, QmmError) and getattr(err, "code", 0) == 5:
+        return True
+    name = type(err).__name__
+    if name in ("AcceleratorError", "OutOfMemoryError"):
+        return True
+    return isinstance(err, RuntimeError) and ("HIP error" in str(err) or "CUDA error" in str(err))
+
+
 def prologue(interp, args) -> bool:
     """Make sure every live match has a pack for exactly these argument
     buffers (packing eagerly what is new) and lay the packed arrays out in
@@ -156,6 +170,8 @@ def prologue(interp, args) -> bool:
         except QmmLibraryError:
             raise                               # a missing library is an error, not a fallback
         except Exception as why:
+            if _device_failure(why):
+                raise                           # a failing device is an error too: the literal chain would hide it
             m.disabled = rewrite_changed = True
             STATS["fallbacks"] += 1
             _debug(f"{m.name} falls back to the literal chain ({why})")

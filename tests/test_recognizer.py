@@ -678,6 +678,32 @@ def test_emit_fails_loudly_without_a_gpu():
     assert not isinstance(e.value, I.UnsupportedOp)
 
 
+def test_a_device_failure_while_packing_is_not_a_fallback(monkeypatch):
+    """A weight that does not verify disables its match (the program runs
+    literally, reference qmm.py:2348-2355); the device failing while a pack is
+    built is not that: a HIP error from the library, or a torch accelerator
+    error, reaches the caller instead of being hidden behind the literal chain."""
+    from metaljax_amd import _lib, packs
+    k, n, m = 128, 64, 2
+    q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 64, seed=8)
+    args = host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32))
+
+    def boom(err):
+        def pack_for(*a, **kw):
+            raise err
+        return pack_for
+    for err in (_lib.QmmError(5, "hipErrorIllegalAddress"), RuntimeError("HIP error: an illegal memory access")):
+        ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+        monkeypatch.setattr(packs, "pack_for", boom(err))
+        with pytest.raises(type(err)):
+            qmm.prologue(ex.interp, args)
+        assert not ex.interp._qmm.matches[0].disabled
+    # an ordinary failure still falls back
+    ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+    monkeypatch.setattr(packs, "pack_for", boom(ValueError("does not verify")))
+    assert qmm.prologue(ex.interp, args) is True and ex.interp._qmm.matches[0].disabled
+
+
 # ------------------------------------------------------- engine surface ----
 
 def test_engine_surface_is_what_the_pjrt_plugin_calls_by_name():
