@@ -110,7 +110,9 @@ int qmm_gather_qmm(const void* x, int x_dtype, const void* w, const void* scales
  * QMM_ERR_WORKSPACE and launches nothing.  The call allocates and frees
  * nothing.  Every call on a GPU uses that GPU's one array: calls that overlap
  * on one GPU (different streams, or threads) race; calls in stream order do
- * not, and each call initialises what it reads. */
+ * not, and each call initialises what it reads.  The first call on a device
+ * looks up the array's address and sets kernel attributes: make it outside a
+ * stream capture (any call, of any size); later calls only launch kernels. */
 #define QMM_STATIC_SCRATCH_BYTES (16u << 20)
 int qmm_gather_qmm_static(const void* x, int x_dtype, const void* w, const void* scales,
                           const void* biases, int table_dtype, void* y, int y_dtype,

@@ -90,6 +90,38 @@ def test_static_scratch_calls_match_the_workspace_entry_point_call_after_call():
         assert allocated <= 2 * (got.numel() * 4 + got16.numel() * 2) + (1 << 20)
 
 
+def test_static_entry_takes_no_device_memory():
+    """Free device memory, as the driver reports it, does not shrink over calls
+    of the static entry point: torch's allocator cannot see a hipMalloc made
+    inside the library, hipMemGetInfo can.  The outputs are allocated up front
+    and one call is made before measuring, because the first call on a device
+    looks up the scratch array's address and sets kernel attributes (that call
+    belongs outside a stream capture; the later ones are capture-safe)."""
+    lib = _lib.load()
+    rng = np.random.default_rng(11)
+    c = _case(rng, 6, 200, 512, 400, 800, "affine")      # prefill kernels: the largest scratch use here
+    d = c["dev"]
+    ys = [torch.empty((c["p"], c["n"]), dtype=torch.float32, device=DEV) for _ in range(3)]
+    st = torch.cuda.current_stream().cuda_stream
+
+    def launch(y):
+        rc = lib.qmm_gather_qmm_static(d["x"].data_ptr(), _lib.BF16, d["w"].data_ptr(), d["s"].data_ptr(),
+                                       d["b"].data_ptr(), _lib.BF16, y.data_ptr(), _lib.F32, d["lhs"].data_ptr(),
+                                       d["rhs"].data_ptr(), c["p"], c["t"], c["e"], c["n"], c["k"], c["gs"], 4, 0, st)
+        _lib.check(rc)
+    launch(ys[0])
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for y in ys:
+        launch(y)
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    need = int(lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"], _lib.BF16))
+    assert need > (1 << 19)                               # the product does use scratch ...
+    assert free_before - free_after < (1 << 18), (free_before, free_after)      # ... and none of it was allocated
+    assert torch.equal(ys[0], ys[1]) and torch.equal(ys[1], ys[2])
+
+
 def test_static_scratch_limit_is_an_error_and_launches_nothing():
     lib = _lib.load()
     rng = np.random.default_rng(7)
