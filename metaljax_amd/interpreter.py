@@ -104,13 +104,37 @@ def from_numpy(a, el=None) -> HostArray:
     return settle(a, el)
 
 
-# Host copies of device tensors, one per tensor object while it lives: a
-# program argument that several literal ops (or several pack builds) read is
-# copied back once.  Engine buffers and fused results are never written in
-# place, which is what makes the copy reusable.
+# Host copies of device tensors, one per tensor object while it lives and is
+# not written: a program argument that several literal ops (or several pack
+# builds) read is copied back once.  An entry holds the tensor's version
+# counter, which torch bumps on every in-place write (through any view), so a
+# caller that refills a buffer between calls gets a fresh copy.  (Writes torch
+# cannot see -- a kernel handed the raw pointer -- would go unnoticed: the
+# fused calls here only ever write into tensors they have just allocated.)
 _MIRRORS = {}
 MIRROR_MAX_BYTES = 16 << 20     # larger tensors (weights) are copied back whenever read: no second copy is kept
 HOST_COPIES = [0]               # device -> host copies made (tests count them)
+
+
+def _version(v):
+    try:
+        return v._version
+    except RuntimeError:            # an inference-mode tensor keeps no counter: never mirrored
+        return None
+
+
+def _mirror_get(v):
+    hit = _MIRRORS.get(id(v))
+    if hit is not None and hit[0]() is v and hit[2] == _version(v):
+        return hit[1]
+    return None
+
+
+def _mirror_put(v, h):
+    import weakref
+    key, version = id(v), _version(v)
+    if version is not None:
+        _MIRRORS[key] = (weakref.ref(v, lambda _, key=key: _MIRRORS.pop(key, None)), h, version)
 
 
 def host(v) -> HostArray:
@@ -121,10 +145,9 @@ def host(v) -> HostArray:
         return host(v.data)
     import torch
     if isinstance(v, torch.Tensor):
-        key = id(v)
-        hit = _MIRRORS.get(key)
-        if hit is not None and hit[0]() is v:
-            return hit[1]
+        hit = _mirror_get(v)
+        if hit is not None:
+            return hit
         if v.is_cuda:
             HOST_COPIES[0] += 1
         if v.dtype == torch.bfloat16:
@@ -132,8 +155,7 @@ def host(v) -> HostArray:
         else:
             h = from_numpy(v.cpu().numpy())
         if v.is_cuda and v.numel() * v.element_size() <= MIRROR_MAX_BYTES:
-            import weakref
-            _MIRRORS[key] = (weakref.ref(v, lambda _, key=key: _MIRRORS.pop(key, None)), h)
+            _mirror_put(v, h)
         return h
     return from_numpy(v)
 

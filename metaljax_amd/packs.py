@@ -434,12 +434,26 @@ class WeightRows:
 
 # ------------------------------------------------------------------ packs ----
 
+def _stamp(buf):
+    """What moves when a source buffer is rewritten in place: torch's version
+    counter of a tensor (bumped by every in-place write, through any view).
+    The reference's buffers are immutable arrays, for which identity says it
+    all; a tensor is not.  Host arrays have no such counter (None): they are
+    taken as not rewritten, which is the reference's own assumption."""
+    try:
+        return buf._version
+    except (AttributeError, RuntimeError):
+        return None
+
+
 class Pack:
     """The packed arrays of one weight and weak references to the buffers they
-    were built from (reference qmm.py:629-664)."""
+    were built from (reference qmm.py:629-664), with each buffer's write stamp
+    at that time."""
 
     def __init__(self, leaves, w, scales, biases, perm, gs, bits, mode="affine"):
         self.sources = [weakref.ref(buf) for buf in leaves]
+        self.stamps = [_stamp(buf) for buf in leaves]
         self.w, self.scales, self.biases, self.perm = w, scales, biases, perm
         self.gs, self.bits, self.mode = gs, bits, mode
         self.blocked = False
@@ -451,7 +465,7 @@ class Pack:
 
     def matches(self, leaves) -> bool:
         return len(leaves) == len(self.sources) and all(
-            ref() is buf for ref, buf in zip(self.sources, leaves))
+            ref() is buf and st == _stamp(buf) for ref, st, buf in zip(self.sources, self.stamps, leaves))
 
     def alias(self, leaves):
         """The same arrays for another set of source buffers."""
@@ -842,16 +856,17 @@ def _cached_build(key, keyleaves):
     hit = _BUILT.get(key)
     if hit is None:
         return None
-    refs, pref = hit
+    refs, stamps, pref = hit
     pk = pref()
-    if pk is None or len(refs) != len(keyleaves) or not all(r() is a for r, a in zip(refs, keyleaves)):
+    if pk is None or len(refs) != len(keyleaves) or not all(
+            r() is a and st == _stamp(a) for r, st, a in zip(refs, stamps, keyleaves)):
         _BUILT.pop(key, None)
         return None
     return pk
 
 
 def _remember_build(key, keyleaves, pk):
-    _BUILT[key] = ([weakref.ref(a) for a in keyleaves], weakref.ref(pk))
+    _BUILT[key] = ([weakref.ref(a) for a in keyleaves], [_stamp(a) for a in keyleaves], weakref.ref(pk))
 
 
 def pack_for(interp, m, args, check=lambda m: None):

@@ -130,3 +130,27 @@ def test_unknown_op_is_reported():
     }"""
     with pytest.raises(I.UnsupportedOp):
         run(text, np.zeros(2, np.float32))
+
+
+def test_a_kept_host_copy_is_dropped_when_the_tensor_is_written_in_place():
+    """The interpreter keeps one host copy per device tensor; a caller that
+    refills the tensor between calls (also through a view) must not meet the
+    old copy, and a dead tensor's entry goes with it."""
+    import gc
+    import torch
+    t = torch.arange(6, dtype=torch.float32)
+    h = I.from_numpy(t.numpy().copy())
+    I._mirror_put(t, h)
+    assert I._mirror_get(t) is h
+    assert I._mirror_get(t.clone()) is None                 # another tensor object, same values
+    t.view(2, 3)[1, 1] = 9.0                                # written through a view: the counter is shared
+    assert I._mirror_get(t) is None
+    I._mirror_put(t, h)
+    t.add_(1)
+    assert I._mirror_get(t) is None
+    I._mirror_put(t, h)
+    key = id(t)
+    assert key in I._MIRRORS
+    del t
+    gc.collect()
+    assert key not in I._MIRRORS

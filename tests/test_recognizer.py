@@ -463,6 +463,32 @@ def test_packs_are_keyed_by_buffer_identity_and_repack_storms_give_up(monkeypatc
     assert ex.interp._qmm.matches[0].disabled and qmm.stats()["fallbacks"] == 1
 
 
+def test_a_weight_tensor_rewritten_in_place_is_packed_again():
+    """The reference's buffers are immutable, so a buffer's identity names its
+    contents; a tensor can be refilled.  Packs (and the cross-executable build
+    cache) also hold each source tensor's write counter."""
+    import torch
+    k, n, m = 128, 64, 2
+    q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 64, seed=8)
+    _, packed2, _, _, _, _ = T.quantize(k, n, 64, seed=9)
+    host_args = host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32))
+    wt = torch.from_numpy(packed.copy())
+    args = [wt] + host_args[1:]
+    ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+    qmm.prologue(ex.interp, args)
+    qmm.prologue(ex.interp, args)
+    assert qmm.stats()["packs"] == 1
+    first = ex.interp._qmm.matches[0].packs[0]
+    wt.copy_(torch.from_numpy(packed2))                     # the same tensor object, other codes
+    qmm.prologue(ex.interp, args)
+    assert qmm.stats()["packs"] == 2 and qmm.stats()["build_hits"] == 0
+    second = ex.interp._qmm.matches[0].packs[0]
+    assert second is not first and not np.array_equal(np.asarray(second.w), np.asarray(first.w))
+    ex2 = engine.compile_program(T.dense_sub(k, n, 2, m))   # another executable: the build cache's entry is the new one
+    qmm.prologue(ex2.interp, args)
+    assert qmm.stats()["build_hits"] == 1 and ex2.interp._qmm.matches[0].packs[0].w is second.w
+
+
 def test_build_cache_serves_a_second_executable_over_the_same_buffers():
     k, n, m = 128, 64, 2
     q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 64, seed=8)
