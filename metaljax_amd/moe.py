@@ -100,6 +100,7 @@ class DevArray:
 _TORCH_EL = {"i1": "bool", "i8": "int8", "i16": "int16", "i32": "int32", "i64": "int64", "ui8": "uint8",
              "f16": "float16", "bf16": "bfloat16", "f32": "float32", "f64": "float64"}
 _FLOATS = ("f16", "bf16", "f32", "f64")
+_WRAPPING_INTS = ("i8", "i16", "i32", "i64", "ui8")
 
 
 class _HostOnly(Exception):
@@ -124,7 +125,7 @@ def dev(v) -> DevArray:
         el = {getattr(torch, name): e for e, name in _TORCH_EL.items()}.get(v.dtype)
         if el is None:
             raise _HostOnly(str(v.dtype))
-        return DevArray(v if v.is_cuda else v.cuda(), el)
+        return DevArray(qmm.to_device(v), el)
     h = host(v)
     if h.el not in _TORCH_EL:
         raise _HostOnly(h.el)
@@ -149,7 +150,14 @@ def _dev_elementwise(op, args, out_el):
     logic = {"and": torch.bitwise_and, "or": torch.bitwise_or, "xor": torch.bitwise_xor}
     if name in binary and fl:
         return binary[name](t[0], t[1])
+    if name == "sign" and fl:
+        return torch.where(torch.isnan(t[0]), t[0], torch.sign(t[0]))      # torch's sign of a NaN is 0
     if name in unary and fl:
+        return unary[name](t[0])
+    ints = all(a.el in _WRAPPING_INTS for a in args)
+    if ints and name in ("add", "subtract", "multiply", "maximum", "minimum"):
+        return binary[name](t[0], t[1])                                    # two's-complement wrap, as numpy's
+    if ints and name in ("abs", "negate", "sign") and not args[0].el.startswith("ui"):
         return unary[name](t[0])
     if name in logic and not fl:
         return logic[name](t[0], t[1])
@@ -763,11 +771,11 @@ class Dispatch:
         if hasattr(iv, "type_enum") and hasattr(iv, "data"):
             iv = iv.data
         if isinstance(iv, torch.Tensor):
-            ctx.eidx32 = iv.cuda().reshape(-1).to(torch.int32)
+            ctx.eidx32 = qmm.to_device(iv).reshape(-1).to(torch.int32)
         else:
-            ctx.eidx32 = torch.from_numpy(np.ascontiguousarray(host(iv).a.reshape(-1), np.int32)).cuda()
+            ctx.eidx32 = torch.from_numpy(np.ascontiguousarray(host(iv).a.reshape(-1), np.int32)).to(qmm.DEVICE)
         if self._tidx is None:                      # token of pair p: p // K, the same every call
-            t32 = torch.arange(self.T, dtype=torch.int32, device="cuda").repeat_interleave(self.K)
+            t32 = torch.arange(self.T, dtype=torch.int32, device=qmm.DEVICE).repeat_interleave(self.K)
             self._tidx = (t32, t32.long())
         ctx.tidx32, ctx.tidx_dev = self._tidx
         ctx.eidx_dev = ctx.eidx32.long()

@@ -250,19 +250,25 @@ def _torch_dtype(el):
     return {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[el]
 
 
+# Where the tensors of the fused calls and of a running expert dispatch live.
+# The kernels take nothing else; the dispatch's tensor program between its
+# kernel calls is plain torch, which is how its tests run it without a GPU.
+DEVICE = "cuda"
+
+
 def to_device(v):
     """A runtime value as a device tensor (bf16 HostArrays become bfloat16)."""
     import torch
     if isinstance(v, torch.Tensor):
-        return v if v.is_cuda else v.cuda()
+        return v if v.device.type == DEVICE else v.to(DEVICE)
     h = host(v)
     if h.el == "bf16":
         bits = packing.f32_to_bf16_bits(h.a).view(np.int16)
-        return torch.from_numpy(np.ascontiguousarray(bits)).cuda().view(torch.bfloat16)
+        return torch.from_numpy(np.ascontiguousarray(bits)).to(DEVICE).view(torch.bfloat16)
     a = np.ascontiguousarray(h.a)
     if not a.flags.writeable:                   # torch refuses to wrap read-only storage without a warning
         a = a.copy()
-    return torch.from_numpy(a).cuda()
+    return torch.from_numpy(a).to(DEVICE)
 
 
 def emit(interp, m, env):

@@ -1008,6 +1008,84 @@ def test_dense_moe_block_is_planned_over_pairs(composite):
     assert qmm.stats()["mxfp4"] == 2 and qmm.stats()["packs"] == 2
 
 
+def _oracle_expert_product(calls):
+    """A stand-in for moe.emit_dot on host tensors: the per-pair products by the
+    oracle (the kernel's place in a dispatch that runs on torch CPU tensors)."""
+    import torch
+    from oracle import qmm_oracle as O
+
+    def product(x, arrays, mode, gs, bits, tidx, eidx, experts, out_dtype=None, has_perm=False):
+        from metaljax_amd import moe
+        assert not has_perm and isinstance(x, torch.Tensor) and x.device.type == "cpu" and x.is_contiguous()
+        biases = arrays[2] if mode == "affine" else None
+        w, scales = moe.split_experts([np.asarray(arrays[0]), np.asarray(arrays[1])], experts)
+        pairs = int(eidx.numel())
+        lhs = np.arange(pairs) if tidx is None else tidx.numpy()
+        assert x.shape[0] == (pairs if tidx is None else x.shape[0])
+        y = O.gather_qmm(x.float().numpy(), w, scales, biases, lhs, eidx.numpy(), gs, bits, mode)
+        calls.append((tuple(x.shape), tidx is None))
+        return torch.from_numpy(y).to(out_dtype or torch.float32)
+    return product
+
+
+@pytest.mark.parametrize("composite", [False, True])
+def test_the_dispatchs_tensor_program_gives_the_dense_blocks_result(composite, monkeypatch):
+    """Everything a planned dispatch does around its two expert products --
+    gathers on the way in, the bias adds, the gated activation's slices,
+    clamps and products, the hand-over from the first product to the second,
+    the routing-weighted sum -- on torch CPU tensors, the products themselves
+    by the oracle: equal to the dense block run literally and to its numpy
+    restatement (reference tests/test_moe.py:500-557 checks the same block
+    end to end)."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    calls = []
+    monkeypatch.setattr(qmm, "DEVICE", "cpu")
+    monkeypatch.setattr(moe, "emit_dot", _oracle_expert_product(calls))
+    E, Tk, H, Ii, K = 4, 5, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K, composite=composite)
+    raw, (gu_ref, d_ref) = _moe_inputs(E, Tk, H, Ii)
+    args = [I.from_numpy(a) for a in raw]
+    ex = engine.compile_program(text)
+    (buf,) = engine.execute(ex, args)
+    st = moe.stats()
+    assert st["recognized"] == 1 and st["dispatches"] == 1 and st["fallbacks"] == 0, st
+    # the first product reads the tokens' rows through the pairs' token numbers, the second one pair rows
+    assert calls == [((Tk, 1, H), False), ((Tk * K, 1, Ii), True)]
+    got = I.host(buf.data).a
+    x, wr, br, _, _, _, _, bgu, bd = raw
+    want = T.moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd, K)
+    np.testing.assert_allclose(got, want, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+    qmm_was = qmm.ENABLED
+    monkeypatch.setattr(qmm, "ENABLED", False)
+    (lit,) = engine.execute(engine.compile_program(text), args)
+    monkeypatch.setattr(qmm, "ENABLED", qmm_was)
+    np.testing.assert_allclose(got, I.host(lit.data).a, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+
+
+def test_the_dispatchs_tensor_program_in_bf16(monkeypatch):
+    """The same block with bf16 activations: every op between the products
+    rounds to bf16 as the literal path does (widened, computed in float32,
+    rounded once), so the two agree to the last bf16 place or two of the
+    result's scale (the expert products sum in another order)."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    monkeypatch.setattr(qmm, "DEVICE", "cpu")
+    monkeypatch.setattr(moe, "emit_dot", _oracle_expert_product([]))
+    E, Tk, H, Ii, K = 4, 5, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K, el="bf16")
+    raw, _ = _moe_inputs(E, Tk, H, Ii)
+    args = [I.from_numpy(a, "bf16") if a.dtype == np.float32 else I.from_numpy(a) for a in raw]
+    (buf,) = engine.execute(engine.compile_program(text), args)
+    assert moe.stats()["dispatches"] == 1 and moe.stats()["fallbacks"] == 0
+    got = I.host(buf.data)
+    assert got.el == "bf16"
+    monkeypatch.setattr(qmm, "ENABLED", False)
+    (lit,) = engine.execute(engine.compile_program(text), args)
+    lit = I.host(lit.data).a
+    assert np.abs(got.a - lit).max() <= 2.0 ** -6 * np.abs(lit).max()
+
+
 def test_a_router_that_is_not_a_top_k_scatter_is_refused():
     from metaljax_amd import moe
     E, Tk, H, Ii, K = 4, 3, 64, 32, 2
