@@ -44,6 +44,10 @@ from .recognize import Match
 QMM_ENABLED = os.environ.get("METALJAX_QMM", "1") != "0"
 ENABLED = QMM_ENABLED or os.environ.get("METALJAX_MOE", "1") != "0"
 _DEBUG = os.environ.get("METALJAX_DEBUG", "") == "1"
+# Row-blocked pack builds between two reclaims in `prologue` (a build that
+# evaluated its weight whole reclaims at once; reference qmm.py:165).
+GC_EVERY = int(os.environ.get("METALJAX_QMM_GC_EVERY", "8"))
+RECLAIMS = [0]                          # reclaims made (tests count them)
 _Reject = Reject
 
 
@@ -162,11 +166,23 @@ def prologue(interp, args) -> bool:
     from ._lib import QmmLibraryError
     rewrite_changed = False
     layout = []
+    built = since_reclaim = 0
     for m in st.matches:
         if m.disabled:
             continue
         try:
+            before = STATS["packs"]
             pk = packs.pack_for(interp, m, args, _kernel_limits)
+            if STATS["packs"] != before:
+                # A fresh build ran the weight's reconstruction at (a block
+                # of) its full size: what that left behind is given back
+                # before the next one adds to it, not after a prologue full of
+                # them (reference qmm.py:2326-2347).
+                built += 1
+                since_reclaim += 1
+                if not pk.blocked or since_reclaim >= GC_EVERY:
+                    since_reclaim = 0
+                    reclaim()
         except QmmLibraryError:
             raise                               # a missing library is an error, not a fallback
         except Exception as why:
@@ -192,7 +208,23 @@ def prologue(interp, args) -> bool:
         st.rebuild()
         interp.invalidate_plans()
     st.values = layout
+    if built:
+        reclaim()                               # also the tail of the blocked builds that skipped theirs
     return rewrite_changed
+
+
+def reclaim():
+    """Give back what pack builds leave behind: reference cycles among the
+    evaluation's dead float32 intermediates (host memory the reference counts
+    alone do not free), then the device blocks torch's allocator caches from
+    the uploads' staging (reference qmm.py:2345-2347, :2382-2386:
+    gc.collect() + mx.clear_cache())."""
+    import gc
+    gc.collect()
+    RECLAIMS[0] += 1
+    import torch
+    if torch.cuda.is_available() and torch.cuda.is_initialized():
+        torch.cuda.empty_cache()
 
 
 # --------------------------------------------------------------------------

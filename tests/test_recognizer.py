@@ -841,6 +841,68 @@ def test_blocked_affine_pack_is_bit_identical(monkeypatch):
     np.testing.assert_allclose(dequant_pack(pk), want, rtol=1e-6, atol=1e-7)
 
 
+def _three_grouped_weights(n, k, gs, t):
+    """y = x.W1^T + x.W2^T + x.W3^T, each weight as in T.affine_grouped."""
+    ng = k // gs
+    t3, q3, tab = f"tensor<{n}x{ng}x{gs}xbf16>", f"tensor<{n}x{ng}x{gs}xi8>", f"tensor<{n}x{ng}xbf16>"
+    nk, tn, tk = f"tensor<{n}x{k}xbf16>", f"tensor<{t}x{n}xbf16>", f"tensor<{t}x{k}xbf16>"
+    params, body = [], []
+    for i in (1, 2, 3):
+        params += [f"%q{i}: tensor<{n}x{k}xi8>", f"%scale{i}: tensor<{n}x{ng}xf32>", f"%zero{i}: tensor<{n}x{ng}xi8>"]
+        body.append(f"""
+    %qs{i} = stablehlo.reshape %q{i} : (tensor<{n}x{k}xi8>) -> {q3}
+    %qf{i} = stablehlo.convert %qs{i} : ({q3}) -> {t3}
+    %sc{i} = stablehlo.convert %scale{i} : (tensor<{n}x{ng}xf32>) -> {tab}
+    %sb{i} = stablehlo.broadcast_in_dim %sc{i}, dims = [0, 1] : ({tab}) -> {t3}
+    %zc{i} = stablehlo.convert %zero{i} : (tensor<{n}x{ng}xi8>) -> {tab}
+    %zb{i} = stablehlo.broadcast_in_dim %zc{i}, dims = [0, 1] : ({tab}) -> {t3}
+    %d{i} = stablehlo.subtract %qf{i}, %zb{i} : {t3}
+    %w3{i} = stablehlo.multiply %d{i}, %sb{i} : {t3}
+    %w{i} = stablehlo.reshape %w3{i} : ({t3}) -> {nk}
+    %y{i} = stablehlo.dot_general %x, %w{i}, contracting_dims = [1] x [1] : ({tk}, {nk}) -> {tn}""")
+    return f"""
+module @jit_three {{
+  func.func public @main({", ".join(params)}, %x: {tk}) -> {tn} {{{"".join(body)}
+    %s = stablehlo.add %y1, %y2 : {tn}
+    %out = stablehlo.add %s, %y3 : {tn}
+    return %out : {tn}
+  }}
+}}
+"""
+
+
+def test_pack_builds_reclaim_what_they_leave_behind(monkeypatch):
+    """A build that evaluated its weight whole reclaims at once, row-blocked
+    builds every METALJAX_QMM_GC_EVERY of them, a prologue that built anything
+    once more at its end, one that built nothing not at all (reference
+    qmm.py:165, :2326-2347, :2382-2386)."""
+    n, k, gs, t = 256, 128, 64, 3
+    text = _three_grouped_weights(n, k, gs, t)
+    data = [T.affine_grouped_data(n, k, gs, seed)[:3] for seed in (31, 32, 33)]
+    x = T.bf16_round(np.random.default_rng(34).standard_normal((t, k)).astype(np.float32) * 0.3)
+
+    def reclaims(block_elems, every):
+        qmm._BUILT.clear()
+        qmm.reset_stats()
+        monkeypatch.setattr(packs, "BLOCK_ELEMS", block_elems)
+        monkeypatch.setattr(qmm, "GC_EVERY", every)
+        ex = engine.compile_program(text)
+        args = [I.from_numpy(a.copy()) for three in data for a in three] + [I.from_numpy(x, "bf16")]
+        before = qmm.RECLAIMS[0]
+        qmm.prologue(ex.interp, args)
+        first = qmm.RECLAIMS[0] - before
+        qmm.prologue(ex.interp, args)                       # the same buffers: nothing built
+        blocked = [m.packs[0].blocked for m in ex.interp._qmm.matches]
+        assert qmm.stats()["packs"] == 3 and qmm.stats()["fallbacks"] == 0
+        assert qmm.RECLAIMS[0] - before == first
+        return first, blocked
+
+    assert reclaims(1 << 40, 8) == (4, [False] * 3)         # after each whole build, and at the end
+    assert reclaims(1 << 10, 8) == (1, [True] * 3)          # blocked builds wait for the end ...
+    assert reclaims(1 << 10, 1) == (4, [True] * 3)          # ... or for every one of them,
+    assert reclaims(1 << 10, 2) == (2, [True] * 3)          # or for every second
+
+
 def test_blocked_affine_falls_back_when_groups_interleave(monkeypatch):
     """Groups scattered along K: the permutation that gathers them is a
     property of the whole contraction axis, so the blocked pass gives up and
