@@ -16,6 +16,7 @@ void gemv_dispatch(const void* x, const void* w, const void* s, const void* b, i
 void gemv_geometry(int64_t M, int64_t N, int64_t K, int* t, int* waves);
 void skinny_geometry(int64_t N, int64_t K, int bits, int* waves, int* rows_per_wg);
 bool skinny2_plan(int64_t M, int64_t N, int64_t K, int bits, int* rows_per_wg);
+bool skinny2_mx_plan(int64_t N, int64_t K, int* rows_per_wg);
 bool skinny2_grouped_supported(int64_t N, int64_t K, int gs, int bits, int mode, int tab,
                                const void* s, const void* b, int64_t E);
 void skinny2_grouped_dispatch(const void* x, const void* w, const void* s, const void* b, void* y,
@@ -309,6 +310,17 @@ int qmm_plan(int64_t M, int64_t N, int64_t K, int group_size, int bits, int mode
     if (grid) *grid = g;
     if (block) *block = b;
     return QMM_OK;
+  }
+  if (M <= kGemvMaxM && mode == QMM_MODE_MXFP4) {
+    // the loader-wavefront kernel from three K-slices a row on, its ragged one-pass form for a K that
+    // is no whole number of slices
+    int rows;
+    if (skinny2_mx_plan(N, K, &rows)) {
+      if (kernel) *kernel = QMM_KERNEL_GEMV;
+      if (grid) *grid = (int)ceil_div(N, (int64_t)rows);
+      if (block) *block = 64 * 12;
+      return QMM_OK;
+    }
   }
   if (M <= kGemvMaxM && mode == QMM_MODE_AFFINE && (group_size == 64 || group_size == 128) &&
       (bits == 4 || bits == 8) && K % (2048 / bits) == 0) {

@@ -1257,6 +1257,14 @@ static int64_t mx_rows_per_wg(int64_t N, int64_t K, int64_t products) {
   return rows;
 }
 
+// For the plan query: whether a dense MXFP4 decode product of this shape runs here (tables taken as
+// aligned), and with how many rows a workgroup.
+bool skinny2_mx_plan(int64_t N, int64_t K, int* rows_per_wg) {
+  if (!skinny2_mx_supported(N, K, nullptr)) return false;
+  *rows_per_wg = (int)mx_rows_per_wg(N, K, 1);
+  return true;
+}
+
 void skinny2_mx_dispatch(const GemvArgs& a0, int64_t batch, hipStream_t st) {
   GemvArgs a = a0;
   a.gshift = a.K % 512 ? 7 : 2;

@@ -90,6 +90,34 @@ def test_plan_of_the_decode_variants(lib):
     assert b.value == 768
 
 
+def test_plan_of_the_mxfp4_kernels(lib):
+    """MXFP4 prefill: the eight-wavefront block-scaled kernel (512 threads, a
+    64 x 128 tile a workgroup) when K is a whole number of 2048-code stages,
+    the four-wavefront one for the other multiples of 512, the bf16 kernels
+    otherwise.  MXFP4 decode: the loader-wavefront kernel (768 threads) from
+    three 512-code slices a row on, for a K that is no whole number of slices
+    (gpt-oss: 2880) its one-pass form with rows dealt by eights."""
+    k, g, b = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.qmm_plan(256, 8192, 8192, 32, 4, 1, k, g, b) == 0
+    assert (k.value, g.value, b.value) == (_lib.KERNEL_MXFP4_MFMA, (8192 // 128) * (256 // 64), 512)
+    assert lib.qmm_plan(300, 260, 1536, 32, 4, 1, k, g, b) == 0
+    assert (k.value, b.value) == (_lib.KERNEL_MXFP4_MFMA, 256) and g.value == 16      # 3 x 5 tiles, dealt to eight XCDs
+    assert lib.qmm_plan(256, 5760, 2880, 32, 4, 1, k, g, b) == 0        # K % 512 != 0: the bf16 prefill kernel
+    assert k.value == _lib.KERNEL_GEMM
+    for m in (1, 16):
+        assert lib.qmm_plan(m, 5760, 2880, 32, 4, 1, k, g, b) == 0
+        rows = -(-5760 // g.value)
+        assert (k.value, b.value) == (_lib.KERNEL_GEMV, 768) and rows % 8 == 0 and 16 <= rows <= 128
+        assert lib.qmm_plan(m, 8192, 8192, 32, 4, 1, k, g, b) == 0
+        assert (k.value, b.value) == (_lib.KERNEL_GEMV, 768) and g.value == 256
+    assert lib.qmm_plan(4, 4096, 1024, 32, 4, 1, k, g, b) == 0          # two slices: the general decode kernel
+    assert k.value == _lib.KERNEL_GEMV and b.value < 768
+    assert lib.qmm_plan(4, 4096, 4160, 32, 4, 1, k, g, b) == 0          # ragged beyond eight slices: general again
+    assert b.value < 768
+    assert lib.qmm_plan(4, 100, 2880, 32, 4, 1, k, g, b) == 0           # an expert's scale table no multiple of 16 bytes
+    assert b.value < 768
+
+
 def test_gather_workspace_covers_the_grouped_decode(lib):
     """From four pairs up to sixteen an expert the workspace holds the expert
     sort and the segment list; below four pairs nothing is needed."""
