@@ -126,7 +126,7 @@ def _upload(arr: np.ndarray, el: str):
 def _resident(v, el):
     """A result value as what a Buffer of this engine holds: a device tensor
     when buffers are device-resident, the value itself otherwise."""
-    if not device_resident() or not isinstance(v, HostArray):
+    if not isinstance(v, HostArray) or not device_resident():       # (a fused result is a device tensor already)
         return v
     if el == "bf16":
         from .packing import f32_to_bf16_bits

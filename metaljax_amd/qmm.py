@@ -317,7 +317,11 @@ def emit(interp, m, env):
     x = to_device(env[m.lhs])
     if m.lperm != list(range(x.dim())):
         x = x.permute(m.lperm)
-    x = x.reshape([m.B, m.M, m.K] if m.bshape else [m.M, m.K]).contiguous()
+    flat = [m.B, m.M, m.K] if m.bshape else [m.M, m.K]
+    if list(x.shape) != flat:
+        x = x.reshape(flat)
+    if not x.is_contiguous():
+        x = x.contiguous()
     if m.has_perm:
         x = kernels.take_k(x, vals[-1])
     y = kernels.quantized_matmul(x, w, scales, biases, transpose=True, group_size=m.gs,
@@ -325,5 +329,7 @@ def emit(interp, m, env):
     if m.swapped:
         y = y.transpose(-1, -2).reshape(m.bshape + m.nshape + m.mshape)
     else:
-        y = y.reshape(m.bshape + m.mshape + m.nshape)
+        shape = m.bshape + m.mshape + m.nshape
+        if list(y.shape) != shape:
+            y = y.reshape(shape)
     return [y]
