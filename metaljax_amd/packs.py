@@ -40,8 +40,11 @@ from .recognize import OPAQUE_OPS, count, dims_of, outer_definition
 
 MAX_PACKS = int(os.environ.get("METALJAX_QMM_CACHE", "2"))
 MAX_REPACKS = int(os.environ.get("METALJAX_QMM_REPACKS", "8"))
-SHARE = os.environ.get("METALJAX_QMM_SHARE", "1") != "0"
-BUILD_CACHE = os.environ.get("METALJAX_QMM_BUILD_CACHE", "1") != "0"
+# Entries the two pack tables keep (0 turns the table off; reference qmm.py:1653, :2209-2211).
+# Entries are weak, so a full table is first swept of its dead ones and only then dropped whole --
+# coarse, and it only ever costs a repack.
+MAX_SHARED = int(os.environ.get("METALJAX_QMM_SHARE", "512"))
+MAX_BUILT = int(os.environ.get("METALJAX_QMM_BUILD_CACHE", "512"))
 # Weight elements evaluated per block (reference qmm.py:1259): the chain that
 # rebuilds a weight is several times wider than the weight.
 BLOCK_ELEMS = int(os.environ.get("METALJAX_QMM_BLOCK", str(1 << 24)))
@@ -727,7 +730,7 @@ def share(leaves, w, scales, biases, perm, gs, bits, mode) -> Pack:
     equal those of a live earlier pack shares that pack's arrays instead of
     uploading a copy (reference qmm.py:1656-1704)."""
     perm = None if perm is None else np.ascontiguousarray(perm, np.int32)
-    key = (mode, gs, bits, _digest([w, scales, biases, perm])) if SHARE else None
+    key = (mode, gs, bits, _digest([w, scales, biases, perm])) if MAX_SHARED > 0 else None
     if key is not None:
         ref = _SHARED.get(key)
         earlier = ref() if ref is not None else None
@@ -736,6 +739,11 @@ def share(leaves, w, scales, biases, perm, gs, bits, mode) -> Pack:
             return earlier.alias(leaves)
     pk = Pack(leaves, _upload(w), _upload(scales), _upload(biases), _upload(perm), gs, bits, mode)
     if key is not None:
+        if len(_SHARED) >= MAX_SHARED:
+            for dead in [k for k, ref in _SHARED.items() if ref() is None]:
+                del _SHARED[dead]
+            if len(_SHARED) >= MAX_SHARED:
+                _SHARED.clear()
         _SHARED[key] = weakref.ref(pk)
     return pk
 
@@ -842,7 +850,7 @@ def fingerprint(m, module=None):
 
 
 def _build_key(m, args, module=None):
-    if not BUILD_CACHE:
+    if MAX_BUILT <= 0:
         return None, None
     fp = fingerprint(m, module)
     if not fp:
@@ -866,6 +874,12 @@ def _cached_build(key, keyleaves):
 
 
 def _remember_build(key, keyleaves, pk):
+    if len(_BUILT) >= MAX_BUILT:
+        for dead in [k for k, (refs, _, pref) in _BUILT.items()
+                     if pref() is None or any(r() is None for r in refs)]:
+            del _BUILT[dead]
+        if len(_BUILT) >= MAX_BUILT:
+            _BUILT.clear()
     _BUILT[key] = ([weakref.ref(a) for a in keyleaves], [_stamp(a) for a in keyleaves], weakref.ref(pk))
 
 

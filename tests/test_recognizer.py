@@ -506,6 +506,44 @@ def test_build_cache_serves_a_second_executable_over_the_same_buffers():
     assert qmm.stats()["packs"] == 2 and qmm.stats()["build_hits"] == 1
 
 
+def test_pack_tables_are_bounded_and_zero_turns_them_off(monkeypatch):
+    """METALJAX_QMM_BUILD_CACHE / METALJAX_QMM_SHARE are entry counts (reference
+    qmm.py:1653, :2209-2211): 0 turns the table off, a full table is swept of
+    its dead entries and dropped whole if that does not make room."""
+    k, n, m = 128, 64, 2
+
+    def packed_executable(seed):
+        q, packed, scale, zero, g_idx, _ = T.quantize(k, n, 64, seed=seed)
+        args = host_args_dense(packed, scale, zero, g_idx, np.zeros((m, k), np.float32))
+        ex = engine.compile_program(T.dense_sub(k, n, 2, m))
+        qmm.prologue(ex.interp, args)
+        return ex, args
+
+    monkeypatch.setattr(packs, "MAX_BUILT", 0)
+    monkeypatch.setattr(packs, "MAX_SHARED", 0)
+    ex1, args = packed_executable(1)
+    ex2 = engine.compile_program(T.dense_sub(k, n, 2, m))
+    qmm.prologue(ex2.interp, args)                                   # same buffers, other executable: built again
+    ex3 = engine.compile_program(T.dense_sub(k, n, 2, m))
+    qmm.prologue(ex3.interp, [I.HostArray(np.array(a.a, copy=True), a.el) for a in args])      # same bytes: no sharing
+    st = qmm.stats()
+    assert (st["packs"], st["build_hits"], st["shared"]) == (3, 0, 0) and not qmm._BUILT and not qmm._SHARED
+    monkeypatch.setattr(packs, "MAX_BUILT", 2)
+    monkeypatch.setattr(packs, "MAX_SHARED", 2)
+    held = [packed_executable(seed) for seed in (2, 3)]
+    assert len(qmm._BUILT) == 2 and len(qmm._SHARED) == 2
+    del held[0]                                                       # its pack and buffers die: a dead entry
+    import gc
+    gc.collect()
+    held.append(packed_executable(4))                                 # full: the sweep makes room, the live entry stays
+    assert len(qmm._BUILT) == 2 and len(qmm._SHARED) == 2
+    ex5 = engine.compile_program(T.dense_sub(k, n, 2, m))
+    qmm.prologue(ex5.interp, held[0][1])
+    assert qmm.stats()["build_hits"] == 1                             # executable 3's entry survived the sweep
+    held.append(packed_executable(5))                                 # full of live entries: dropped whole
+    assert len(qmm._BUILT) == 1 and len(qmm._SHARED) == 1
+
+
 def test_different_weight_content_misses_the_build_cache():
     """Same shapes and types, different bytes in different buffers: the key
     names buffers by identity, so nothing is reused and each executable's pack
