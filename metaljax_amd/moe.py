@@ -50,11 +50,14 @@ from .interpreter import REGISTRY, HostArray, host, settle
 from .packing import Reject
 from .recognize import OPAQUE_OPS, count, dims_of, elem, op_key
 
-MOE_ENABLED = os.environ.get("METALJAX_MOE", "1") != "0"
+ENABLED = os.environ.get("METALJAX_MOE", "1") != "0"           # (reference moe.py:93; its tests flip it at run time)
 VERIFY = os.environ.get("METALJAX_MOE_VERIFY", "1") != "0"
 VERIFY_DRAWS = int(os.environ.get("METALJAX_MOE_VERIFY_DRAWS", "3"))
 _DEBUG = os.environ.get("METALJAX_DEBUG", "") == "1"
-STATS = {"recognized": 0, "verified": 0, "fallbacks": 0, "gather_qmm": 0, "dispatches": 0, "host_copies": 0}
+# The reference's keys (moe.py:100-101; "gather_mm", its float-weight product, stays 0 here: experts
+# whose weights are not quantized packs are left to the dense block) plus two of this package's own.
+STATS = {"recognized": 0, "verified": 0, "fallbacks": 0, "gather_qmm": 0, "gather_mm": 0,
+         "dispatches": 0, "host_copies": 0}
 
 
 def stats() -> dict:
@@ -800,6 +803,9 @@ class Dispatch:
         return [total.to(qmm._torch_dtype(self.out_el))]
 
 
+Match = Dispatch            # the reference's name for a gathered dispatch (moe.py; qmm.py:670)
+
+
 def plan_root(interp, qst, block, root) -> Dispatch:
     """`root` as the weighted sum over the experts of a dense dispatch."""
     e_axis = sum_axis(root)
@@ -891,7 +897,7 @@ def sweep_dead(block, skip, g):
 def plan_dispatches(interp, qst):
     """Every gatherable dispatch of the program (reference moe.py:1022-1090);
     the quantized-matmul matches they read are marked absorbed."""
-    if not MOE_ENABLED:
+    if not ENABLED:
         return []
     found = []
     for block in ir.walk_blocks(interp._main_block()):
@@ -916,6 +922,12 @@ def plan_dispatches(interp, qst):
     if kept:
         _debug(f"{len(kept)} expert dispatch(es) gathered ({', '.join(g.name for g in kept)})")
     return kept
+
+
+def analyze(interp, qst):
+    """The reference's entry point under its own name (moe.py:1016-1090): find
+    the gatherable dispatches and extend the recognizer's state with them."""
+    qst.moe = plan_dispatches(interp, qst)
 
 
 # ----------------------------------------------------------- verification ----

@@ -115,10 +115,10 @@ def analyze(interp) -> State:
     STATS["recognized"] += len(st.matches)
     if st.matches:
         _debug(f"{len(st.matches)} quantized matmul(s) recognized")
-    if os.environ.get("METALJAX_MOE", "1") != "0" and st.matches:
+    if st.matches:
         try:
             from . import moe
-            st.moe = moe.plan_dispatches(interp, st)
+            moe.analyze(interp, st)             # (nothing when moe.ENABLED is off)
         except Exception as e:                  # like the matcher: never fails the program
             _debug(f"expert-dispatch analysis failed ({e})")
             st.moe = []

@@ -1186,6 +1186,21 @@ def test_the_dispatchs_tensor_program_in_bf16(monkeypatch):
     assert np.abs(got.a - lit).max() <= 2.0 ** -6 * np.abs(lit).max()
 
 
+def test_expert_dispatch_disabled_by_its_flag(monkeypatch):
+    """METALJAX_MOE=0 (the reference's tests flip moe.ENABLED at run time,
+    tests/test_moe.py:406-417): the block stays dense, its quantized dots are
+    still fused one by one; the reference's names for the planner are there."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    monkeypatch.setattr(moe, "ENABLED", False)
+    st = qmm.analyze(engine.compile_program(T.moe_block_mxfp4(4, 3, 64, 32, 2)).interp)
+    assert st.moe == [] and len(st.matches) == 2 and not any(m.absorbed for m in st.matches)
+    assert moe.stats()["recognized"] == 0 and moe.stats()["gather_mm"] == 0
+    monkeypatch.setattr(moe, "ENABLED", True)
+    st = qmm.analyze(engine.compile_program(T.moe_block_mxfp4(4, 3, 64, 32, 2)).interp)
+    assert len(st.moe) == 1 and isinstance(st.moe[0], moe.Match) and callable(moe.analyze)
+
+
 def test_a_router_that_is_not_a_top_k_scatter_is_refused():
     from metaljax_amd import moe
     E, Tk, H, Ii, K = 4, 3, 64, 32, 2
