@@ -551,3 +551,107 @@ def moe_block_reference(x, wr, br, gu_ref, d_ref, bgu, bd, k):
     s = np.zeros_like(logits, dtype=np.float64)
     np.put_along_axis(s, order, w, -1)
     return np.einsum("eth,te->th", y, s)
+
+
+def moe_block_gemma4_mxfp4(E, T, H, I, K, el="f32"):
+    """keras-hub's Gemma4 router and expert block as the reference's test
+    writes them (reference tests/test_moe.py:192-240), the three expert
+    weights as MXFP4 checkpoints:
+
+        probs = softmax((x * rsqrt(mean(x^2) + 1e-6) * H^-0.5 * per_dim) @ proj)
+        vals, idx = top_k(probs);  w = vals / max(sum(vals), 1e-9);  S = sum_k one_hot(idx) * w
+        y = einsum("eti,ehi->eth", gelu_tanh(x.Wg^T) * (x.Wu^T), Wd) * escale[:, None, None]
+        out = sum_e y[e] * S[:, e]
+
+    What sets it apart from the gpt-oss block: three products, separate gate
+    and up weights, and a per-expert OUTPUT SCALE [E] reshaped to [E, 1, 1]
+    and broadcast over [E, T, H] -- at T = 1 the token axis it is broadcast
+    along is a unit axis on both sides."""
+    f = el
+    th, te, tk_, tke = _t((T, H), f), _t((T, E), f), _t((T, K), f), (T, K, E)
+    eti, eth, tei = _t((E, T, I), f), _t((E, T, H), f), _t((T, E, I), f)
+
+    def splat(name, value, shape):
+        return (f"    %{name}s = stablehlo.constant dense<{value}> : tensor<{f}>\n"
+                f"    %{name} = stablehlo.broadcast_in_dim %{name}s, dims = [] : (tensor<{f}>) -> {_t(shape, f)}\n")
+    return f"""
+module @jit_gemma4_block {{
+  func.func public @main(%x: {th}, %proj: {_t((H, E), f)}, %perdim: {_t((H,), f)}, %gc: {_t((E, I, H // 2), "ui8")}, %gs: {_t((E, I, H // 32), "ui8")}, %uc: {_t((E, I, H // 2), "ui8")}, %us: {_t((E, I, H // 32), "ui8")}, %dc: {_t((E, H, I // 2), "ui8")}, %ds: {_t((E, H, I // 32), "ui8")}, %escale: {_t((E,), f)}) -> {th} {{{_tagged_mxfp4_weight("g", "%gc", "%gs", (E,), I, H, f)}{_tagged_mxfp4_weight("u", "%uc", "%us", (E,), I, H, f)}{_tagged_mxfp4_weight("d", "%dc", "%ds", (E,), H, I, f)}
+    %zero = stablehlo.constant dense<0.000000e+00> : tensor<{f}>
+    %ninf = stablehlo.constant dense<0xFF800000> : tensor<{f}>
+    %xx = stablehlo.multiply %x, %x : {th}
+    %ss = stablehlo.reduce(%xx init: %zero) applies stablehlo.add across dimensions = [1] : ({th}, tensor<{f}>) -> {_t((T,), f)}
+{splat("invh", f"{1.0 / H:.8e}", (T,))}{splat("eps", "1.000000e-06", (T,))}    %ms = stablehlo.multiply %ss, %invh : {_t((T,), f)}
+    %mse = stablehlo.add %ms, %eps : {_t((T,), f)}
+    %rs = stablehlo.rsqrt %mse : {_t((T,), f)}
+    %rsb = stablehlo.broadcast_in_dim %rs, dims = [0] : ({_t((T,), f)}) -> {th}
+    %n0 = stablehlo.multiply %x, %rsb : {th}
+{splat("hs", f"{H ** -0.5:.8e}", (T, H))}    %n1 = stablehlo.multiply %n0, %hs : {th}
+    %pdb = stablehlo.broadcast_in_dim %perdim, dims = [1] : ({_t((H,), f)}) -> {th}
+    %n2 = stablehlo.multiply %n1, %pdb : {th}
+    %lg = stablehlo.dot_general %n2, %proj, contracting_dims = [1] x [0] : ({th}, {_t((H, E), f)}) -> {te}
+    %lmx = stablehlo.reduce(%lg init: %ninf) applies stablehlo.maximum across dimensions = [1] : ({te}, tensor<{f}>) -> {_t((T,), f)}
+    %lmxb = stablehlo.broadcast_in_dim %lmx, dims = [0] : ({_t((T,), f)}) -> {te}
+    %lsh = stablehlo.subtract %lg, %lmxb : {te}
+    %lex = stablehlo.exponential %lsh : {te}
+    %lsm = stablehlo.reduce(%lex init: %zero) applies stablehlo.add across dimensions = [1] : ({te}, tensor<{f}>) -> {_t((T,), f)}
+    %lsmb = stablehlo.broadcast_in_dim %lsm, dims = [0] : ({_t((T,), f)}) -> {te}
+    %probs = stablehlo.divide %lex, %lsmb : {te}
+    %vals, %idx = chlo.top_k(%probs, k = {K}) : {te} -> ({tk_}, {_t((T, K), "i32")})
+    %vs = stablehlo.reduce(%vals init: %zero) applies stablehlo.add across dimensions = [1] : ({tk_}, tensor<{f}>) -> {_t((T,), f)}
+{splat("tiny", "1.000000e-09", (T,))}    %vsm = stablehlo.maximum %vs, %tiny : {_t((T,), f)}
+    %vsb = stablehlo.broadcast_in_dim %vsm, dims = [0] : ({_t((T,), f)}) -> {tk_}
+    %w = stablehlo.divide %vals, %vsb : {tk_}
+    %idxb = stablehlo.broadcast_in_dim %idx, dims = [0, 1] : ({_t((T, K), "i32")}) -> {_t(tke, "i32")}
+    %io = stablehlo.iota dim = 2 : {_t(tke, "i32")}
+    %eq = stablehlo.compare EQ, %idxb, %io, SIGNED : ({_t(tke, "i32")}, {_t(tke, "i32")}) -> {_t(tke, "i1")}
+    %hot = stablehlo.convert %eq : ({_t(tke, "i1")}) -> {_t(tke, f)}
+    %wb = stablehlo.broadcast_in_dim %w, dims = [0, 1] : ({tk_}) -> {_t(tke, f)}
+    %hw = stablehlo.multiply %hot, %wb : {_t(tke, f)}
+    %s = stablehlo.reduce(%hw init: %zero) applies stablehlo.add across dimensions = [1] : ({_t(tke, f)}, tensor<{f}>) -> {te}
+    %g0 = stablehlo.dot_general %x, %wtg, contracting_dims = [1] x [2] : ({th}, {_t((E, I, H), f)}) -> {tei}
+    %g = stablehlo.transpose %g0, dims = [1, 0, 2] : ({tei}) -> {eti}
+    %u0 = stablehlo.dot_general %x, %wtu, contracting_dims = [1] x [2] : ({th}, {_t((E, I, H), f)}) -> {tei}
+    %u = stablehlo.transpose %u0, dims = [1, 0, 2] : ({tei}) -> {eti}
+{splat("c3", "4.471500e-02", (E, T, I))}{splat("c2", "7.978846e-01", (E, T, I))}{splat("one", "1.000000e+00", (E, T, I))}{splat("half", "5.000000e-01", (E, T, I))}    %g2 = stablehlo.multiply %g, %g : {eti}
+    %g3 = stablehlo.multiply %g2, %g : {eti}
+    %g3c = stablehlo.multiply %g3, %c3 : {eti}
+    %gin = stablehlo.add %g, %g3c : {eti}
+    %gsc = stablehlo.multiply %gin, %c2 : {eti}
+    %gth = stablehlo.tanh %gsc : {eti}
+    %g1p = stablehlo.add %gth, %one : {eti}
+    %gh = stablehlo.multiply %g, %half : {eti}
+    %gelu = stablehlo.multiply %gh, %g1p : {eti}
+    %act = stablehlo.multiply %gelu, %u : {eti}
+    %y0 = stablehlo.dot_general %act, %wtd, batching_dims = [0] x [0], contracting_dims = [2] x [2] : ({eti}, {_t((E, H, I), f)}) -> {eth}
+    %es3 = stablehlo.reshape %escale : ({_t((E,), f)}) -> {_t((E, 1, 1), f)}
+    %esb = stablehlo.broadcast_in_dim %es3, dims = [0, 1, 2] : ({_t((E, 1, 1), f)}) -> {eth}
+    %y = stablehlo.multiply %y0, %esb : {eth}
+    %st = stablehlo.transpose %s, dims = [1, 0] : ({te}) -> {_t((E, T), f)}
+    %sb = stablehlo.broadcast_in_dim %st, dims = [0, 1] : ({_t((E, T), f)}) -> {eth}
+    %ys = stablehlo.multiply %y, %sb : {eth}
+    %out = stablehlo.reduce(%ys init: %zero) applies stablehlo.add across dimensions = [0] : ({eth}, tensor<{f}>) -> {th}
+    return %out : {th}
+  }}
+}}
+"""
+
+
+def gemma4_block_reference(x, proj, per_dim, g_ref, u_ref, d_ref, escale, k):
+    """The Gemma4 block on exactly dequantized weights, in float64 numpy; the
+    selection itself from the float32 probabilities the graph would compare."""
+    x64, H = np.asarray(x, np.float64), x.shape[-1]
+    normed = x64 / np.sqrt(np.mean(x64 * x64, -1, keepdims=True) + 1e-6) * H ** -0.5 * np.asarray(per_dim, np.float64)
+    lg = normed @ np.asarray(proj, np.float64)
+    ex = np.exp(lg - lg.max(-1, keepdims=True))
+    probs = ex / ex.sum(-1, keepdims=True)
+    order = np.argsort(-probs.astype(np.float32), axis=-1, kind="stable")[:, :k]
+    vals = np.take_along_axis(probs, order, -1)
+    w = vals / np.maximum(vals.sum(-1, keepdims=True), 1e-9)
+    s = np.zeros_like(probs)
+    np.put_along_axis(s, order, w, -1)
+    g = np.einsum("th,eih->eti", x64, g_ref.astype(np.float64))
+    u = np.einsum("th,eih->eti", x64, u_ref.astype(np.float64))
+    gelu = 0.5 * g * (1.0 + np.tanh(0.7978846 * (g + 0.044715 * g ** 3)))
+    y = np.einsum("eti,ehi->eth", gelu * u, d_ref.astype(np.float64)) * np.asarray(escale, np.float64)[:, None, None]
+    return np.einsum("eth,te->th", y, s)

@@ -1186,6 +1186,48 @@ def test_the_dispatchs_tensor_program_in_bf16(monkeypatch):
     assert np.abs(got.a - lit).max() <= 2.0 ** -6 * np.abs(lit).max()
 
 
+@pytest.mark.parametrize("Tk", [1, 6])
+@pytest.mark.parametrize("E,K", [(4, 2), (8, 4)])
+def test_gemma4_block_is_gathered_also_at_one_token(E, K, Tk, monkeypatch):
+    """keras-hub's Gemma4 block (reference tests/test_moe.py:192-262) with
+    MXFP4 experts: a softmax -> top-k -> renormalise router, three expert
+    products, and a per-expert output scale [E] -> [E, 1, 1] broadcast over
+    [E, T, H].  At T = 1 (every decode step) that broadcast's token axis is a
+    unit axis on both sides and must be read as a broadcast, not as the token
+    axis.  The dispatch's tensor program runs on torch CPU tensors, the three
+    products by the oracle."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    calls = []
+    monkeypatch.setattr(qmm, "DEVICE", "cpu")
+    monkeypatch.setattr(moe, "emit_dot", _oracle_expert_product(calls))
+    H, Ii = 64, 32
+    rng = np.random.default_rng(Tk * 100 + E)
+    g_c, g_s, g_ref = T.make_mxfp4_experts(Ii, H, E, seed=E)
+    u_c, u_s, u_ref = T.make_mxfp4_experts(Ii, H, E, seed=E + 1)
+    d_c, d_s, d_ref = T.make_mxfp4_experts(H, Ii, E, seed=E + 2)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    proj = rng.standard_normal((H, E)).astype(np.float32)
+    per_dim = (1.0 + rng.standard_normal(H) / 8).astype(np.float32)
+    escale = (1.0 + rng.standard_normal(E) / 8).astype(np.float32)
+    text = T.moe_block_gemma4_mxfp4(E, Tk, H, Ii, K)
+    args = [I.from_numpy(a) for a in (x, proj, per_dim, g_c, g_s, u_c, u_s, d_c, d_s, escale)]
+    ex = engine.compile_program(text)
+    (buf,) = engine.execute(ex, args)
+    st = moe.stats()
+    assert st["recognized"] == 1 and st["verified"] == 1 and st["dispatches"] == 1 and st["fallbacks"] == 0, st
+    assert qmm.stats()["mxfp4"] == 3 and all(m.absorbed for m in ex.interp._qmm.matches)
+    # gate and up read the tokens' rows through the pairs' token numbers, down reads pair rows
+    assert sorted(calls) == sorted([((Tk, 1, H), False)] * 2 + [((Tk * K, 1, Ii), True)])
+    got = I.host(buf.data).a
+    assert got.shape == (Tk, H)
+    want = T.gemma4_block_reference(x, proj, per_dim, g_ref, u_ref, d_ref, escale, K)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5 * max(1.0, np.abs(want).max()))
+    monkeypatch.setattr(qmm, "ENABLED", False)
+    (lit,) = engine.execute(engine.compile_program(text), args)
+    np.testing.assert_allclose(got, I.host(lit.data).a, rtol=1e-4, atol=1e-5 * max(1.0, np.abs(want).max()))
+
+
 def test_expert_dispatch_disabled_by_its_flag(monkeypatch):
     """METALJAX_MOE=0 (the reference's tests flip moe.ENABLED at run time,
     tests/test_moe.py:406-417): the block stays dense, its quantized dots are
