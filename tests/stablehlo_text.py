@@ -571,6 +571,8 @@ def moe_block_gemma4_mxfp4(E, T, H, I, K, el="f32"):
     th, te, tk_, tke = _t((T, H), f), _t((T, E), f), _t((T, K), f), (T, K, E)
     eti, eth, tei = _t((E, T, I), f), _t((E, T, H), f), _t((T, E, I), f)
 
+    ninf = {"f32": "0xFF800000", "bf16": "0xFF80", "f16": "0xFC00"}[f]
+
     def splat(name, value, shape):
         return (f"    %{name}s = stablehlo.constant dense<{value}> : tensor<{f}>\n"
                 f"    %{name} = stablehlo.broadcast_in_dim %{name}s, dims = [] : (tensor<{f}>) -> {_t(shape, f)}\n")
@@ -578,7 +580,7 @@ def moe_block_gemma4_mxfp4(E, T, H, I, K, el="f32"):
 module @jit_gemma4_block {{
   func.func public @main(%x: {th}, %proj: {_t((H, E), f)}, %perdim: {_t((H,), f)}, %gc: {_t((E, I, H // 2), "ui8")}, %gs: {_t((E, I, H // 32), "ui8")}, %uc: {_t((E, I, H // 2), "ui8")}, %us: {_t((E, I, H // 32), "ui8")}, %dc: {_t((E, H, I // 2), "ui8")}, %ds: {_t((E, H, I // 32), "ui8")}, %escale: {_t((E,), f)}) -> {th} {{{_tagged_mxfp4_weight("g", "%gc", "%gs", (E,), I, H, f)}{_tagged_mxfp4_weight("u", "%uc", "%us", (E,), I, H, f)}{_tagged_mxfp4_weight("d", "%dc", "%ds", (E,), H, I, f)}
     %zero = stablehlo.constant dense<0.000000e+00> : tensor<{f}>
-    %ninf = stablehlo.constant dense<0xFF800000> : tensor<{f}>
+    %ninf = stablehlo.constant dense<{ninf}> : tensor<{f}>
     %xx = stablehlo.multiply %x, %x : {th}
     %ss = stablehlo.reduce(%xx init: %zero) applies stablehlo.add across dimensions = [1] : ({th}, tensor<{f}>) -> {_t((T,), f)}
 {splat("invh", f"{1.0 / H:.8e}", (T,))}{splat("eps", "1.000000e-06", (T,))}    %ms = stablehlo.multiply %ss, %invh : {_t((T,), f)}
@@ -655,3 +657,51 @@ def gemma4_block_reference(x, proj, per_dim, g_ref, u_ref, d_ref, escale, k):
     gelu = 0.5 * g * (1.0 + np.tanh(0.7978846 * (g + 0.044715 * g ** 3)))
     y = np.einsum("eti,ehi->eth", gelu * u, d_ref.astype(np.float64)) * np.asarray(escale, np.float64)[:, None, None]
     return np.einsum("eth,te->th", y, s)
+
+
+def moe_gemma4_decode_loop(E, T, H, I, K, steps, el="f32"):
+    """Prefill plus a decode step inside a while body, as a sampler emits it
+    (reference tests/test_moe.py:262-296): the Gemma4 block over [T, H], then
+    `steps` times over the [1, H] row the previous step produced, starting
+    from the prefill's last row.  The loop's closed-over weights arrive as
+    carries returned unchanged, which is how jax lowers them.  Returns both
+    results: ([T, H], [1, H])."""
+    import re
+    f = el
+
+    def body_of(text):
+        start = text.index("{", text.index("@main")) + 1
+        return text[start:text.index("    return %out")]
+
+    pre = body_of(moe_block_gemma4_mxfp4(E, T, H, I, K, el))
+    step = body_of(moe_block_gemma4_mxfp4(E, 1, H, I, K, el))
+    inputs = ["proj", "perdim", "gc", "gs", "uc", "us", "dc", "ds", "escale"]
+    carried = {"x": "tok", **{n: "c" + n for n in inputs}}
+    step = re.sub(r"%([A-Za-z_][A-Za-z0-9_]*)", lambda mo: "%" + carried.get(mo.group(1), mo.group(1) + "_b"), step)
+    types = {"proj": _t((H, E), f), "perdim": _t((H,), f), "gc": _t((E, I, H // 2), "ui8"),
+             "gs": _t((E, I, H // 32), "ui8"), "uc": _t((E, I, H // 2), "ui8"), "us": _t((E, I, H // 32), "ui8"),
+             "dc": _t((E, H, I // 2), "ui8"), "ds": _t((E, H, I // 32), "ui8"), "escale": _t((E,), f)}
+    th, one = _t((T, H), f), _t((1, H), f)
+    params = ", ".join([f"%x: {th}"] + [f"%{n}: {types[n]}" for n in inputs])
+    carries = ", ".join([f"%i = %i0", f"%tok = %last"] + [f"%c{n} = %{n}" for n in inputs])
+    ctypes_ = ", ".join(["tensor<i32>", one] + [types[n] for n in inputs])
+    back = ", ".join(["%ni", "%out_b"] + [f"%c{n}" for n in inputs])
+    return f"""
+module @jit_gemma4_generate {{
+  func.func public @main({params}) -> ({th}, {one}) {{{pre}
+    %last = stablehlo.slice %out [{T - 1}:{T}, 0:{H}] : ({th}) -> {one}
+    %i0 = stablehlo.constant dense<0> : tensor<i32>
+    %r:{2 + len(inputs)} = stablehlo.while({carries}) : {ctypes_}
+     cond {{
+      %lim = stablehlo.constant dense<{steps}> : tensor<i32>
+      %p = stablehlo.compare LT, %i, %lim, SIGNED : (tensor<i32>, tensor<i32>) -> tensor<i1>
+      stablehlo.return %p : tensor<i1>
+    }} do {{{step}
+      %onei = stablehlo.constant dense<1> : tensor<i32>
+      %ni = stablehlo.add %i, %onei : tensor<i32>
+      stablehlo.return {back} : {ctypes_}
+    }}
+    return %out, %r#1 : {th}, {one}
+  }}
+}}
+"""

@@ -1228,6 +1228,47 @@ def test_gemma4_block_is_gathered_also_at_one_token(E, K, Tk, monkeypatch):
     np.testing.assert_allclose(got, I.host(lit.data).a, rtol=1e-4, atol=1e-5 * max(1.0, np.abs(want).max()))
 
 
+@pytest.mark.parametrize("el", ["f32", "bf16"])
+def test_gemma4_prefill_and_a_decode_step_inside_a_while_body_are_both_gathered(el, monkeypatch):
+    """What a sampler emits (reference tests/test_moe.py:262-296): the block
+    over [T, H], then a loop whose body is the block over the [1, H] row of
+    the step before; the loop's weights are carries returned unchanged.  Both
+    dispatches are planned, verified and run; the six recognized weights are
+    three buffers, so three packs are built and the loop body's matches reuse
+    them."""
+    from metaljax_amd import moe
+    moe.reset_stats()
+    calls = []
+    monkeypatch.setattr(qmm, "DEVICE", "cpu")
+    monkeypatch.setattr(moe, "emit_dot", _oracle_expert_product(calls))
+    E, Tk, H, Ii, K, steps = 8, 5, 64, 32, 2, 3
+    rng = np.random.default_rng(57)
+    g_c, g_s, _ = T.make_mxfp4_experts(Ii, H, E, seed=58)
+    u_c, u_s, _ = T.make_mxfp4_experts(Ii, H, E, seed=59)
+    d_c, d_s, _ = T.make_mxfp4_experts(H, Ii, E, seed=60)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    proj = rng.standard_normal((H, E)).astype(np.float32)
+    per_dim = (1.0 + rng.standard_normal(H) / 8).astype(np.float32)
+    escale = (1.0 + rng.standard_normal(E) / 8).astype(np.float32)
+    text = T.moe_gemma4_decode_loop(E, Tk, H, Ii, K, steps, el=el)
+    args = [I.from_numpy(a, el) if a.dtype == np.float32 else I.from_numpy(a)
+            for a in (x, proj, per_dim, g_c, g_s, u_c, u_s, d_c, d_s, escale)]
+    ex = engine.compile_program(text)
+    pre, tok = engine.execute(ex, args)
+    st, qst = moe.stats(), qmm.stats()
+    assert st["recognized"] == 2 and st["verified"] == 2 and st["fallbacks"] == 0, st
+    assert st["dispatches"] == 1 + steps and len(calls) == 3 * (1 + steps)
+    assert qst["recognized"] == 6 and qst["fallbacks"] == 0 and qst["packs"] + qst["build_hits"] + qst["shared"] >= 3, qst
+    assert qst["packs"] - qst["shared"] == 3, qst            # three weights' worth of packed arrays, whoever built them
+    monkeypatch.setattr(qmm, "ENABLED", False)
+    lit_pre, lit_tok = engine.execute(engine.compile_program(text), args)
+    tol = 4e-2 if el == "bf16" else 1e-4
+    for got, want in ((pre, lit_pre), (tok, lit_tok)):
+        got, want = I.host(got.data).a, I.host(want.data).a
+        assert got.shape == want.shape
+        np.testing.assert_allclose(got, want, rtol=tol, atol=tol * max(1e-2, np.abs(want).max()))
+
+
 def test_expert_dispatch_disabled_by_its_flag(monkeypatch):
     """METALJAX_MOE=0 (the reference's tests flip moe.ENABLED at run time,
     tests/test_moe.py:406-417): the block stays dense, its quantized dots are
