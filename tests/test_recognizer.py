@@ -1401,6 +1401,87 @@ def test_a_dispatch_that_fails_its_check_runs_densely(monkeypatch):
     assert not any(m.absorbed for m in st.matches) and set(st.roots) == {m.key for m in st.matches}
 
 
+def test_scores_that_are_not_a_top_k_scatter_leave_the_block_dense():
+    """Scores masked by a threshold instead of scattered from a top-k
+    (reference tests/test_moe.py:340-352), and Gemma4's router with the top-k
+    taken out -- every expert weighted by its softmax probability
+    (tests/test_moe.py:355-372), at one token and at several: no dispatch, the
+    quantized products are still fused one by one."""
+    from metaljax_amd import moe
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    scores = f"%s = stablehlo.reduce(%hw init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<{Tk}x{K}x{E}xf32>, tensor<f32>) -> tensor<{Tk}x{E}xf32>"
+    assert scores in text
+    te, tei1 = f"tensor<{Tk}x{E}xf32>", f"tensor<{Tk}x{E}xi1>"
+    masked = text.replace(scores, f"""%thrs = stablehlo.constant dense<2.000000e-01> : tensor<f32>
+    %thr = stablehlo.broadcast_in_dim %thrs, dims = [] : (tensor<f32>) -> {te}
+    %zte = stablehlo.broadcast_in_dim %zero, dims = [] : (tensor<f32>) -> {te}
+    %pex = stablehlo.exponential %logits : {te}
+    %keep = stablehlo.compare GT, %pex, %thr, FLOAT : ({te}, {te}) -> {tei1}
+    %s = stablehlo.select %keep, %pex, %zte : {tei1}, {te}""")
+    moe.reset_stats()
+    st = qmm.analyze(engine.compile_program(masked).interp)
+    assert st.moe == [] and moe.stats()["recognized"] == 0 and len(st.roots) == 2
+    for tokens in (1, 6):
+        text = T.moe_block_gemma4_mxfp4(E, tokens, H, Ii, K)
+        scatter = text[text.index("    %vals, %idx = chlo.top_k"):text.index("    %g0 = stablehlo.dot_general")]
+        dense = text.replace(scatter, f"    %s = stablehlo.add %probs, %probs : tensor<{tokens}x{E}xf32>\n")
+        moe.reset_stats()
+        st = qmm.analyze(engine.compile_program(dense).interp)
+        assert st.moe == [] and moe.stats()["recognized"] == 0 and len(st.roots) == 3, tokens
+
+
+def test_an_expert_weight_that_does_not_pack_leaves_the_block_dense_and_correct():
+    """One down-projection value sits off the E2M1 grid (reference
+    tests/test_moe.py:561-573 has the whole weight off it): that weight cannot
+    be packed, so the dispatch must not claim its pack -- it is disabled at
+    the first call, the other product is still fused on its own (here: by the
+    stand-in), and the result is the dense block's."""
+    from metaljax_amd import kernels, moe
+    moe.reset_stats()
+    E, Tk, H, Ii, K = 4, 3, 64, 32, 2
+    text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    # the decode table's entry for code 5 (3.0) becomes 3.25: no E2M1 value
+    assert text.count("3.000000e+00") >= 2
+    head, sep, tail = text.rpartition("3.000000e+00")
+    bad = head + "3.250000e+00" + tail                      # in the down projection's table (the second one)
+    raw, _ = _moe_inputs(E, Tk, H, Ii)
+    args = [I.from_numpy(a) for a in raw]
+    ex = engine.compile_program(bad)
+    st = qmm.analyze(ex.interp)
+    assert len(st.moe) == 1
+    assert qmm.prologue(ex.interp, args) is True
+    assert st.moe[0].disabled and moe.stats()["fallbacks"] == 1 and qmm.stats()["fallbacks"] == 1
+    live = [m for m in st.matches if not m.disabled]
+    assert len(live) == 1 and not live[0].absorbed and set(st.roots) == {live[0].key}
+    want = I.host(I.Interpreter(bad).run(args)[0]).a
+    with pytest.MonkeyPatch.context() as mp:
+        calls = {"qmm": [], "take_k": 0}
+        mp.setattr(qmm, "DEVICE", "cpu")
+        mp.setattr(kernels, "quantized_matmul", _oracle_dense_product(calls))
+        (buf,) = engine.execute(ex, args)
+    assert len(calls["qmm"]) == 1 and moe.stats()["dispatches"] == 0
+    np.testing.assert_allclose(I.host(buf.data).a, want, rtol=3e-5, atol=3e-6 * max(1.0, np.abs(want).max()))
+
+
+def _oracle_dense_product(calls):
+    """A stand-in for kernels.quantized_matmul on host tensors (the oracle)."""
+    import torch
+    from oracle import qmm_oracle as O
+
+    def product(x, w, scales, biases, transpose=True, group_size=64, bits=4, mode="affine", out_dtype=None):
+        tables = np.asarray(scales) if mode == "mxfp4" else pack_tables_like(scales)
+        y = O.qmm(x.float().numpy(), np.asarray(w), tables, None if biases is None else pack_tables_like(biases),
+                  group_size, bits, mode)
+        calls["qmm"].append(tuple(x.shape))
+        return torch.from_numpy(y).to(out_dtype or x.dtype)
+    return product
+
+
+def pack_tables_like(a):
+    return (a.to_f32() if isinstance(a, packing.BF16Array) else np.asarray(a)).astype(np.float32)
+
+
 def test_router_check_catches_a_misplaced_weight(monkeypatch):
     """`verify` compares the evaluated scores with the scatter of the matched
     weights at the matched indices: a router record pointing at other weights
