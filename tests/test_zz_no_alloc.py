@@ -95,8 +95,9 @@ def test_static_entry_takes_no_device_memory():
     of the static entry point: torch's allocator cannot see a hipMalloc made
     inside the library, hipMemGetInfo can.  The outputs are allocated up front
     and one call is made before measuring, because the first call on a device
-    looks up the scratch array's address and sets kernel attributes (that call
-    belongs outside a stream capture; the later ones are capture-safe)."""
+    looks up the scratch array's address, sets kernel attributes and has the
+    kernels' code loaded (that call belongs outside a stream capture; the
+    later ones are capture-safe)."""
     lib = _lib.load()
     rng = np.random.default_rng(11)
     c = _case(rng, 6, 200, 512, 400, 800, "affine")      # prefill kernels: the largest scratch use here
@@ -111,14 +112,18 @@ def test_static_entry_takes_no_device_memory():
         _lib.check(rc)
     launch(ys[0])
     torch.cuda.synchronize()
-    free_before = torch.cuda.mem_get_info()[0]
-    for y in ys:
-        launch(y)
-    torch.cuda.synchronize()
-    free_after = torch.cuda.mem_get_info()[0]
+    free = [torch.cuda.mem_get_info()[0]]
+    for _ in range(3):                                    # three rounds of three calls
+        for y in ys:
+            launch(y)
+        torch.cuda.synchronize()
+        free.append(torch.cuda.mem_get_info()[0])
     need = int(lib.qmm_gather_workspace_bytes(c["p"], c["e"], c["n"], c["k"], _lib.BF16))
     assert need > (1 << 19)                               # the product does use scratch ...
-    assert free_before - free_after < (1 << 18), (free_before, free_after)      # ... and none of it was allocated
+    # ... and no call allocates it: over the nine calls less than half their worth went missing (the
+    # runtime may grow a pool of its own once), over the last three nothing at all
+    assert free[0] - free[-1] < 4 * need, free
+    assert free[-2] - free[-1] < (1 << 16), free
     assert torch.equal(ys[0], ys[1]) and torch.equal(ys[1], ys[2])
 
 
