@@ -412,20 +412,27 @@ def main():
         out["dense_bf16"] = {"C3 [2048,4096]x[4096,4096]": bench_dense_bf16(2048, 4096, 4096),
                              "C4 [256,8192]x[8192,8192]": bench_dense_bf16(256, 8192, 8192),
                              "C5 8 x [128,4096]x[14336,4096]": bench_dense_bf16(128, 14336, 4096, experts=8)}
-        # decode shapes outside the named configurations (random codes, timing only)
+        # Legs outside the named configurations (random codes, timing only).  An exception in one of
+        # them is reported in its place: it must not take the named configurations' line with it.
+        def extra(fn, *a, **kw):
+            try:
+                return fn(*a, **kw)
+            except Exception as why:                        # noqa: BLE001 -- reported, not hidden
+                return {"error": f"{type(why).__name__}: {why}"}
         out["other_decode_shapes"] = {
-            "int4 g64 [28672,4096] M=4": bench_decode_random(4, 28672, 4096),
-            "int4 g64 [4096,14336] M=4": bench_decode_random(4, 4096, 14336),
-            "int4 g64 f16 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f16"),
-            "int4 g64 f32 tables [14336,4096] M=4": bench_decode_random(4, 14336, 4096, tables="f32"),
-            "int8 g64 [14336,4096] M=4": bench_decode_random(4, 14336, 4096, bits=8),
-            "int4 g64 [37888,3584] M=4": bench_decode_random(4, 37888, 3584),
-            "mxfp4 [8192,8192] M=1": bench_decode_random(1, 8192, 8192, mode="mxfp4"),
-            "mxfp4 [5760,2880] M=1 (K no whole number of slices)": bench_decode_random(1, 5760, 2880, mode="mxfp4"),
-            "mxfp4 [5760,2880] M=16": bench_decode_random(16, 5760, 2880, mode="mxfp4"),
+            "int4 g64 [28672,4096] M=4": extra(bench_decode_random, 4, 28672, 4096),
+            "int4 g64 [4096,14336] M=4": extra(bench_decode_random, 4, 4096, 14336),
+            "int4 g64 f16 tables [14336,4096] M=4": extra(bench_decode_random, 4, 14336, 4096, tables="f16"),
+            "int4 g64 f32 tables [14336,4096] M=4": extra(bench_decode_random, 4, 14336, 4096, tables="f32"),
+            "int8 g64 [14336,4096] M=4": extra(bench_decode_random, 4, 14336, 4096, bits=8),
+            "int4 g64 [37888,3584] M=4": extra(bench_decode_random, 4, 37888, 3584),
+            "mxfp4 [8192,8192] M=1": extra(bench_decode_random, 1, 8192, 8192, mode="mxfp4"),
+            "mxfp4 [5760,2880] M=1 (K no whole number of slices)": extra(bench_decode_random, 1, 5760, 2880, mode="mxfp4"),
+            "mxfp4 [5760,2880] M=16": extra(bench_decode_random, 16, 5760, 2880, mode="mxfp4"),
         }
-        out["moe_decode"] = {f"8 experts int4 g64 [14336,4096], top-2, {t} token(s)": bench_moe_decode(t) for t in (1, 16)}
-        out["engine_execute_C2"] = bench_engine_execute(2, 16)
+        out["moe_decode"] = {f"8 experts int4 g64 [14336,4096], top-2, {t} token(s)": extra(bench_moe_decode, t)
+                             for t in (1, 16)}
+        out["engine_execute_C2"] = extra(bench_engine_execute, 2, 16)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
