@@ -184,3 +184,54 @@ def test_weight_as_the_left_operand_comes_back_transposed(_kernels_stood_in_for)
     assert ex.interp._qmm.matches[0].swapped
     (call,) = _kernels_stood_in_for["qmm"]
     assert call[0] == (t, k)
+
+
+from hypothesis import HealthCheck, given, settings, strategies as st  # noqa: E402
+
+
+@settings(max_examples=40, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+@given(k=st.sampled_from([64, 128, 192, 256, 384]), n=st.integers(4, 40).map(lambda v: 8 * v),
+       block=st.sampled_from([32, 64, 128, -1]), m=st.integers(1, 40), el=st.sampled_from(["bf16", "f32"]),
+       bits=st.sampled_from([4, 8]), seed=st.integers(0, 10_000))
+def test_dense_subchannel_over_drawn_shapes(k, n, block, m, el, bits, seed):
+    """The sub-channel chain over drawn sizes, group widths, code widths and
+    element types: recognized, packed once, and the fused result within the
+    literal chain's distance of the exact product."""
+    if block > 0 and k % block:
+        block = 32
+    qmm.reset_stats()
+    qmm._BUILT.clear()
+    qmm._SHARED.clear()
+    q, packed, scale, zero, g_idx, wref = T.quantize(k, n, block, seed=seed, bits=bits, bf16=el == "bf16")
+    x = np.random.default_rng(seed + 1).standard_normal((m, k)).astype(np.float32) * 0.5
+    if el == "bf16":
+        x = T.bf16_round(x)
+    ng = scale.shape[0]
+    text = T.dense_sub(k, n, ng, m, el=el) if bits == 4 else T.dense_i8_codes(k, n, ng, m, el=el)
+    args = [I.from_numpy(packed if bits == 4 else q), I.from_numpy(scale, el), I.from_numpy(zero),
+            I.from_numpy(g_idx), I.from_numpy(x, el)]
+    compare(text, args, x @ wref)
+    assert qmm.stats()["recognized"] == 1
+
+
+@settings(max_examples=30, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+@given(n=st.integers(1, 12).map(lambda v: 8 * v), k=st.integers(1, 12).map(lambda v: 32 * v), t=st.integers(1, 24),
+       experts=st.sampled_from([None, 2, 3]), rows_form=st.booleans(), seed=st.integers(0, 10_000))
+def test_mxfp4_chains_over_drawn_shapes(n, k, t, experts, rows_form, seed):
+    """MXFP4 weights of drawn sizes, dense and batched over experts, in both
+    spellings of the E2M1 decode (a gather of the value table in line, or jax's
+    private @_take callee): recognized, packed, the fused result the exact
+    product up to the activations' rounding."""
+    qmm.reset_stats()
+    qmm._BUILT.clear()
+    qmm._SHARED.clear()
+    lead = () if experts is None else (experts,)
+    codes, blocks, sb, w = T.random_mxfp4(lead + (n, k), seed=seed)
+    x = _x(seed + 1, lead + (t, k), 1.0)
+    if rows_form:
+        text = T.dense_mxfp4_rows(n, k, t, e=experts)
+    else:
+        text = T.dense_mxfp4(n, k, t) if experts is None else T.experts_mxfp4(experts, n, k, t)
+    exact = x @ w.T if experts is None else np.einsum("etk,enk->etn", x, w)
+    compare(text, [I.from_numpy(blocks), I.from_numpy(sb), I.from_numpy(x, "bf16")], exact)
+    assert qmm.stats()["mxfp4"] == 1 and qmm.stats()["batched"] == (0 if experts is None else 1)
