@@ -1269,6 +1269,51 @@ def test_gemma4_prefill_and_a_decode_step_inside_a_while_body_are_both_gathered(
         np.testing.assert_allclose(got, want, rtol=tol, atol=tol * max(1e-2, np.abs(want).max()))
 
 
+from hypothesis import HealthCheck, given, settings, strategies as st  # noqa: E402
+
+
+@settings(max_examples=20, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+@given(E=st.sampled_from([2, 4, 8]), kfrac=st.sampled_from([1, 2, 4]), Tk=st.integers(1, 6),
+       H=st.sampled_from([32, 64, 96]), Ii=st.sampled_from([32, 64]), gemma=st.booleans(), seed=st.integers(0, 1000))
+def test_expert_blocks_over_drawn_sizes(E, kfrac, Tk, H, Ii, gemma, seed):
+    """Both expert blocks over drawn expert counts, selection widths (down to
+    one expert a token, up to every expert), token counts and widths: always
+    one verified dispatch whose result is the dense block's."""
+    from metaljax_amd import moe
+    K = max(1, E // kfrac)
+    moe.reset_stats()
+    qmm.reset_stats()
+    qmm._BUILT.clear()
+    qmm._SHARED.clear()
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((Tk, H)) / 8).astype(np.float32)
+    if gemma:
+        packs3 = [T.make_mxfp4_experts(r, c, E, seed=seed + i) for i, (r, c) in enumerate(((Ii, H), (Ii, H), (H, Ii)))]
+        raw = (x, rng.standard_normal((H, E)).astype(np.float32), (1.0 + rng.standard_normal(H) / 8).astype(np.float32),
+               packs3[0][0], packs3[0][1], packs3[1][0], packs3[1][1], packs3[2][0], packs3[2][1],
+               (1.0 + rng.standard_normal(E) / 8).astype(np.float32))
+        text = T.moe_block_gemma4_mxfp4(E, Tk, H, Ii, K)
+    else:
+        gu_c, gu_s, _ = T.make_mxfp4_experts(2 * Ii, H, E, seed=seed)
+        d_c, d_s, _ = T.make_mxfp4_experts(H, Ii, E, seed=seed + 1)
+        raw = (x, (rng.standard_normal((H, E)) / 8).astype(np.float32), rng.standard_normal(E).astype(np.float32),
+               gu_c, gu_s, d_c, d_s, (rng.standard_normal((E, 2 * Ii)) / 8).astype(np.float32),
+               (rng.standard_normal((E, H)) / 8).astype(np.float32))
+        text = T.moe_block_mxfp4(E, Tk, H, Ii, K)
+    args = [I.from_numpy(a) for a in raw]
+    with pytest.MonkeyPatch.context() as mp:
+        mp.setattr(qmm, "DEVICE", "cpu")
+        mp.setattr(moe, "emit_dot", _oracle_expert_product([]))
+        (buf,) = engine.execute(engine.compile_program(text), args)
+        st_ = moe.stats()
+        assert st_["recognized"] == 1 and st_["verified"] == 1 and st_["dispatches"] == 1 and st_["fallbacks"] == 0, st_
+        got = I.host(buf.data).a
+        mp.setattr(qmm, "ENABLED", False)
+        (lit,) = engine.execute(engine.compile_program(text), args)
+    want = I.host(lit.data).a
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5 * max(1.0, np.abs(want).max()))
+
+
 def test_expert_dispatch_disabled_by_its_flag(monkeypatch):
     """METALJAX_MOE=0 (the reference's tests flip moe.ENABLED at run time,
     tests/test_moe.py:406-417): the block stays dense, its quantized dots are
