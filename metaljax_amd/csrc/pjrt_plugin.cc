@@ -846,6 +846,26 @@ PJRT_Error* LoadedLogicalIds(PJRT_LoadedExecutable_AddressableDeviceLogicalIds_A
   return nullptr;
 }
 
+// One replica of one computation on device 0, as an xla.DeviceAssignmentProto written out by hand
+// (reference metal_pjrt.cc:930-942 answers the same way): field 1 replica_count = 1, field 2
+// computation_count = 1, field 3 one ComputationDevice whose field 1, the packed replica_device_ids,
+// holds the single id 0.  The bytes are static, so there is nothing for the deleter to free.
+void keep_assignment(PJRT_DeviceAssignmentSerialized*) {}
+
+PJRT_Error* LoadedDeviceAssignment(PJRT_LoadedExecutable_GetDeviceAssignment_Args* a) {
+  static const char proto[] = {
+      (1 << 3) | 0, 1,            // replica_count: varint 1
+      (2 << 3) | 0, 1,            // computation_count: varint 1
+      (3 << 3) | 2, 3,            // computation_devices: a message of three bytes
+      (1 << 3) | 2, 1, 0,         //   replica_device_ids, packed: one varint, 0
+  };
+  a->serialized_bytes = proto;
+  a->serialized_bytes_size = sizeof(proto);
+  a->serialized_device_assignment = nullptr;
+  a->serialized_device_assignment_deleter = keep_assignment;
+  return nullptr;
+}
+
 PJRT_Error* LoadedDestroy(PJRT_LoadedExecutable_Destroy_Args* a) {
   if (a->executable) {
     release(a->executable->program);
@@ -1191,7 +1211,7 @@ void fill_api(PJRT_Api& api) {
   HAVE(PJRT_LoadedExecutable_IsDeleted, LoadedIsDeleted);
   HAVE(PJRT_LoadedExecutable_Execute, LoadedExecute);
   HAVE(PJRT_LoadedExecutable_Fingerprint, LoadedFingerprint);
-  LACK(PJRT_LoadedExecutable_GetDeviceAssignment);
+  HAVE(PJRT_LoadedExecutable_GetDeviceAssignment, LoadedDeviceAssignment);
   HAVE(PJRT_LoadedExecutable_AddressableDeviceLogicalIds, LoadedLogicalIds);
 
   HAVE(PJRT_Buffer_Destroy, BufferDestroy);

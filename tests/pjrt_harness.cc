@@ -691,6 +691,48 @@ int pjrt_harness_walk(int buffer, int exe) {
                  lids.num_addressable_device_logical_ids == 1 && lids.addressable_device_logical_ids[0].replica == 0 &&
                  lids.addressable_device_logical_ids[0].partition == 0);
   }
+  {   // the device assignment, decoded field by field: one replica of one computation, on device 0
+    ARGS(PJRT_LoadedExecutable_GetDeviceAssignment_Args, da);
+    da.executable = le;
+    STEP(53, taken(g_api->PJRT_LoadedExecutable_GetDeviceAssignment(&da)) == 0 && da.serialized_bytes &&
+                 da.serialized_device_assignment_deleter);
+    const unsigned char* p = reinterpret_cast<const unsigned char*>(da.serialized_bytes);
+    const unsigned char* end = p + da.serialized_bytes_size;
+    long replicas = -1, computations = -1, devices = 0, first_id = -1;
+    auto varint = [&](const unsigned char*& q, const unsigned char* lim) {
+      unsigned long v = 0;
+      for (int shift = 0; q < lim; shift += 7) {
+        const unsigned char c = *q++;
+        v |= (unsigned long)(c & 0x7F) << shift;
+        if (!(c & 0x80)) break;
+      }
+      return (long)v;
+    };
+    bool well_formed = true;
+    while (p < end && well_formed) {
+      const long key = varint(p, end);
+      if (key == ((1 << 3) | 0)) replicas = varint(p, end);
+      else if (key == ((2 << 3) | 0)) computations = varint(p, end);
+      else if (key == ((3 << 3) | 2)) {
+        const long len = varint(p, end);
+        const unsigned char* sub_end = p + len;
+        well_formed = sub_end <= end;
+        while (well_formed && p < sub_end) {
+          const long sub = varint(p, sub_end);
+          if (sub != ((1 << 3) | 2)) { well_formed = false; break; }
+          const long n = varint(p, sub_end);
+          const unsigned char* ids_end = p + n;
+          well_formed = ids_end <= sub_end;
+          while (well_formed && p < ids_end) {
+            const long id = varint(p, ids_end);
+            if (devices++ == 0) first_id = id;
+          }
+        }
+      } else well_formed = false;
+    }
+    STEP(54, well_formed && replicas == 1 && computations == 1 && devices == 1 && first_id == 0);
+    da.serialized_device_assignment_deleter(da.serialized_device_assignment);
+  }
   ARGS(PJRT_Executable_Destroy_Args, xd);
   xd.executable = ge.executable;
   STEP(46, taken(g_api->PJRT_Executable_Destroy(&xd)) == 0);
