@@ -16,6 +16,12 @@ from metaljax_amd import engine, interpreter as I, kernels, packing, qmm
 from oracle import qmm_oracle as O
 
 
+# Packs are uploaded when a GPU is visible; the stand-ins below read them as host arrays.
+pytestmark = pytest.mark.skipif(torch.cuda.is_available(),
+                                reason="stands in for the kernels on a machine without a GPU; with one, "
+                                       "test_gpu_recognizer.py runs the same programs on the kernels")
+
+
 def _f32(a):
     if a is None:
         return None
