@@ -27,7 +27,9 @@ def _stream(t: torch.Tensor) -> int:
 
 # One scratch allocation per (device, stream), grown to the largest request seen:
 # calls on one stream are ordered, so the next call may overwrite what the
-# previous one used; nothing is allocated per call once it has grown.
+# previous one used; nothing is allocated per call once it has grown.  (A call
+# recorded into a graph keeps the address it saw: record the Bound* forms below,
+# which own their workspace for as long as they live, not these calls.)
 _SCRATCH = {}
 
 
